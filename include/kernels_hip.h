@@ -1,0 +1,161 @@
+/* include/kernels_hip.h - C entry points of the MI355X (gfx950) SeedLM decode-in-matmul backend.
+ *
+ * This is the drop-in boundary: every kc_ and kq4_ function below keeps the name, argument order, argument meaning and error
+ * behaviour of the reference's launcher of the same name (engine/kernels_cuda.h, engine/kernels_qwen4.h), so the
+ * reference's C99 engine (engine/mova_cuda.c encode_layer :1218-1327, engine/qwen4_cuda.c moe :1023-1083) and its
+ * kernel tests (tests/kernel_backend_cuda.c) can call this library in place of engine/kernels_moe.cu.
+ * Differences a host must know:
+ *   - the first argument is a kc_stream_t: an opaque pointer that carries a hipStream_t (0 = the default stream), where
+ *     the reference takes a cudaStream_t;
+ *   - the stream table argument G is accepted and ignored (the kernels hold the 512-entry GF(2) basis themselves);
+ *   - launchers are asynchronous, allocate nothing and keep no per-call state, so whole forwards can be captured into
+ *     graphs as the reference does (engine/mova_cuda.c:1402-1406).
+ * The structs are layout-identical to the reference's (engine/kernels_cuda.h:19-48, engine/kernels_moe.metal:96-130).
+ * Plain C99: no HIP header is needed to include this file.
+ */
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* kc_stream_t; /* holds a hipStream_t; replaces cudaStream_t in every signature */
+
+/* weight formats = the reference's MF_ and NS_ codes (engine/kernels_moe.metal:17, nslm/model_st.h:31) */
+enum { MF_BF16 = 0, MF_SEED4 = 1, MF_Q8 = 2, MF_Q4 = 3, MF_SEED4P4 = 4 };
+#define MV_MAXT 8 /* dense matvec: tokens per call (engine/kernels_moe.metal:20) */
+
+/* One slice's device stream addresses (engine/kernels_cuda.h:19-24).  Stream order (engine/kernels_cuda.h:4-7):
+ * BF16 0 values; Q8/Q4 0 packed words, 1 scales, 2 biases; SEED4 0 seeds, 1 nibble words; SEED4P4 0 seeds,
+ * 1 coefficient words, 3 exponent codes (block g of the slice in nibble g&1 of byte g>>1). */
+typedef struct {
+    const void* p[4];
+    int32_t eb;     /* seeds: the slice's exponent bias */
+    int32_t gs;     /* Q8 / Q4: log2 of the affine group (5: 32, 6: 64); 0 is 64 */
+    int32_t pad[2];
+} WSlice;
+
+typedef struct { /* engine/kernels_moe.metal:104-108 */
+    int d, n, top_k;
+    int hw;      /* router partition width (d / 2) */
+    float scale; /* router_scaling_factor */
+} RouterArgs;
+
+typedef struct { int slice, start, count, pad; } MmTile; /* engine/kernels_moe.metal:130 */
+
+/* the expert slot table (engine/kernels_cuda.h:32-48) */
+typedef struct {
+    int32_t* unit_slot;  /* [units]: slot, or -1 */
+    int32_t* slot_unit;  /* [slots]: unit, or -1 */
+    uint32_t* slot_last; /* [slots]: the admit tick of the last use */
+    uint32_t* tick;      /* [4]: the admit tick (from CACHE_TICK_BASE), unused */
+    uint32_t* stats;     /* [2]: hits, misses */
+    int32_t* jobs;       /* [2 * per_layer]: (unit, slot) pairs queued by the last admit */
+    int32_t* njobs;      /* [1] */
+    uint8_t* vram;       /* the pool */
+    const uint8_t* host; /* device address of the arena that holds every unit */
+    uint64_t unit_bytes;
+    int32_t slots, per_layer, ntens;
+    WSlice* tab;         /* [sparse layer][ntens][per_layer] */
+    uint32_t off[3][4];  /* byte offset of tensor i's stream s in a unit (0xFFFFFFFF: no stream) */
+    uint64_t hits, misses;
+} CachePool;
+#define CACHE_TICK_BASE 0x40000000u
+enum { CACHE_PROTECT_PREV = 2 };
+#define CACHE_MAX_PER_LAYER 1024
+
+/* ---- seed / affine / BF16 matvec family ------------------------------------------------------------------------- */
+/* engine/kernels_cuda.h:78-79, engine/kernels_moe.cu:2308-2316.  Dense matvec, T <= MV_MAXT tokens:
+ * y[t][r] = bf16(W[r] . x[t]), or with add: bf16(y + bf16(W[r] . x[t])).  Token t's rows do not depend on T. */
+void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int xs, float* y, int ys, int T, int add,
+           const uint32_t* G);
+/* engine/kernels_cuda.h:81-82, engine/kernels_moe.cu:2317-2323.  Gather matvec over P (token, expert) pairs: pair p
+ * uses slice sel[p] and input row p / xdiv. */
+void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
+               const int32_t* sel, int P, int xdiv, const uint32_t* G);
+/* engine/kernels_cuda.h:84-85, engine/kernels_moe.cu:2324-2328.  Routed experts' gate + up + SwiGLU in one pass:
+ * a[p][r] = bf16(silu_bf(bf16(g . x)) * bf16(u . x)). */
+void kc_mv_gu(kc_stream_t s, int fmt, const WSlice* wg, const WSlice* wu, int K, int R, const float* x, int xs, float* a,
+              int ys, const int32_t* sel, int P, int xdiv, const uint32_t* G);
+
+/* ---- prefill GEMM ------------------------------------------------------------------------------------------------- */
+/* engine/kernels_cuda.h:95, engine/kernels_moe.cu:2354-2355: seed weights exact in f32 (three BF16 terms) instead of
+ * rounded to BF16.  Process-global, as in the reference. */
+void kc_seed_gemm_f32(int on);
+/* engine/kernels_cuda.h:96-97, engine/kernels_moe.cu:2360-2364 */
+void kc_mm(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int xs, float* y, int ys, int T, int add,
+           const uint32_t* G);
+/* engine/kernels_cuda.h:98-99, engine/kernels_moe.cu:2365-2372 */
+void kc_mm_grouped(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
+                   int xdiv, const int32_t* perm, const MmTile* tiles, int ntiles, const uint32_t* G);
+/* engine/kernels_cuda.h:103-108, engine/kernels_moe.cu:2373-2383, 2396-2399 */
+#define BUCKET_MAX_EXPERTS 1024
+void kc_bucket(kc_stream_t s, const int32_t* inds, int count, int n, int32_t* perm, MmTile* tiles, int32_t* ntiles);
+void kc_mm_grouped_dev(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
+                       int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int max_tiles,
+                       const uint32_t* G);
+/* engine/kernels_cuda.h:110-114, engine/kernels_moe.cu:2384-2395 */
+void kc_pack_input_bf16(kc_stream_t s, const float* x, uint16_t* y, size_t n);
+void kc_mm_packed(kc_stream_t s, int fmt, WSlice w, int K, int R, const uint16_t* x, int xs, float* y, int ys, int T,
+                  int add, const uint32_t* G);
+void kc_mm_grouped_packed(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
+                          int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
+                          const uint32_t* G);
+/* pairs per tile of the grouped GEMM: MmTile.count <= MMT_BN (engine/kernels_cuda.h:116) */
+#define MMT_BN 128
+
+/* ---- routers, elementwise ------------------------------------------------------------------------------------------ */
+/* engine/kernels_cuda.h:120-123, engine/kernels_moe.cu:2400-2407: sigmoid scores, selection scores, top-k, weights */
+void kc_router(kc_stream_t s, RouterArgs a, const uint16_t* W, const uint16_t* bias, const float* x, float* score,
+               float* sel, int32_t* inds, float* wts, int T);
+void kc_router_topk(kc_stream_t s, RouterArgs a, const float* score, const float* sel, int32_t* inds, float* wts, int T);
+/* engine/kernels_qwen4.h:53-54, engine/kernels_qwen4.cu:417-422: softmax top-k (ties to the higher index), n_exp <= 1024,
+ * top_k <= 32.  Qwen4Cfg is the reference's configuration struct (nslm/qwen4_cfg.h:9-26), layout-identical here; the
+ * kernels read only n_exp and top_k. */
+#define QWEN4_MAX_LAYERS 128
+typedef struct {
+    int n_layer, d, vocab, eos;
+    int hc, hc_rank;
+    int n_head, n_kv, head_dim, rot_dim;
+    float rope_theta, eps;
+    int ix_heads, ix_dim, ix_budget, ix_ratio;
+    int lin_hk, lin_hv, lin_dk, lin_dv, lin_conv;
+    int n_exp, top_k, ff_exp, ff_shared;
+    int ple_dim, ple_conv, ngram, heads_per_ngram, ngram_parts;
+    int64_t ngram_base, ngram_div, seed;
+    uint8_t attn[QWEN4_MAX_LAYERS];
+    int8_t ple[QWEN4_MAX_LAYERS];
+} Qwen4Cfg;
+void kq4_route(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int32_t* ind, float* wt, int T);
+void kq4_route_ld(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int ld, int32_t* ind, float* wt, int T);
+/* engine/kernels_cuda.h:124-125, engine/kernels_moe.cu:2408-2413 */
+void kc_swiglu(kc_stream_t s, const float* g, const float* u, float* a, int n);
+void kc_moe_combine(kc_stream_t s, const float* D, const float* w, const float* shared, float* x, int d, int k, int T);
+/* engine/kernels_qwen4.h:71, engine/kernels_qwen4.cu:514-516 */
+void kq4_moe_combine(kc_stream_t s, int d, int k, const float* D, const float* wt, const float* sh, const float* sg,
+                     int sgld, float* out, int T);
+
+/* ---- expert slot table (engine/kernels_cuda.h:53-55, engine/kernels_moe.cu:2710-2722) ------------------------------ */
+void kc_cache_admit(kc_stream_t s, const CachePool* p, int sl, const int32_t* inds, int count, int flags);
+void kc_cache_copy(kc_stream_t s, const CachePool* p, int blocks);
+
+/* ---- weights to BF16 in memory (engine/kernels_cuda.h:161, engine/kernels_moe.cu:2441-2444) ------------------------
+ * A per-head map [H][O][I] in fmt decoded to BF16 bits: SEED4P4 with W.p = seeds, coefficients, exponent biases [H]
+ * (int32, device), exponent codes; Q8 / Q4 as bf16(scale * code + bias). */
+void kc_heads_deq(kc_stream_t s, int fmt, WSlice W, const uint32_t* G, int H, int O, int I, uint16_t* out);
+
+/* ---- additions of this backend (no counterpart in the reference) --------------------------------------------------- */
+/* Rows [0,R) of one slice of any format decoded to BF16 bits [R][K] (seeds with the slice's own eb; SEED4 too):
+ * the bit-exact weight regeneration check. */
+void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out);
+/* 1: the matvec family stores unrounded f32 instead of BF16-rounded values (for comparison with CPU references that do
+ * not round, nslm/lib_cpu_seed4.c).  Process-global like kc_seed_gemm_f32; default 0 = the reference's store. */
+void kc_store_f32(int on);
+/* last launch-configuration error of this library on the calling thread's device: 0 none, else a hipError_t value */
+int kc_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,152 @@
+// nslm_dev.h - device-side building blocks shared by the gfx950 kernels: BF16 rounding, the LFSR stream basis, and the
+// exact integer decode of one 8-weight SeedLM block on 16-bit integer dot products.
+//
+// Arithmetic contract (reference: nslm/lfsr.h:4-10, nslm/search4.h:4-6): state_k of seed s is bits k..k+15 of the bit
+// stream s | g(s) << 16, where g(s) is GF(2)-linear in s; weight c of a block is
+//   isum_c = sum_p (state_(P*c+p+1) - 32768) * q_p   (exact, |isum| < 2^20),   w_c = (float) isum_c * fl(R32 * 2^e).
+// Everything up to isum_c is done in integers here, so regenerated weights are bit-exact by construction.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernels_hip.h"
+
+namespace nslm {
+
+// ---- BF16 (round to nearest even; reference engine/kernels_moe.cu:17-31) ---------------------------------------------
+__device__ __forceinline__ float bfr(float x) {
+    uint32_t u = __float_as_uint(x);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return __uint_as_float(u & 0xFFFF0000u);
+}
+__device__ __forceinline__ uint32_t tobf(float x) {
+    uint32_t u = __float_as_uint(x);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ float bf(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t pack_bf2(float a, float b) { return tobf(a) | (tobf(b) << 16); }
+// nn.silu on a BF16 tensor: the sigmoid and the product are each rounded to BF16
+__device__ __forceinline__ float silu_bf(float g) {
+    const float s = bfr(1.0f / (1.0f + expf(-g)));
+    return bfr(g * s);
+}
+// y = bf16(acc), or the residual form bf16(y + bf16(acc)); f32out keeps the unrounded sum (a switch of this backend)
+__device__ __forceinline__ void store_y(float* yo, float s, int add, int f32out) {
+    if (f32out) *yo = add ? *yo + s : s;
+    else *yo = add ? bfr(*yo + bfr(s)) : bfr(s);
+}
+
+// ---- the stream basis -------------------------------------------------------------------------------------------------
+// g(s) = the 32 stream bits that follow seed s: bit k = top bit of state k+1.  g is linear over GF(2), so
+// g(s) = lo[s & 0xFF] ^ hi[s >> 8] with two 256-entry tables, built here at compile time from the LFSR definition
+// (taps 0, 1, 3, 12; shift right; feedback into bit 15).  The P = 3 format reads the low 24 bits of the same table.
+struct StreamBasis {
+    uint32_t v[512];
+};
+constexpr uint32_t stream32_of(uint32_t s) {
+    uint32_t g = 0;
+    for (int k = 0; k < 32; ++k) {
+        const uint32_t fb = (s ^ (s >> 1) ^ (s >> 3) ^ (s >> 12)) & 1u;
+        s = (s >> 1) | (fb << 15);
+        g |= (s >> 15) << k;
+    }
+    return g;
+}
+constexpr StreamBasis make_basis() {
+    StreamBasis b{};
+    for (uint32_t i = 0; i < 256; ++i) {
+        b.v[i] = stream32_of(i);
+        b.v[256 + i] = stream32_of(i << 8);
+    }
+    return b;
+}
+// Pairs of sign-extended int4 coefficients as packed int16: entry b = { sext4(b & 15), sext4(b >> 4) }.
+struct CoefPairs {
+    uint32_t v[256];
+};
+constexpr CoefPairs make_pairs() {
+    CoefPairs t{};
+    for (uint32_t b = 0; b < 256; ++b) {
+        const int lo = (int) (b & 15u) - (int) ((b & 8u) << 1), hi = (int) (b >> 4) - (int) (((b >> 4) & 8u) << 1);
+        t.v[b] = ((uint32_t) lo & 0xFFFFu) | ((uint32_t) hi << 16);
+    }
+    return t;
+}
+__device__ const StreamBasis kBasis = make_basis();
+__device__ const CoefPairs kPairs = make_pairs();
+
+// LDS copy of both tables: [0,512) stream basis, [512,768) coefficient pairs
+#define NSLM_TAB_WORDS 768
+__device__ __forceinline__ void load_tables(uint32_t* tab) {
+    for (int i = threadIdx.x; i < 512; i += blockDim.x) tab[i] = kBasis.v[i];
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) tab[512 + i] = kPairs.v[i];
+}
+__device__ __forceinline__ uint32_t stream_of(const uint32_t* tab, uint32_t seed16) {
+    return tab[seed16 & 0xFFu] ^ tab[256 + (seed16 >> 8)];
+}
+
+// ---- exact block decode -----------------------------------------------------------------------------------------------
+typedef short short2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int dot2(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot2(__builtin_bit_cast(short2v, a), __builtin_bit_cast(short2v, b), c, false);
+}
+// { word X's half hx, word Y's half hy } as one packed pair
+__device__ __forceinline__ uint32_t halves(uint32_t X, int hx, uint32_t Y, int hy) {
+    const uint32_t sel = (uint32_t) (2 * hx) | ((uint32_t) (2 * hx + 1) << 8) | ((uint32_t) (4 + 2 * hy) << 16) |
+                         ((uint32_t) (5 + 2 * hy) << 24);
+    return __builtin_amdgcn_perm(Y, X, sel);
+}
+
+// The 16 windows of a block's stream.  `up` is any word whose upper 16 bits are the seed, g the 32 bits that follow.
+// A[k], k = 1..16: low half = state_k - 32768, high half = state_(k+16) - 32768 as int16 (state ^ 0x8000).
+__device__ __forceinline__ void windows(uint32_t up, uint32_t g, uint32_t (&A)[17]) {
+#pragma unroll
+    for (int k = 1; k <= 15; ++k) A[k] = __builtin_amdgcn_alignbit(g, up, 16 + k) ^ 0x80008000u;
+    A[16] = g ^ 0x80008000u;
+}
+
+// P = 4: weight c reads states 4c+1..4c+4; q01 = {q0,q1}, q23 = {q2,q3} as packed int16 (reference nslm/lib_search4.c:22-31)
+__device__ __forceinline__ void isum_p4(uint32_t up, uint32_t g, uint32_t q01, uint32_t q23, int (&is)[8]) {
+    uint32_t A[17];
+    windows(up, g, A);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int k = 4 * c + 1;
+        is[c] = dot2(halves(A[k], 0, A[k + 1], 0), q01, dot2(halves(A[k + 2], 0, A[k + 3], 0), q23, 0));
+        is[c + 4] = dot2(halves(A[k], 1, A[k + 1], 1), q01, dot2(halves(A[k + 2], 1, A[k + 3], 1), q23, 0));
+    }
+}
+// P = 3: weight c reads states 3c+1..3c+3; q01 = {q0,q1}, q2 = {q2,0} (reference nslm/lfsr.h:116-128)
+__device__ __forceinline__ void isum_p3(uint32_t up, uint32_t g, uint32_t q01, uint32_t q2, int (&is)[8]) {
+    uint32_t A[17];
+    windows(up, g, A);
+    const uint32_t q2hi = q2 << 16;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int k0 = 3 * c + 1, k1 = k0 + 1, k2 = k0 + 2;   // state k lives in A[k] low (k <= 16) or A[k-16] high
+        const uint32_t pr = halves(A[k0 <= 16 ? k0 : k0 - 16], k0 > 16, A[k1 <= 16 ? k1 : k1 - 16], k1 > 16);
+        const int third = k2 <= 16 ? dot2(A[k2], q2, 0) : dot2(A[k2 - 16], q2hi, 0);
+        is[c] = dot2(pr, q01, third);
+    }
+}
+
+// One block of either seed format from its raw fields.  seed16 / word16: the 16-bit seed and coefficient (P = 4) or
+// nibble (P = 3) word, zero-extended.  Returns the integer sums and the block's exponent e = eb + code.
+template <int P>
+__device__ __forceinline__ void block_isum(const uint32_t* tab, uint32_t seed16, uint32_t word16, int (&is)[8]) {
+    const uint32_t g = stream_of(tab, seed16), up = seed16 << 16;
+    if (P == 4) isum_p4(up, g, tab[512 + (word16 & 0xFFu)], tab[512 + (word16 >> 8)], is);
+    else isum_p3(up, g, tab[512 + ((word16 >> 4) & 0xFFu)], tab[512 + (word16 >> 12)], is);
+}
+// 2^e as f32 bits; e in the normal range
+__device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t) (e + 127) << 23); }
+#define NSLM_R32 (1.0f / 32767.0f)
+
+__device__ __forceinline__ int group_shift(const WSlice& w) { return w.gs ? w.gs : 6; }
+
+// process-wide switches and launch-error bookkeeping (defined in nslm_mv.hip)
+int host_store_f32();
+void host_note_launch();
+
+}   // namespace nslm

@@ -1,0 +1,59 @@
+// nslm_rt.hip - the thin C-ABI layer over the HIP runtime (include/nslm_rt.h): what the reference's C99 host code calls
+// the CUDA runtime for (engine/mova_cuda.c:183-222, 590, 892-896; tests/kernel_backend_cuda.c:17-41), one-to-one.
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "nslm_rt.h"
+
+extern "C" {
+
+int nh_device_count(int* n) { return (int) hipGetDeviceCount(n); }
+int nh_set_device(int dev) { return (int) hipSetDevice(dev); }
+int nh_malloc(void** p, size_t n) { return (int) hipMalloc(p, n ? n : 16); }
+int nh_free(void* p) { return (int) hipFree(p); }
+int nh_host_alloc(void** p, size_t n) { return (int) hipHostMalloc(p, n ? n : 16, hipHostMallocMapped); }
+int nh_host_free(void* p) { return (int) hipHostFree(p); }
+int nh_memcpy_h2d(void* dst, const void* src, size_t n) { return n ? (int) hipMemcpy(dst, src, n, hipMemcpyHostToDevice) : 0; }
+int nh_memcpy_d2h(void* dst, const void* src, size_t n) { return n ? (int) hipMemcpy(dst, src, n, hipMemcpyDeviceToHost) : 0; }
+int nh_memcpy_d2d(void* dst, const void* src, size_t n) { return n ? (int) hipMemcpy(dst, src, n, hipMemcpyDeviceToDevice) : 0; }
+int nh_memcpy_h2d_async(void* dst, const void* src, size_t n, nh_stream_t s) {
+    return n ? (int) hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, (hipStream_t) s) : 0;
+}
+int nh_memcpy_d2h_async(void* dst, const void* src, size_t n, nh_stream_t s) {
+    return n ? (int) hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, (hipStream_t) s) : 0;
+}
+int nh_memset(void* p, int v, size_t n) { return n ? (int) hipMemset(p, v, n) : 0; }
+int nh_stream_create(nh_stream_t* s) { return (int) hipStreamCreateWithFlags((hipStream_t*) s, hipStreamNonBlocking); }
+int nh_stream_destroy(nh_stream_t s) { return (int) hipStreamDestroy((hipStream_t) s); }
+int nh_stream_sync(nh_stream_t s) { return (int) hipStreamSynchronize((hipStream_t) s); }
+int nh_device_sync(void) { return (int) hipDeviceSynchronize(); }
+int nh_event_create(nh_event_t* e) { return (int) hipEventCreate((hipEvent_t*) e); }
+int nh_event_destroy(nh_event_t e) { return (int) hipEventDestroy((hipEvent_t) e); }
+int nh_event_record(nh_event_t e, nh_stream_t s) { return (int) hipEventRecord((hipEvent_t) e, (hipStream_t) s); }
+int nh_event_sync(nh_event_t e) { return (int) hipEventSynchronize((hipEvent_t) e); }
+int nh_event_elapsed_ms(float* ms, nh_event_t a, nh_event_t b) { return (int) hipEventElapsedTime(ms, (hipEvent_t) a, (hipEvent_t) b); }
+int nh_stream_wait_event(nh_stream_t s, nh_event_t e) { return (int) hipStreamWaitEvent((hipStream_t) s, (hipEvent_t) e, 0); }
+int nh_last_error(void) { return (int) hipGetLastError(); }
+const char* nh_error_string(int err) { return hipGetErrorString((hipError_t) err); }
+int nh_device_info(int dev, char* name, int namelen, int* cus, uint64_t* mem_bytes, int* clock_khz) {
+    hipDeviceProp_t p;
+    const hipError_t e = hipGetDeviceProperties(&p, dev);
+    if (e != hipSuccess) return (int) e;
+    if (name && namelen > 0) {
+        strncpy(name, p.name, (size_t) namelen - 1);
+        name[namelen - 1] = 0;
+    }
+    if (cus) *cus = p.multiProcessorCount;
+    if (mem_bytes) *mem_bytes = (uint64_t) p.totalGlobalMem;
+    if (clock_khz) *clock_khz = p.clockRate;
+    return 0;
+}
+int nh_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {
+    size_t f = 0, t = 0;
+    const hipError_t e = hipMemGetInfo(&f, &t);
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return (int) e;
+}
+
+}   // extern "C"

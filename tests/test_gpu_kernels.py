@@ -1,0 +1,382 @@
+"""Parity of the gfx950 kernels against the CPU oracle, through the C ABI (kt_* -> kc_* / kq4_*), on the GPU.
+
+Bars (as the reference's tests/test_mova_kernels.c): regenerated weights bit-exact; matvec / GEMM outputs within one BF16
+ulp of the double-precision reference rounded at the kernel's rounding points, plus the f32 accumulation bound
+64 * 1.2e-7 * sum |w x| (:27-30, :171); unrounded f32 stores within max-rel-err 2e-3 of the double reference (the bar the
+benchmark definition states for fp32 accumulation; measured errors are ~1e-6); index outputs (routers, grouping, slot
+table) exact."""
+import os
+
+import numpy as np
+import pytest
+
+from nanoseedlm_amd import packs
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+F32B = 64 * 1.2e-7
+
+
+@pytest.fixture(scope="module")
+def be():
+    from nanoseedlm_amd import backend
+    backend.require_gpu()
+    return backend
+
+
+def slice_of(orc, p, s=0):
+    f = p["fmt"]
+    if f == packs.MF_SEED4P4:
+        return orc.make_slice(f, p["seeds"][s], p["coefs"][s], None, p["codes"][s], eb=p["eb"][s])
+    if f == packs.MF_SEED4:
+        return orc.make_slice(f, p["seeds"][s], p["nibs"][s], eb=p["eb"][s])
+    if f in (packs.MF_Q4, packs.MF_Q8):
+        return orc.make_slice(f, p["words"][s], p["scales"][s], p["biases"][s], gs={32: 5, 64: 6}[p["group"]])
+    return orc.make_slice(f, p["w"][s])
+
+
+def make_pack(rng, fmt, S, R, K, group=64):
+    if fmt == packs.MF_SEED4P4:
+        return packs.seed4p4(rng, S, R, K, eb=[-19, -17, -21, -20][:S] if S <= 4 else -20, code_max=5)
+    if fmt == packs.MF_SEED4:
+        return packs.seed4(rng, S, R, K, eb=[-18, -16, -20, -19][:S] if S <= 4 else -19)
+    if fmt == packs.MF_Q4:
+        return packs.affine(rng, S, R, K, 4, group)
+    if fmt == packs.MF_Q8:
+        return packs.affine(rng, S, R, K, 8, group)
+    return packs.bf16(rng, S, R, K, std=0.03)
+
+
+def close_bf(got, ref, extra):
+    """|got - ref| within one BF16 ulp of ref plus extra (tests/test_mova_kernels.c:27-30)."""
+    return np.abs(got.astype(np.float64) - ref) <= np.abs(ref) / 128.0 + 1e-30 + extra
+
+
+def ref_mv(orc, p, s, x, fmt_mv=True):
+    """double reference y[T,R] and mag for slice s: seeds exact, Q4 in the matvec's unrounded form, others BF16 values"""
+    return orc.mv_double(p["fmt"], slice_of(orc, p, s), p["R"], p["K"], x, qmv=1 if fmt_mv else 0)
+
+
+ALL_FMT = [packs.MF_BF16, packs.MF_SEED4, packs.MF_Q8, packs.MF_Q4, packs.MF_SEED4P4]
+NAMES = {0: "bf16", 1: "seed4", 2: "q8", 3: "q4", 4: "seed4p4"}
+
+
+# ---- bit-exact weight regeneration -----------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4, packs.MF_Q4, packs.MF_Q8])
+def test_slice_deq_bit_exact(be, oracle, fmt):
+    rng = np.random.default_rng(100 + fmt)
+    p = make_pack(rng, fmt, 2, 48, 320)
+    for s in range(2):
+        got = be.kt_slice_deq(p, s)
+        want = oracle.slice_bf16(fmt, slice_of(oracle, p, s), 48, 320)
+        assert np.array_equal(got, want), NAMES[fmt]
+
+
+def test_deq_every_seed_and_coefficient(be, oracle):
+    """All 65,535 seeds (one block each) and all 65,536 coefficient words, every exponent code: exact against the oracle."""
+    n = 65536
+    rng = np.random.default_rng(7)
+    seeds = np.arange(n, dtype=np.uint16)
+    seeds[0] = 1
+    for fmt in (packs.MF_SEED4P4, packs.MF_SEED4):
+        words = rng.permutation(n).astype(np.uint16)
+        codes = rng.integers(0, 16, size=(1, n), dtype=np.uint8)
+        if fmt == packs.MF_SEED4P4:
+            p = {"fmt": fmt, "S": 1, "R": n // 8, "K": 64, "seeds": seeds.reshape(1, n // 8, 8), "coefs": words.reshape(1, n // 8, 8),
+                 "codes": packs._pack_nibbles(codes), "eb": np.array([-22], dtype=np.int32)}
+        else:
+            p = {"fmt": fmt, "S": 1, "R": n // 8, "K": 64, "seeds": seeds.reshape(1, n // 8, 8), "nibs": words.reshape(1, n // 8, 8),
+                 "eb": np.array([-22], dtype=np.int32)}
+        got = be.kt_slice_deq(p, 0)
+        want = oracle.slice_bf16(fmt, slice_of(oracle, p, 0), n // 8, 64)
+        assert np.array_equal(got, want)
+
+
+def test_deq_golden_fixtures(be):
+    g = np.load(os.path.join(GOLD, "matvec_p4.npz"))
+    rows, kb = int(g["rows"]), int(g["kb"])
+    p = {"fmt": packs.MF_SEED4P4, "S": 1, "R": rows, "K": kb * 8, "seeds": g["seeds"][None], "coefs": g["coefs"][None],
+         "codes": g["codes"][None], "eb": np.array([int(g["bias"])], dtype=np.int32)}
+    assert np.array_equal(be.kt_slice_deq(p, 0), packs.f32_to_bf16_bits(g["rows_ref"]))
+    h = np.load(os.path.join(GOLD, "rows_p3_q4.npz"))
+    p3 = {"fmt": packs.MF_SEED4, "S": 1, "R": int(h["rows"]), "K": int(h["K"]), "seeds": h["p3_seeds"][None], "nibs": h["p3_nibs"][None],
+          "eb": np.array([int(h["p3_eb"])], dtype=np.int32)}
+    assert np.array_equal(be.kt_slice_deq(p3, 0), packs.f32_to_bf16_bits(h["p3_rows"]))
+    q4 = {"fmt": packs.MF_Q4, "S": 1, "R": int(h["rows"]), "K": int(h["K"]), "group": 64, "words": h["q4_words"][None],
+          "scales": h["q4_scales"][None], "biases": h["q4_biases"][None]}
+    assert np.array_equal(be.kt_slice_deq(q4, 0), h["q4_rows_bf16"])
+    # unrounded f32 matvec against the compiled reference's cpu_seed4 result held in the fixture (it does not round)
+    be.kt().kt_store_f32(1)
+    try:
+        y = be.kt_mv(p, g["x"])
+    finally:
+        be.kt().kt_store_f32(0)
+    assert np.max(np.abs(y[0] - g["y_ref"])) / np.max(np.abs(g["y_ref"])) < 2e-6
+
+
+def test_heads_deq(be, oracle):
+    rng = np.random.default_rng(21)
+    H, O, I = 3, 10, 64
+    p = packs.seed4p4(rng, 1, H * O, I, eb=0)
+    ebias = np.array([-20, -18, -23], dtype=np.int32)
+    got = be.kt_heads_deq_p4(p["seeds"], p["coefs"], ebias, p["codes"], H, O, I)
+    codes_all = packs.unpack_nibbles(p["codes"][0], H * O * I // 8)
+    for h in range(H):
+        ph = {"fmt": packs.MF_SEED4P4, "S": 1, "R": O, "K": I, "seeds": p["seeds"][:, h * O:(h + 1) * O], "coefs": p["coefs"][:, h * O:(h + 1) * O],
+              "codes": packs._pack_nibbles(codes_all[None, h * O * I // 8:(h + 1) * O * I // 8]), "eb": ebias[h:h + 1]}
+        assert np.array_equal(got[h], oracle.slice_bf16(packs.MF_SEED4P4, slice_of(oracle, ph, 0), O, I))
+
+
+# ---- matvec family ------------------------------------------------------------------------------------------------------------
+
+# K: 256 / 512 the reference's cases (tests/test_mova_kernels.c:161); 768 and 2880 rows whose chunk count is not a power
+# of two (LDS row sums); 2048 / 4096 the benchmark shapes; 136 not a multiple of 64 (generic path)
+@pytest.mark.parametrize("K", [256, 512, 768, 2880, 2048, 4096, 136])
+@pytest.mark.parametrize("fmt", ALL_FMT)
+def test_mv_dense_gather_gateup(be, oracle, fmt, K):
+    if fmt in (packs.MF_Q4, packs.MF_Q8) and K % 64:
+        pytest.skip("affine groups of 64 need K % 64 == 0")
+    rng = np.random.default_rng(K * 8 + fmt)
+    R, S = 24, 3
+    p = make_pack(rng, fmt, S, R, K)
+    x = packs.round_bf16(rng.uniform(-1, 1, (8, K)).astype(np.float32))
+    xg = packs.round_bf16(rng.uniform(-1, 1, (16, K)).astype(np.float32))
+    ref, mag = ref_mv(oracle, p, 0, x)
+    y1 = None
+    for T in range(1, 9):
+        add = T == 3
+        y0 = packs.round_bf16(rng.uniform(-1, 1, (T, R)).astype(np.float32))
+        y = be.kt_mv(p, x[:T], add=int(add), y0=y0)
+        if T == 1:
+            y1 = y.copy()
+        elif not add:   # token 0 with T = k equals T = 1 bit for bit (:173-183)
+            assert np.array_equal(y[0].view(np.uint32), y1[0].view(np.uint32)), f"{NAMES[fmt]} K={K} T={T}: token 0 differs from T=1"
+        want = packs.round_bf16(ref[:T].astype(np.float32)).astype(np.float64)
+        if add:
+            want = packs.round_bf16((y0 + want).astype(np.float32)).astype(np.float64)
+        ok = close_bf(y, want, F32B * mag[:T] * (2 if add else 1))
+        assert ok.all(), f"{NAMES[fmt]} K={K} dense T={T}: {np.count_nonzero(~ok)} mismatches"
+    # gather: 6 pairs, slices sel[p], inputs p / xdiv (:201-217)
+    sel = np.array([2, 0, 1, 2, 1, 0], dtype=np.int32)
+    y = be.kt_mv_sel(p, sel, xg[:3], 2)
+    for pi, s in enumerate(sel):
+        r, m = ref_mv(oracle, p, int(s), xg[pi // 2])
+        assert close_bf(y[pi], packs.round_bf16(r[0].astype(np.float32)).astype(np.float64), F32B * m[0]).all(), (NAMES[fmt], K, pi)
+    # gate + up + SwiGLU: gate slice sel[p], up slice sel[p] + 1; within one BF16 flip of g or u (:218-241)
+    sel = np.array([1, 0, 1, 1, 0, 0], dtype=np.int32)
+    a = be.kt_mv_gu(p, sel, xg[:3], 2)
+    for pi, s in enumerate(sel):
+        g, _ = ref_mv(oracle, p, int(s), xg[pi // 2])
+        u, _ = ref_mv(oracle, p, int(s) + 1, xg[pi // 2])
+        gg = packs.round_bf16(g[0].astype(np.float32)).astype(np.float64)
+        uu = packs.round_bf16(u[0].astype(np.float32)).astype(np.float64)
+        sg = packs.round_bf16((1 / (1 + np.exp(-gg))).astype(np.float32)).astype(np.float64)
+        want = packs.round_bf16((packs.round_bf16((gg * sg).astype(np.float32)).astype(np.float64) * uu).astype(np.float32)).astype(np.float64)
+        slack = (np.abs(uu) * (np.abs(gg) + 1) + np.abs(gg) * np.abs(uu)) / 128 + 1e-7
+        assert close_bf(a[pi], want, slack).all(), (NAMES[fmt], K, pi)
+
+
+@pytest.mark.parametrize("fmt,K,R", [(packs.MF_SEED4P4, 4096, 512), (packs.MF_SEED4P4, 2048, 768), (packs.MF_SEED4P4, 768, 2048),
+                                     (packs.MF_SEED4, 2880, 300), (packs.MF_SEED4P4, 8192, 64)])
+def test_mv_f32_store_max_rel_err(be, oracle, fmt, K, R):
+    """Unrounded f32 stores: max |y - ref| / max |ref| < 2e-3 (fp32 accumulate); rows span several workgroups."""
+    rng = np.random.default_rng(K + R)
+    p = make_pack(rng, fmt, 1, R, K)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    be.kt().kt_store_f32(1)
+    try:
+        y = be.kt_mv(p, x)
+        ys = be.kt_mv_sel(p, np.zeros(2, dtype=np.int32), x, 2)
+    finally:
+        be.kt().kt_store_f32(0)
+    ref, _ = ref_mv(oracle, p, 0, x)
+    err = np.max(np.abs(y - ref)) / np.max(np.abs(ref))
+    assert err < 2e-3 and err < 1e-5, err
+    assert np.array_equal(ys[0], ys[1]) and np.max(np.abs(ys[0] - ref[0])) / np.max(np.abs(ref)) < 1e-5
+    if fmt == packs.MF_SEED4P4:   # and against the CPU decode-in-dot-product restatement (no rounding there either)
+        yc = oracle.cpu_seed4_matvec(p["seeds"][0], p["coefs"][0], p["codes"][0], int(p["eb"][0]), x[0], R, K // 8, threads=4)
+        assert np.max(np.abs(y[0] - yc)) / np.max(np.abs(yc)) < 2e-6
+
+
+def test_mv_empty_and_ragged(be, oracle):
+    rng = np.random.default_rng(5)
+    p = make_pack(rng, packs.MF_SEED4P4, 1, 1, 64)            # one row of one chunk
+    x = packs.round_bf16(rng.uniform(-1, 1, (1, 64)).astype(np.float32))
+    ref, mag = ref_mv(oracle, p, 0, x)
+    assert close_bf(be.kt_mv(p, x), packs.round_bf16(ref.astype(np.float32)).astype(np.float64), F32B * mag).all()
+    p = make_pack(rng, packs.MF_SEED4P4, 1, 37, 192)          # rows not a multiple of the rows per iteration
+    x = packs.round_bf16(rng.uniform(-1, 1, (5, 192)).astype(np.float32))
+    ref, mag = ref_mv(oracle, p, 0, x)
+    assert close_bf(be.kt_mv(p, x), packs.round_bf16(ref.astype(np.float32)).astype(np.float64), F32B * mag).all()
+
+
+# ---- GEMM -----------------------------------------------------------------------------------------------------------------------
+
+def ref_mm(orc, p, s, x, exact):
+    fmt = p["fmt"]
+    seed = fmt in (packs.MF_SEED4, packs.MF_SEED4P4)
+    w = orc.rows_f32(fmt, slice_of(orc, p, s), p["R"], p["K"], 0 if seed else 1)
+    if seed and not exact:
+        w = packs.round_bf16(w)
+    xd = x.astype(np.float64)
+    return xd @ w.astype(np.float64).T, np.abs(xd) @ np.abs(w.astype(np.float64)).T
+
+
+@pytest.mark.parametrize("fmt", ALL_FMT)
+@pytest.mark.parametrize("exact", [1, 0])
+def test_mm_dense_and_grouped(be, oracle, fmt, exact):
+    """R 40: not a multiple of a tile; K 128: four K steps; T 45, 50 pairs over 3 slices (tests/test_mova_kernels.c:247-317)"""
+    seed = fmt in (packs.MF_SEED4, packs.MF_SEED4P4)
+    if not seed and not exact:
+        pytest.skip("only seed weights have a BF16-rounded mode")
+    rng = np.random.default_rng(300 + fmt)
+    S, R, K, T, P, xdiv = 3, 40, 128, 45, 50, 2
+    p = make_pack(rng, fmt, S, R, K)
+    x = packs.round_bf16(rng.uniform(-1, 1, (T, K)).astype(np.float32))
+    be.kt().kt_seed_gemm_exact(exact)
+    try:
+        y0 = packs.round_bf16(rng.uniform(-1, 1, (T, R)).astype(np.float32))
+        y = be.kt_mm(p, x, y0)
+        ref, mag = ref_mm(oracle, p, 0, x, exact)
+        want = packs.round_bf16((y0 + packs.round_bf16(ref.astype(np.float32))).astype(np.float32)).astype(np.float64)
+        assert close_bf(y, want, 2 * F32B * mag).all(), NAMES[fmt]
+        slc = (np.arange(P) * 7) % S
+        perm, tiles = oracle.bucket(slc.astype(np.int32), S, be.kt().kt_mm_tile())
+        yg = be.kt_mm_grouped(p, perm, tiles, x[:P // xdiv], xdiv)
+        for pi in range(P):
+            r, m = ref_mm(oracle, p, int(slc[pi]), x[pi // xdiv][None], exact)
+            assert close_bf(yg[pi], packs.round_bf16(r[0].astype(np.float32)).astype(np.float64), F32B * m[0]).all(), (NAMES[fmt], pi)
+        yb, perm2, tiles2 = be.kt_mm_bucketed(p, slc.astype(np.int32), x[:P // xdiv], xdiv, packed=0)
+        assert np.array_equal(perm2, perm) and np.array_equal(tiles2, tiles)
+        assert np.array_equal(yb.view(np.uint32), yg.view(np.uint32))
+        ybp, _, _ = be.kt_mm_bucketed(p, slc.astype(np.int32), x[:P // xdiv], xdiv, packed=1)
+        assert np.array_equal(ybp.view(np.uint32), yg.view(np.uint32))   # BF16-valued inputs: packing changes nothing
+    finally:
+        be.kt().kt_seed_gemm_exact(0)
+
+
+@pytest.mark.parametrize("T", [130, 300, 512, 600])
+def test_mm_token_tiles(be, oracle, T):
+    """every token-tile width of the dense GEMM (128, 256, 512 per workgroup, and more than one workgroup of tokens)"""
+    rng = np.random.default_rng(T)
+    R, K = 96, 256
+    p = make_pack(rng, packs.MF_SEED4P4, 1, R, K)
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    xb = packs.round_bf16(x)
+    y = be.kt_mm_plain(p, x, packed=0)
+    yp = be.kt_mm_plain(p, x, packed=1)
+    assert np.array_equal(y.view(np.uint32), yp.view(np.uint32))
+    ref, mag = ref_mm(oracle, p, 0, xb, 0)
+    assert close_bf(y, packs.round_bf16(ref.astype(np.float32)).astype(np.float64), F32B * mag).all()
+    be.kt().kt_store_f32(1)
+    try:
+        yf = be.kt_mm_plain(p, x, packed=0)
+    finally:
+        be.kt().kt_store_f32(0)
+    assert np.max(np.abs(yf - ref)) / np.max(np.abs(ref)) < 1e-2   # the bar for the BF16 MFMA prefill
+
+
+# ---- grouping, routers, elementwise, slot table -------------------------------------------------------------------------------
+
+def test_bucket(be, oracle):
+    rng = np.random.default_rng(13)
+    for n, count in ((512, 1000), (128, 256), (64, 64), (1024, 3000), (8, 5)):
+        inds = rng.integers(0, n, count).astype(np.int32)
+        inds[::2] = 0   # half the pairs on expert 0 (tests/test_qwen4_engine.c:33-61)
+        perm, tiles = be.kt_bucket(inds, n)
+        operm, otiles = oracle.bucket(inds, n, 128)
+        assert np.array_equal(perm, operm) and np.array_equal(tiles, otiles)
+
+
+def test_routers(be, oracle):
+    rng = np.random.default_rng(10)
+    n, k, T, d = 128, 8, 5, 256
+    score = rng.uniform(0, 1, (T, n)).astype(np.float32)
+    sel = score + rng.standard_normal((T, n)).astype(np.float32) * 0.1
+    sel[1] = np.round(sel[1] * 4) / 4
+    sel[2, :] = 0.5
+    ind, wt = be.kt_router_topk(score, sel, k, 2.5)
+    oi, ow = oracle.topk_sigmoid(score, sel, k, 2.5)
+    assert np.array_equal(ind, oi) and np.allclose(wt, ow, rtol=1e-6)
+    W = packs.f32_to_bf16_bits((rng.standard_normal((n, d)) * 0.05).astype(np.float32))
+    bias = packs.f32_to_bf16_bits((rng.standard_normal(n) * 0.01).astype(np.float32))
+    x = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
+    ind, wt = be.kt_router(W, bias, x, k, d // 2, 1.0)
+    sc, se, oi, ow = oracle.route_sigmoid(W, bias, x, k, d // 2, 1.0)
+    # a BF16 flip of a partial sum may swap near-tied experts: bound the flips as the reference's engine test does
+    same = np.mean([len(set(ind[t]) & set(oi[t])) / k for t in range(T)])
+    assert same >= 0.95
+    for t in range(T):
+        if np.array_equal(ind[t], oi[t]):
+            assert np.allclose(wt[t], ow[t], rtol=2e-2)
+    # softmax top-k with an engineered tie (tests/test_qwen4_kernels.c:233-245) and many exact ties
+    E = 512
+    lg = rng.standard_normal((6, E)).astype(np.float32)
+    lg[0, 7] = lg[0, 300] = 9.0
+    lg[1] = np.round(lg[1] * 2) / 2
+    ind, wt = be.kt_q4_route(lg, 10)
+    oi, ow = oracle.route_softmax(lg, 10)
+    assert ind[0, 0] == 300 and ind[0, 1] == 7
+    assert np.array_equal(ind, oi) and np.allclose(wt, ow, rtol=1e-5)
+    lg = rng.standard_normal((3, 128)).astype(np.float32)
+    ind, wt = be.kt_q4_route(lg, 8)
+    oi, ow = oracle.route_softmax(lg, 8)
+    assert np.array_equal(ind, oi) and np.allclose(wt, ow, rtol=1e-5)
+
+
+def test_swiglu_and_combines(be, oracle):
+    rng = np.random.default_rng(12)
+    r = packs.round_bf16
+    g = r(rng.standard_normal(5000).astype(np.float32) * 3)
+    u = r(rng.standard_normal(5000).astype(np.float32))
+    a = be.kt_swiglu(g, u)
+    want = oracle.swiglu(g, u)
+    # expf on the GPU and in libm may differ in the last bit: at most a BF16 flip of the sigmoid on a few elements
+    assert np.mean(a != want) < 0.01 and np.allclose(a, want, rtol=1.6e-2, atol=1e-30)
+    T, k, d = 3, 8, 300
+    D = r(rng.standard_normal((T * k, d)).astype(np.float32))
+    w = rng.uniform(0, 1, (T, k)).astype(np.float32)
+    sh = r(rng.standard_normal((T, d)).astype(np.float32))
+    x = r(rng.standard_normal((T, d)).astype(np.float32))
+    assert np.array_equal(be.kt_combine(D, w, sh, x).view(np.uint32), oracle.moe_combine(D, w, sh, x).view(np.uint32))
+    sg = rng.standard_normal((T, 1)).astype(np.float32)
+    assert np.allclose(be.kt_q4_combine(D, w, sh, sg), oracle.q4_moe_combine(D, w, sh, sg), rtol=1e-5, atol=1e-6)
+
+
+def test_cache_admit_matches_host_model(be, oracle):
+    rng = np.random.default_rng(3)
+    per_layer, layers, slots = 64, 3, 100
+    dev = dict(unit_slot=np.full(per_layer * layers, -1, dtype=np.int32), slot_unit=np.full(slots, -1, dtype=np.int32),
+               slot_last=np.zeros(slots, dtype=np.uint32), tick=np.array([0x40000000, 0, 0, 0], dtype=np.uint32),
+               stats=np.zeros(2, dtype=np.uint32))
+    host = {k: v.copy() for k, v in dev.items()}
+    hh = hm = 0
+    for step in range(12):
+        sl = step % layers
+        inds = rng.integers(0, per_layer, 24).astype(np.int32)
+        flags = 2 if step % 4 == 3 else 0
+        jobs = be.kt_cache_admit(dev["unit_slot"], dev["slot_unit"], dev["slot_last"], dev["tick"], dev["stats"], per_layer, sl, inds, flags)
+        oj, h, m = oracle.cache_admit(host["unit_slot"], host["slot_unit"], host["slot_last"], host["tick"], per_layer, sl, inds, 1 if flags else 0)
+        hh += h
+        hm += m
+        assert np.array_equal(jobs, oj), step
+        for k in ("unit_slot", "slot_unit", "slot_last"):
+            assert np.array_equal(dev[k], host[k]), (step, k)
+        assert dev["tick"][0] == host["tick"][0] and tuple(dev["stats"]) == (hh, hm)
+    # all resident (slots == units): no job is ever queued
+    us = np.arange(per_layer, dtype=np.int32)
+    jobs = be.kt_cache_admit(us.copy(), us.copy(), np.zeros(per_layer, dtype=np.uint32), np.array([0x40000000, 0, 0, 0], dtype=np.uint32),
+                             np.zeros(2, dtype=np.uint32), per_layer, 0, np.array([1, 5, 9], dtype=np.int32))
+    assert jobs.size == 0
+
+
+def test_cache_copy_moves_units(be):
+    rng = np.random.default_rng(4)
+    units, slots, unit_bytes = 16, 6, 4096
+    arena = rng.integers(0, 256, (units, unit_bytes), dtype=np.uint8)
+    inds = np.array([3, 7, 11, 7], dtype=np.int32)
+    pool, unit_slot = be.kt_cache_roundtrip(arena, slots, units, inds)
+    for u in (3, 7, 11):
+        assert unit_slot[u] >= 0 and np.array_equal(pool[unit_slot[u]], arena[u])
+    assert np.count_nonzero(unit_slot >= 0) == 3
