@@ -292,17 +292,18 @@ void or_cpu_seed3_matvec(const uint16_t* seeds, const uint16_t* nibs, int bias, 
 }
 
 /* ------------------------------------------------------------------------------------------------------------------ */
-/* GEMV in double.  qmv != 0: Q4/Q8 weights unrounded s*q+b (MLX's qmv form, tests/test_mova_kernels.c:150-152).     */
+/* GEMV in double.  qmv != 0: Q4 weights unrounded s*q+b (MLX's qmv form); BF16 and Q8 as their BF16 values, seeds exact
+ * (tests/test_mova_kernels.c:146-158).                                                                               */
 
 void or_mv_double(int fmt, const OrSlice* w, int R, int K, const float* x, int xs, int T, int qmv, double* y,
                   double* mag) {
     float* row = (float*) malloc(sizeof(float) * (size_t) K);
     const int seed = fmt == OR_SEED4 || fmt == OR_SEED4P4;
     for (int r = 0; r < R; ++r) {
-        or_row_f32(fmt, w, R, K, r, !(qmv || seed), row);
+        or_row_f32(fmt, w, R, K, r, !seed, row);
         for (int t = 0; t < T; ++t) {
             double acc = 0, m = 0;
-            if (!seed && qmv && (fmt == OR_Q4 || fmt == OR_Q8)) {
+            if (qmv && fmt == OR_Q4) {
                 /* exact products of the unrounded affine value: recompute s*q+b in double */
                 const uint32_t* q = (const uint32_t*) w->p[0];
                 const uint16_t* S = (const uint16_t*) w->p[1];
@@ -310,7 +311,7 @@ void or_mv_double(int fmt, const OrSlice* w, int R, int K, const float* x, int x
                 const int sh = group_shift(w);
                 for (int c = 0; c < K; ++c) {
                     const size_t i = (size_t) r * K + c;
-                    const uint32_t code = fmt == OR_Q8 ? (q[i >> 2] >> (8 * (i & 3))) & 255u : (q[i >> 3] >> (4 * (i & 7))) & 15u;
+                    const uint32_t code = (q[i >> 3] >> (4 * (i & 7))) & 15u;
                     const double wv = (double) or_bf2f(S[i >> sh]) * (double) code + (double) or_bf2f(B[i >> sh]);
                     const double v = wv * (double) x[(size_t) t * xs + c];
                     acc += v;
