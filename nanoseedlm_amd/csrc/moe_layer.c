@@ -1,0 +1,233 @@
+/* moe_layer.c - see moe_layer.h.  Plain C99 over the kc_ / kq4_ / nh_ entry points. */
+#include "moe_layer.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "nslm_rt.h"
+
+struct NslmMoe {
+    NslmMoeCfg c;
+    int units, resident, final;
+    uint64_t unit_bytes, stream_len[3][4];
+    CachePool pool;             /* device pointers inside */
+    uint8_t* arena;             /* device: every unit */
+    uint8_t* unit_host;         /* staging for one unit */
+    int32_t* eb;                /* host: [units][3] exponent biases */
+    uint16_t *rw, *rb;          /* device: router weights [layer][n_exp][d], biases [layer][n_exp] */
+    float *logit, *score, *wt, *A, *G, *U, *D, *zero;
+    int32_t *ind, *perm, *ntiles;
+    MmTile* tiles;
+    int max_tiles;
+};
+
+static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
+
+NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
+    if (c->n_exp > CACHE_MAX_PER_LAYER || c->top_k > 32 || c->n_exp < c->top_k || (c->fmt != MF_SEED4P4 && c->fmt != MF_SEED4) ||
+        c->d % 8 || c->ff % 8 || c->max_rows < 1) {
+        snprintf(err, (size_t) errlen, "moe: unsupported configuration");
+        return NULL;
+    }
+    NslmMoe* m = (NslmMoe*) calloc(1, sizeof *m);
+    m->c = *c;
+    m->units = c->n_layer * c->n_exp;
+    /* unit layout: tensor i's stream s at a 256-byte aligned offset (engine/mova_cuda.c:318-327) */
+    uint64_t cur = 0;
+    for (int i = 0; i < 3; ++i)
+        for (int s = 0; s < 4; ++s) {
+            const uint64_t nblk = (uint64_t) c->d * c->ff / 8;
+            uint64_t len = 0;
+            if (s == 0 || s == 1) len = nblk * 2;
+            else if (s == 3 && c->fmt == MF_SEED4P4) len = (nblk + 1) / 2;
+            m->stream_len[i][s] = len;
+            m->pool.off[i][s] = 0xFFFFFFFFu;
+            if (!len) continue;
+            m->pool.off[i][s] = (uint32_t) cur;
+            cur += pad256(len);
+        }
+    m->unit_bytes = m->pool.unit_bytes = cur;
+    m->pool.per_layer = c->n_exp;
+    m->pool.ntens = 3;
+    m->pool.slots = (c->slots <= 0 || c->slots >= m->units) ? m->units : c->slots;
+    m->resident = m->pool.slots == m->units;
+    if (!m->resident && m->pool.slots < 2 * c->top_k * c->max_rows && m->pool.slots < c->n_exp) {
+        snprintf(err, (size_t) errlen, "moe: a pool of %d slots cannot hold one step's experts", m->pool.slots);
+        free(m);
+        return NULL;
+    }
+    const int P = c->max_rows * c->top_k;
+    m->max_tiles = P / MMT_BN + c->n_exp + 1;
+    int bad = 0;
+    bad |= nh_malloc((void**) &m->arena, cur * (uint64_t) m->units);
+    if (m->resident) m->pool.vram = m->arena;
+    else bad |= nh_malloc((void**) &m->pool.vram, cur * (uint64_t) m->pool.slots);
+    m->pool.host = m->arena;
+    bad |= nh_malloc((void**) &m->pool.unit_slot, 4 * (size_t) m->units);
+    bad |= nh_malloc((void**) &m->pool.slot_unit, 4 * (size_t) m->pool.slots);
+    bad |= nh_malloc((void**) &m->pool.slot_last, 4 * (size_t) m->pool.slots);
+    bad |= nh_malloc((void**) &m->pool.tick, 16);
+    bad |= nh_malloc((void**) &m->pool.stats, 16);
+    bad |= nh_malloc((void**) &m->pool.jobs, 8 * (size_t) c->n_exp);
+    bad |= nh_malloc((void**) &m->pool.njobs, 16);
+    bad |= nh_malloc((void**) &m->pool.tab, sizeof(WSlice) * (size_t) m->units * 3);
+    bad |= nh_malloc((void**) &m->rw, 2 * (size_t) c->n_layer * c->n_exp * c->d);
+    bad |= nh_malloc((void**) &m->rb, 2 * (size_t) c->n_layer * c->n_exp);
+    bad |= nh_malloc((void**) &m->logit, 4 * (size_t) c->max_rows * c->n_exp);
+    bad |= nh_malloc((void**) &m->score, 4 * (size_t) c->max_rows * c->n_exp);
+    bad |= nh_malloc((void**) &m->wt, 4 * (size_t) P);
+    bad |= nh_malloc((void**) &m->ind, 4 * (size_t) P);
+    bad |= nh_malloc((void**) &m->A, 4 * (size_t) P * c->ff);
+    bad |= nh_malloc((void**) &m->G, 4 * (size_t) P * c->ff);
+    bad |= nh_malloc((void**) &m->U, 4 * (size_t) P * c->ff);
+    bad |= nh_malloc((void**) &m->D, 4 * (size_t) P * c->d);
+    bad |= nh_malloc((void**) &m->zero, 4 * (size_t) c->max_rows * c->d);
+    bad |= nh_malloc((void**) &m->perm, 4 * (size_t) P);
+    bad |= nh_malloc((void**) &m->tiles, sizeof(MmTile) * (size_t) m->max_tiles);
+    bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 3));
+    m->unit_host = (uint8_t*) calloc(1, cur);
+    m->eb = (int32_t*) calloc((size_t) m->units * 3, 4);
+    if (bad || !m->unit_host || !m->eb) {
+        snprintf(err, (size_t) errlen, "moe: out of memory (%.2f GB of experts)", (double) cur * m->units / 1e9);
+        nslm_moe_close(m);
+        return NULL;
+    }
+    nh_memset(m->zero, 0, 4 * (size_t) c->max_rows * c->d);
+    nh_memset(m->rb, 0, 2 * (size_t) c->n_layer * c->n_exp);
+    return m;
+}
+
+void nslm_moe_close(NslmMoe* m) {
+    if (!m) return;
+    void* d[] = {m->arena, m->resident ? NULL : m->pool.vram, m->pool.unit_slot, m->pool.slot_unit, m->pool.slot_last, m->pool.tick,
+                 m->pool.stats, m->pool.jobs, m->pool.njobs, m->pool.tab, m->rw, m->rb, m->logit, m->score, m->wt, m->ind, m->A,
+                 m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles};
+    for (size_t i = 0; i < sizeof d / sizeof d[0]; ++i)
+        if (d[i]) nh_free(d[i]);
+    free(m->unit_host);
+    free(m->eb);
+    free(m);
+}
+
+int nslm_moe_set_expert(NslmMoe* m, int layer, int expert, int tensor, const uint16_t* seeds, const uint16_t* words,
+                        const uint8_t* codes, int eb) {
+    if (layer < 0 || layer >= m->c.n_layer || expert < 0 || expert >= m->c.n_exp || tensor < 0 || tensor > 2) return -1;
+    const int u = layer * m->c.n_exp + expert;
+    uint8_t* base = m->arena + (uint64_t) u * m->unit_bytes;
+    int e = nh_memcpy_h2d(base + m->pool.off[tensor][0], seeds, m->stream_len[tensor][0]);
+    e |= nh_memcpy_h2d(base + m->pool.off[tensor][1], words, m->stream_len[tensor][1]);
+    if (m->c.fmt == MF_SEED4P4) e |= nh_memcpy_h2d(base + m->pool.off[tensor][3], codes, m->stream_len[tensor][3]);
+    m->eb[u * 3 + tensor] = eb;
+    return e ? -1 : 0;
+}
+
+int nslm_moe_set_router(NslmMoe* m, int layer, const uint16_t* W, const uint16_t* bias) {
+    if (layer < 0 || layer >= m->c.n_layer) return -1;
+    int e = nh_memcpy_h2d(m->rw + (size_t) layer * m->c.n_exp * m->c.d, W, 2 * (size_t) m->c.n_exp * m->c.d);
+    if (bias) e |= nh_memcpy_h2d(m->rb + (size_t) layer * m->c.n_exp, bias, 2 * (size_t) m->c.n_exp);
+    return e ? -1 : 0;
+}
+
+/* initial residency round-robin over the layers, expert-major, and the slice tables (engine/mova_cuda.c:372-392) */
+int nslm_moe_finalize(NslmMoe* m) {
+    const int units = m->units, slots = m->pool.slots, E = m->c.n_exp, nl = m->c.n_layer;
+    int32_t* us = (int32_t*) malloc(4 * (size_t) units);
+    int32_t* su = (int32_t*) malloc(4 * (size_t) slots);
+    WSlice* tab = (WSlice*) calloc((size_t) units * 3, sizeof(WSlice));
+    const uint32_t tick0[4] = {CACHE_TICK_BASE, 0, 0, 0};
+    int bad = 0, s = 0;
+    for (int u = 0; u < units; ++u) us[u] = -1;
+    for (int i = 0; i < slots; ++i) su[i] = -1;
+    if (m->resident) {
+        for (int u = 0; u < units; ++u) us[u] = su[u] = u;   /* the arena is the pool */
+    } else {
+        for (int x = 0; x < E && s < slots; ++x)
+            for (int sl = 0; sl < nl && s < slots; ++sl, ++s) {
+                const int u = sl * E + x;
+                us[u] = s;
+                su[s] = u;
+                bad |= nh_memcpy_d2d(m->pool.vram + (uint64_t) s * m->unit_bytes, m->arena + (uint64_t) u * m->unit_bytes, m->unit_bytes);
+            }
+    }
+    for (int sl = 0; sl < nl; ++sl)
+        for (int i = 0; i < 3; ++i)
+            for (int x = 0; x < E; ++x) {
+                WSlice* t = &tab[((size_t) sl * 3 + i) * E + x];
+                const int u = sl * E + x;
+                t->eb = m->eb[u * 3 + i];
+                if (us[u] < 0) continue;
+                for (int st = 0; st < 4; ++st)
+                    if (m->pool.off[i][st] != 0xFFFFFFFFu) t->p[st] = m->pool.vram + (uint64_t) us[u] * m->unit_bytes + m->pool.off[i][st];
+            }
+    bad |= nh_memcpy_h2d(m->pool.unit_slot, us, 4 * (size_t) units);
+    bad |= nh_memcpy_h2d(m->pool.slot_unit, su, 4 * (size_t) slots);
+    bad |= nh_memset(m->pool.slot_last, 0, 4 * (size_t) slots);
+    bad |= nh_memcpy_h2d(m->pool.tick, tick0, 16);
+    bad |= nh_memset(m->pool.njobs, 0, 16);
+    bad |= nh_memset(m->pool.stats, 0, 16);
+    bad |= nh_memcpy_h2d(m->pool.tab, tab, sizeof(WSlice) * (size_t) units * 3);
+    free(us); free(su); free(tab);
+    m->final = !bad;
+    return bad ? -1 : 0;
+}
+
+int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, float* io) {
+    const NslmMoeCfg* c = &m->c;
+    if (!m->final || T < 1 || T > c->max_rows || layer < 0 || layer >= c->n_layer) return -1;
+    const int E = c->n_exp, k = c->top_k, d = c->d, ff = c->ff, P = T * k;
+    const WSlice* gate = m->pool.tab + ((size_t) layer * 3 + 0) * E;
+    const WSlice* up = m->pool.tab + ((size_t) layer * 3 + 1) * E;
+    const WSlice* down = m->pool.tab + ((size_t) layer * 3 + 2) * E;
+    if (c->router == NSLM_ROUTE_SOFTMAX) {
+        WSlice rw;
+        memset(&rw, 0, sizeof rw);
+        rw.p[0] = m->rw + (size_t) layer * E * d;
+        Qwen4Cfg qc;
+        memset(&qc, 0, sizeof qc);
+        qc.n_exp = E;
+        qc.top_k = k;
+        if (T <= MV_MAXT) kc_mv(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+        else kc_mm(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+        kq4_route(s, &qc, m->logit, m->ind, m->wt, T);
+    } else {
+        RouterArgs ra = {d, E, k, d / 2, c->route_scale};
+        kc_router(s, ra, m->rw + (size_t) layer * E * d, m->rb + (size_t) layer * E, xn, m->logit, m->score, m->ind, m->wt, T);
+    }
+    if (!m->resident) {   /* with every expert resident the table never changes: nothing to admit, nothing to copy */
+        kc_cache_admit(s, &m->pool, layer, m->ind, P, 0);
+        kc_cache_copy(s, &m->pool, 64);
+    }
+    if (T <= MV_MAXT) {   /* decode: one gather pass per (token, expert) pair (engine/mova_cuda.c:1301-1307) */
+        kc_mv_gu(s, c->fmt, gate, up, d, ff, xn, d, m->A, ff, m->ind, P, k, NULL);
+        kc_mv_sel(s, c->fmt, down, ff, d, m->A, ff, m->D, d, m->ind, P, 1, NULL);
+    } else {              /* batched: pairs grouped by expert, three grouped GEMMs (engine/mova_cuda.c:1308-1317) */
+        kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
+        kc_mm_grouped_dev(s, c->fmt, gate, d, ff, xn, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+        kc_mm_grouped_dev(s, c->fmt, up, d, ff, xn, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+        kc_swiglu(s, m->G, m->U, m->A, P * ff);
+        kc_mm_grouped_dev(s, c->fmt, down, ff, d, m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+    }
+    if (c->router == NSLM_ROUTE_SOFTMAX) kq4_moe_combine(s, d, k, m->D, m->wt, m->zero, m->zero, 0, io, T);
+    else kc_moe_combine(s, m->D, m->wt, m->zero, io, d, k, T);
+    return kc_last_error() ? -1 : 0;
+}
+
+int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {
+    if (nh_device_sync()) return -1;
+    return (nh_memcpy_d2h(ind, m->ind, 4 * (size_t) T * m->c.top_k) | nh_memcpy_d2h(wt, m->wt, 4 * (size_t) T * m->c.top_k)) ? -1 : 0;
+}
+int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses) {
+    uint32_t st[2] = {0, 0};
+    if (nh_device_sync() || nh_memcpy_d2h(st, m->pool.stats, 8)) return -1;
+    *hits = st[0];
+    *misses = st[1];
+    return 0;
+}
+uint64_t nslm_moe_unit_bytes(const NslmMoe* m) { return m->unit_bytes; }
+uint64_t nslm_moe_expert_bytes(const NslmMoe* m) {
+    uint64_t n = 0;
+    for (int i = 0; i < 3; ++i)
+        for (int s = 0; s < 4; ++s) n += m->stream_len[i][s];
+    return n;
+}

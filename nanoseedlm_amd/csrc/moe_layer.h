@@ -1,0 +1,61 @@
+/* moe_layer.h - host side of one routed-expert MoE layer stack on the gfx950 kernels, in C99: the expert slot table
+ * (layout and initial residency as the reference's build_pool, engine/mova_cuda.c:311-404) and the per-layer launch
+ * sequence of the reference's engines (engine/mova_cuda.c:1279-1325 encode_layer; engine/qwen4_cuda.c:1023-1083 moe).
+ * All experts of all layers live in one HBM arena; with slots == units (the default on a 288 GB GPU) the arena is the
+ * pool, every expert is resident, and the admit / copy kernels are skipped.  A smaller pool exercises the LRU table.
+ */
+#pragma once
+#include <stdint.h>
+
+#include "kernels_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { NSLM_ROUTE_SOFTMAX = 0, NSLM_ROUTE_SIGMOID = 1 };
+
+typedef struct {
+    int n_layer, n_exp, top_k, d, ff;
+    int fmt;       /* MF_SEED4P4 or MF_SEED4: the experts' format */
+    int router;    /* NSLM_ROUTE_SOFTMAX: logits = bf16(W x) by kc_mv on a BF16 router weight, kq4_route, kq4_moe_combine
+                      (f32 sums; the Qwen composition).  NSLM_ROUTE_SIGMOID: kc_router, kc_moe_combine (BF16 rounding at
+                      every tensor boundary; the MoVA composition) */
+    int max_rows;  /* most tokens a step takes */
+    int slots;     /* pool slots; 0 or >= n_layer * n_exp: all resident */
+    float route_scale;
+} NslmMoeCfg;
+
+typedef struct NslmMoe NslmMoe;
+
+NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen);
+void nslm_moe_close(NslmMoe* m);
+/* tensor: 0 gate [ff][d], 1 up [ff][d], 2 down [d][ff].  Host streams of ONE expert: seeds, words (coefficient or nibble
+ * words), codes (P = 4 only), exponent bias.  Call for every (layer, expert, tensor) before nslm_moe_finalize. */
+int nslm_moe_set_expert(NslmMoe* m, int layer, int expert, int tensor, const uint16_t* seeds, const uint16_t* words,
+                        const uint8_t* codes, int eb);
+/* router weight [n_exp][d] as BF16 bits; bias [n_exp] BF16 bits (sigmoid router only, else NULL) */
+int nslm_moe_set_router(NslmMoe* m, int layer, const uint16_t* W, const uint16_t* bias);
+int nslm_moe_finalize(NslmMoe* m);
+/* One MoE layer for T rows, asynchronous on stream s (launches only, capturable into a graph).
+ * xn: the layer input [T][d] (device).  io [T][d] (device): softmax composition: receives sum_k wt_k y_k;
+ * sigmoid composition: the residual stream, updated in place x = bf16(x + bf16(bf16(sum) + 0)). */
+int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, float* io);
+/* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */
+int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
+/* the slot table's counters and state (synchronises): hits, misses since open */
+int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
+uint64_t nslm_moe_unit_bytes(const NslmMoe* m);
+/* compressed bytes one expert's three matrices occupy (without alignment padding) */
+uint64_t nslm_moe_expert_bytes(const NslmMoe* m);
+
+/* ---- capture / replay of a launch sequence (hipGraph), and event timing, for hosts without HIP headers ---- */
+typedef struct NslmGraph NslmGraph;
+int nslm_graph_begin(kc_stream_t s);                 /* start capturing s */
+NslmGraph* nslm_graph_end(kc_stream_t s);            /* end capture and instantiate; NULL on failure */
+int nslm_graph_launch(NslmGraph* g, kc_stream_t s);
+void nslm_graph_free(NslmGraph* g);
+
+#ifdef __cplusplus
+}
+#endif

@@ -56,4 +56,28 @@ int nh_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {
     return (int) e;
 }
 
+// ---- capture / replay of a launch sequence (declared in moe_layer.h) ----
+struct NslmGraph {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+int nslm_graph_begin(void* s) { return (int) hipStreamBeginCapture((hipStream_t) s, hipStreamCaptureModeThreadLocal); }
+NslmGraph* nslm_graph_end(void* s) {
+    hipGraph_t g = nullptr;
+    if (hipStreamEndCapture((hipStream_t) s, &g) != hipSuccess || !g) return nullptr;
+    hipGraphExec_t ex = nullptr;
+    if (hipGraphInstantiate(&ex, g, nullptr, nullptr, 0) != hipSuccess) {
+        hipGraphDestroy(g);
+        return nullptr;
+    }
+    return new NslmGraph{g, ex};
+}
+int nslm_graph_launch(NslmGraph* g, void* s) { return (int) hipGraphLaunch(g->exec, (hipStream_t) s); }
+void nslm_graph_free(NslmGraph* g) {
+    if (!g) return;
+    hipGraphExecDestroy(g->exec);
+    hipGraphDestroy(g->graph);
+    delete g;
+}
+
 }   // extern "C"
