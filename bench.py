@@ -1,0 +1,291 @@
+#!/usr/bin/env python3
+"""bench.py - the SeedLM decode-in-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1] [--no-cpu]
+
+A step is one pass of the workload over one batch of seeded synthetic input already resident in HBM:
+  c2b1 (default; the configuration the metric is quoted on): one MoE decode layer step at batch 1 - 128 experts seeded
+        P=4, top-8 softmax routing, hidden 2048, expert intermediate 768 (router GEMV, top-k, fused gate+up+SwiGLU
+        gather, down gather, combine).  Steps rotate over `layers` resident layers and 16 inputs so the selected experts
+        change from step to step and the traffic comes from HBM, not from the 256 MB Infinity Cache.
+  c2b8 / c2b32: the same at 8 and 32 tokens (32: grouping + grouped MFMA GEMMs).
+  c0:   dense GEMV, W 4096x4096 P=4, batch 1, rotating over 64 matrices (604 MB).
+  c1:   prefill GEMM, W 14336x4096 P=4, X bf16 [512 x 4096].
+  c3b1: 64 experts P=3 top-4, hidden 2880, intermediate 2880, batch 1.
+Prints ONE JSON line: value = effective GB/s of compressed weight bytes (whole job), with the dominant kernel's roofline
+(timed live with HIP events on the launch stream) and the CPU baseline (the reference's own lib_cpu_seed4 when the
+compiled reference is present, else this repository's restatement) on a bounded sample of the same workload."""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "seeded GEMV effective GB/s (%HBM peak); MoE decode tokens/s at batch 1"
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def moe_workload(name, steps, warmup, n_layers, no_graph):
+    from nanoseedlm_amd import backend, moe, packs
+    cfgs = {"c2": dict(E=128, k=8, d=2048, ff=768, fmt=packs.MF_SEED4P4), "c3": dict(E=64, k=4, d=2880, ff=2880, fmt=packs.MF_SEED4)}
+    c = cfgs[name[:2]]
+    T = int(name[3:])
+    E, k, d, ff, fmt = c["E"], c["k"], c["d"], c["ff"], c["fmt"]
+    rng = np.random.default_rng(20261125)
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    st = moe.MoeStack(n_layers, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=max(T, 8))
+    for l in range(n_layers):
+        gate, up, down = mk(rng, E, ff, d, eb=-22), mk(rng, E, ff, d, eb=-22), mk(rng, E, d, ff, eb=-22)
+        rw = packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.02).astype(np.float32))
+        st.set_layer(l, gate, up, down, rw)
+        del gate, up, down
+    st.finalize()
+    NX = 16
+    xs = [moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))) for _ in range(NX)]
+    out = moe.DevBuf(4 * T * d)
+    stream = moe.new_stream()
+    combos = [(l, xi) for xi in range(NX) for l in range(n_layers)]
+    graphs = None
+    if not no_graph:
+        for l, xi in combos[:2]:
+            st.step(stream, l, xs[xi].ptr, T, out.ptr)          # warm every kernel before capture
+        moe.device_sync()
+        graphs = [st.graph_of_step(stream, l, xs[xi].ptr, T, out.ptr) for l, xi in combos]
+
+    def run(i):
+        l, xi = combos[i % len(combos)]
+        if graphs:
+            st.launch(graphs[i % len(combos)], stream)
+        else:
+            st.step(stream, l, xs[xi].ptr, T, out.ptr)
+
+    for i in range(warmup):
+        run(i)
+    moe.device_sync()
+    e0, e1 = moe.Event(), moe.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        run(warmup + i)
+    e1.record(stream)
+    e1.sync()
+    moe.device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = e1.ms_since(e0) / steps
+
+    # bytes: unique selected experts x expert bytes + the BF16 router weight; at batch 1 every pair is unique
+    uniq = []
+    for i in range(min(steps, len(combos))):
+        l, xi = combos[(warmup + i) % len(combos)]
+        st.step(stream, l, xs[xi].ptr, T, out.ptr)
+        ind, _ = st.last_routing(T)
+        uniq.append(len(set(ind.reshape(-1).tolist())))
+    eb = st.expert_bytes()
+    bytes_step = float(np.mean(uniq)) * eb + E * d * 2
+    res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T,
+               flops_per_step=2.0 * T * k * 3 * d * ff)
+
+    # dominant kernel alone, timed with events on its stream
+    P = T * k
+    L = backend.hip()
+    if T <= 8:
+        ind = moe.DevBuf.from_array(np.stack([rng.permutation(E)[:k] for _ in range(T * NX)]).astype(np.int32))
+        A = moe.DevBuf(4 * P * ff)
+        reps = max(50, steps)
+        st.L.nslm_moe_tab.restype = C.c_void_p
+
+        def gu(i):
+            l, xi = combos[i % len(combos)]
+            g = C.c_void_p(st.L.nslm_moe_tab(st.h, l, 0))
+            u = C.c_void_p(st.L.nslm_moe_tab(st.h, l, 1))
+            L.kc_mv_gu(stream, fmt, g, u, d, ff, xs[xi].ptr, d, A.ptr, ff, ind.at(4 * P * xi), P, k, None)
+        for i in range(10):
+            gu(i)
+        moe.device_sync()
+        e0.record(stream)
+        for i in range(reps):
+            gu(i)
+        e1.record(stream)
+        e1.sync()
+        kms = e1.ms_since(e0) / reps
+        kbytes = P * 2 * eb / 3.0        # P pairs x (gate + up) records
+        res["roofline"] = dict(bound="hbm", achieved=kbytes / kms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
+                               frac=kbytes / kms / 1e6 / HBM_PEAK_GBS, traffic=None, kernel="k_mv_seed<gate+up+SwiGLU>",
+                               launch_us=kms * 1e3, algorithmic_bytes=kbytes)
+        ind.free(); A.free()
+    else:
+        res["roofline"] = dict(bound="mfma", achieved=res["flops_per_step"] / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                               frac=res["flops_per_step"] / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, traffic=None,
+                               kernel="k_mm grouped (whole step)")
+    desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",
+            "c3": "C3 MoE decode layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880"}[name[:2]]
+    res["config"] = {"workload": f"{desc}, batch {T}", "layers_rotated": n_layers, "inputs_rotated": NX,
+                     "launch": "stream" if no_graph else "hipGraph per step"}
+    res["cpu_sample"] = dict(shapes=[(ff, d), (ff, d), (d, ff)], reps=k, fmt=fmt)
+    st.close()
+    return res
+
+
+def dense_workload(name, steps, warmup):
+    from nanoseedlm_amd import backend, moe, packs
+    L = backend.hip()
+    rng = np.random.default_rng(20261125)
+    stream = moe.new_stream()
+    e0, e1 = moe.Event(), moe.Event()
+    if name == "c0":
+        R = K = 4096
+        NM = 64
+        p = packs.seed4p4(rng, NM, R, K, eb=-22)
+        ds, dc, de = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
+        x = moe.DevBuf.from_array(rng.standard_normal(K).astype(np.float32))
+        y = moe.DevBuf(4 * R)
+        sl = []
+        for i in range(NM):
+            w = backend.WSlice()
+            w.p[0], w.p[1], w.p[3] = ds.ptr.value + i * R * K // 4, dc.ptr.value + i * R * K // 4, de.ptr.value + i * R * K // 16
+            w.eb = -22
+            sl.append(w)
+
+        def run(i):
+            L.kc_mv(stream, packs.MF_SEED4P4, sl[i % NM], K, R, x.ptr, K, y.ptr, R, 1, 0, None)
+        bytes_step, flops, T = R * K * 36 / 64.0, 2.0 * R * K, 1
+        desc, bound = "C0 dense seeded GEMV: W 4096x4096 P=4, batch 1, rotating over 64 matrices", "hbm"
+        sample = dict(shapes=[(R, K)], reps=1, fmt=packs.MF_SEED4P4)
+    else:
+        R, K, T = 14336, 4096, 512
+        p = packs.seed4p4(rng, 1, R, K, eb=-22)
+        ds, dc, de = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
+        x = moe.DevBuf.from_array(packs.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32)))
+        y = moe.DevBuf(4 * T * R)
+        w = backend.WSlice()
+        w.p[0], w.p[1], w.p[3] = ds.ptr.value, dc.ptr.value, de.ptr.value
+        w.eb = -22
+
+        def run(i):
+            L.kc_mm_packed(stream, packs.MF_SEED4P4, w, K, R, x.ptr, K, y.ptr, R, T, 0, None)
+        bytes_step, flops = R * K * 36 / 64.0, 2.0 * T * R * K
+        desc, bound = "C1 seeded prefill GEMM: W 14336x4096 P=4, X bf16 [512 x 4096], bf16 MFMA, fp32 accumulate", "mfma"
+        sample = dict(shapes=[(R, K)], reps=1, fmt=packs.MF_SEED4P4)
+    for i in range(warmup):
+        run(i)
+    moe.device_sync()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        run(warmup + i)
+    e1.record(stream)
+    e1.sync()
+    moe.device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = e1.ms_since(e0) / steps
+    backend.check(L.kc_last_error(), "kernel launch")
+    res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
+    if bound == "hbm":
+        res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=None, kernel="k_mv_seed<dense>",
+                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
+    else:
+        res["roofline"] = dict(bound="mfma", achieved=flops / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                               frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, traffic=None, kernel="k_mm<4,1,packed>",
+                               launch_us=ms * 1e3, algorithmic_flops=flops)
+    res["config"] = {"workload": desc, "launch": "stream"}
+    res["cpu_sample"] = sample
+    return res
+
+
+def cpu_baseline(sample, budget_s=12.0):
+    """The CPU decode-in-dot-product on this host's cores over the workload's matrices (a bounded sample: the matrices
+    one token reads, repeated until about budget_s of CPU time)."""
+    from nanoseedlm_amd import packs
+    from oracle import oracle as orc
+    orc.build()
+    ref = orc.ref()
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    rng = np.random.default_rng(7)
+    fmt = sample["fmt"]
+    mats = []
+    weights = 0
+    for (R, K) in sample["shapes"]:
+        if R * K > 2 ** 25:          # bound the sample: at most 32 M weights per matrix
+            R = 2 ** 25 // K
+        p = (packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4)(rng, 1, R, K, eb=-22)
+        mats.append((p, R, K, rng.standard_normal(K).astype(np.float32)))
+        weights += R * K
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)
+    if ref is not None:
+        kind = "reference"
+        tiled = []
+        for p, R, K, x in mats:
+            t = ref.ref_tile4(vp(p["seeds"][0]), vp(p["coefs"][0]), vp(p["codes"][0]), -22, R, K // 8) if fmt == packs.MF_SEED4P4 \
+                else ref.ref_tile3(vp(p["seeds"][0]), vp(p["nibs"][0]), -22, R, K // 8)
+            tiled.append((C.c_void_p(t), x, np.zeros(R, dtype=np.float32)))
+
+        def once():
+            for t, x, y in tiled:
+                ref.ref_tiled_matmul(t, vp(x), 1, vp(y), threads)
+    else:
+        kind = "port"
+        threads = min(cores, 16)
+
+        def once():
+            for p, R, K, x in mats:
+                if fmt == packs.MF_SEED4P4:
+                    orc.cpu_seed4_matvec(p["seeds"][0], p["coefs"][0], p["codes"][0], -22, x, R, K // 8, threads)
+                else:
+                    orc.cpu_seed3_matvec(p["seeds"][0], p["nibs"][0], -22, x, R, K // 8, threads)
+    once()
+    n, t0 = 0, time.perf_counter()
+    best = 1e30
+    while time.perf_counter() - t0 < budget_s:
+        t1 = time.perf_counter()
+        once()
+        best = min(best, time.perf_counter() - t1)
+        n += 1
+    bpw = 0.5625 if fmt == packs.MF_SEED4P4 else 0.5
+    return dict(value=weights * bpw / best / 1e9, unit="GB/s", cores=threads, kind=kind, gweights_per_s=weights / best / 1e9,
+                sample=f"{len(mats)} matrices {[(R, K) for _, R, K, _ in mats]} ({weights / 1e6:.1f} M weights) x {n} passes, best pass "
+                       f"{best * 1e3:.2f} ms, host cores visible {cores}, loadavg {open('/proc/loadavg').read().split()[0]}"
+                       + ("" if ref is not None else "; scalar C restatement (compiled reference not present)"))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default="c2b1")
+    ap.add_argument("--layers", type=int, default=4)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU (one process, one MI355X, no collectives); run with --gpus 1")
+    from nanoseedlm_amd import backend
+    backend.require_gpu()
+    if a.workload[:2] in ("c2", "c3"):
+        r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph)
+    else:
+        r = dense_workload(a.workload, a.steps, a.warmup)
+    gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6
+    line = {
+        "metric": METRIC, "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic", "config": r["config"], "pct_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
+        "tokens_per_s": r["tokens"] / r["ms_per_step"] * 1e3, "bytes_per_step": r["bytes_per_step"],
+        "tflops": r["flops_per_step"] / r["ms_per_step"] / 1e9, "host_ms_per_step": r["wall_ms_per_step"],
+        "roofline": r["roofline"],
+    }
+    line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(r["cpu_sample"])
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

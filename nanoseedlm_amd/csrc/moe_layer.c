@@ -224,6 +224,7 @@ int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses) {
     *misses = st[1];
     return 0;
 }
+const WSlice* nslm_moe_tab(const NslmMoe* m, int layer, int tensor) { return m->pool.tab + ((size_t) layer * 3 + tensor) * m->c.n_exp; }
 uint64_t nslm_moe_unit_bytes(const NslmMoe* m) { return m->unit_bytes; }
 uint64_t nslm_moe_expert_bytes(const NslmMoe* m) {
     uint64_t n = 0;

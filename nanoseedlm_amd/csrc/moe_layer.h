@@ -45,6 +45,8 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
 /* the slot table's counters and state (synchronises): hits, misses since open */
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
+/* the device slice table [n_exp] of a layer's tensor (0 gate, 1 up, 2 down): what kc_mv_gu / kc_mv_sel take */
+const WSlice* nslm_moe_tab(const NslmMoe* m, int layer, int tensor);
 uint64_t nslm_moe_unit_bytes(const NslmMoe* m);
 /* compressed bytes one expert's three matrices occupy (without alignment padding) */
 uint64_t nslm_moe_expert_bytes(const NslmMoe* m);

@@ -67,7 +67,7 @@ NslmGraph* nslm_graph_end(void* s) {
     if (hipStreamEndCapture((hipStream_t) s, &g) != hipSuccess || !g) return nullptr;
     hipGraphExec_t ex = nullptr;
     if (hipGraphInstantiate(&ex, g, nullptr, nullptr, 0) != hipSuccess) {
-        hipGraphDestroy(g);
+        (void) hipGraphDestroy(g);
         return nullptr;
     }
     return new NslmGraph{g, ex};
@@ -75,8 +75,8 @@ NslmGraph* nslm_graph_end(void* s) {
 int nslm_graph_launch(NslmGraph* g, void* s) { return (int) hipGraphLaunch(g->exec, (hipStream_t) s); }
 void nslm_graph_free(NslmGraph* g) {
     if (!g) return;
-    hipGraphExecDestroy(g->exec);
-    hipGraphDestroy(g->graph);
+    (void) hipGraphExecDestroy(g->exec);
+    (void) hipGraphDestroy(g->graph);
     delete g;
 }
 

@@ -18,6 +18,7 @@ def _lib():
     L = backend.kt()
     L.nslm_moe_open.restype = C.c_void_p
     L.nslm_graph_end.restype = C.c_void_p
+    L.nslm_moe_tab.restype = C.c_void_p
     L.nslm_moe_unit_bytes.restype = C.c_uint64
     L.nslm_moe_expert_bytes.restype = C.c_uint64
     return L
