@@ -91,6 +91,13 @@ typedef short short2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ int dot2(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot2(__builtin_bit_cast(short2v, a), __builtin_bit_cast(short2v, b), c, false);
 }
+// the same with a zero addend: the three-source encoding takes the constant inline, where the accumulating two-source
+// form the compiler picks for dot2(a, b, 0) would first spend a move on zeroing its destination
+__device__ __forceinline__ int dot2z(uint32_t a, uint32_t b) {
+    int d;
+    asm("v_dot2_i32_i16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
 // { word X's half hx, word Y's half hy } as one packed pair
 __device__ __forceinline__ uint32_t halves(uint32_t X, int hx, uint32_t Y, int hy) {
     const uint32_t sel = (uint32_t) (2 * hx) | ((uint32_t) (2 * hx + 1) << 8) | ((uint32_t) (4 + 2 * hy) << 16) |
@@ -113,8 +120,8 @@ __device__ __forceinline__ void isum_p4(uint32_t up, uint32_t g, uint32_t q01, u
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const int k = 4 * c + 1;
-        is[c] = dot2(halves(A[k], 0, A[k + 1], 0), q01, dot2(halves(A[k + 2], 0, A[k + 3], 0), q23, 0));
-        is[c + 4] = dot2(halves(A[k], 1, A[k + 1], 1), q01, dot2(halves(A[k + 2], 1, A[k + 3], 1), q23, 0));
+        is[c] = dot2(halves(A[k], 0, A[k + 1], 0), q01, dot2z(halves(A[k + 2], 0, A[k + 3], 0), q23));
+        is[c + 4] = dot2(halves(A[k], 1, A[k + 1], 1), q01, dot2z(halves(A[k + 2], 1, A[k + 3], 1), q23));
     }
 }
 // P = 3: weight c reads states 3c+1..3c+3; q01 = {q0,q1}, q2 = {q2,0} (reference nslm/lfsr.h:116-128)
@@ -126,7 +133,7 @@ __device__ __forceinline__ void isum_p3(uint32_t up, uint32_t g, uint32_t q01, u
     for (int c = 0; c < 8; ++c) {
         const int k0 = 3 * c + 1, k1 = k0 + 1, k2 = k0 + 2;   // state k lives in A[k] low (k <= 16) or A[k-16] high
         const uint32_t pr = halves(A[k0 <= 16 ? k0 : k0 - 16], k0 > 16, A[k1 <= 16 ? k1 : k1 - 16], k1 > 16);
-        const int third = k2 <= 16 ? dot2(A[k2], q2, 0) : dot2(A[k2 - 16], q2hi, 0);
+        const int third = k2 <= 16 ? dot2z(A[k2], q2) : dot2z(A[k2 - 16], q2hi);
         is[c] = dot2(pr, q01, third);
     }
 }

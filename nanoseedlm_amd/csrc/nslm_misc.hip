@@ -29,12 +29,13 @@ __global__ void __launch_bounds__(256) k_router_logits(RouterArgs a, const uint1
     const uint16_t* wr = W + (size_t) e * a.d;
     float s0 = 0.0f, s1 = 0.0f;
     for (int c = lane * 4; c < a.d; c += 256) {
-        float v = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (c + i < a.d) v = fmaf(bf(wr[c + i]), xr[c + i], v);
-        if (c < a.hw) s0 += v;   // hw is a multiple of 4 for every model width; a straddling group counts on its first column
-        else s1 += v;
+        for (int i = 0; i < 4; ++i) {
+            if (c + i >= a.d) break;
+            const float v = bf(wr[c + i]) * xr[c + i];
+            if (c + i < a.hw) s0 += v;
+            else s1 += v;
+        }
     }
     s0 = wave_sum(s0);
     s1 = wave_sum(s1);
@@ -54,8 +55,8 @@ __global__ void __launch_bounds__(64) k_router_topk(RouterArgs a, const float* s
     float v[RT_PER];
 #pragma unroll
     for (int j = 0; j < RT_PER; ++j) v[j] = lane + 64 * j < a.n ? se[lane + 64 * j] : NEG_INF;
-    int chosen[32];
-    float sum = 0.0f;
+    int mine = 0;          // round r's winner is kept by lane r (top_k <= 32)
+    float mine_sc = 0.0f, sum = 0.0f;
     for (int k = 0; k < a.top_k; ++k) {
         float bv = NEG_INF;
         int bi = 1 << 20;
@@ -72,21 +73,23 @@ __global__ void __launch_bounds__(64) k_router_topk(RouterArgs a, const float* s
 #pragma unroll
         for (int j = 0; j < RT_PER; ++j)
             if (lane + 64 * j == bi) v[j] = NEG_INF;
-        chosen[k] = bi;
-        sum += sc[bi];
+        const float s = sc[bi];
+        sum += s;
+        if (lane == k) { mine = bi; mine_sc = s; }
     }
-    if (lane == 0)
-        for (int k = 0; k < a.top_k; ++k) {
-            inds[t * a.top_k + k] = chosen[k];
-            wts[t * a.top_k + k] = sc[chosen[k]] / sum * a.scale;
-        }
+    if (lane < a.top_k) {
+        inds[t * a.top_k + lane] = mine;
+        wts[t * a.top_k + lane] = mine_sc / sum * a.scale;
+    }
 }
 
 // ---- softmax router: top k by logit (ties to the HIGHER index), weights = softmax renormalised over the k picked ------
+// Round r's winner is kept by lane r (k <= 32 < 64 lanes), so nothing is indexed dynamically.
 __global__ void __launch_bounds__(64) k_q4_route(int E, int k, const float* logits, int ld, int32_t* ind, float* wt) {
     const int t = (int) blockIdx.x, lane = threadIdx.x;
     const float* l = logits + (size_t) t * ld;
-    float v[RT_PER], mx = NEG_INF, top = 0.0f, w[32];
+    float v[RT_PER], mx = NEG_INF, top = 0.0f, mine = 0.0f;
+    int mine_id = 0;
 #pragma unroll
     for (int j = 0; j < RT_PER; ++j) {
         v[j] = lane + 64 * j < E ? l[lane + 64 * j] : NEG_INF;
@@ -109,12 +112,14 @@ __global__ void __launch_bounds__(64) k_q4_route(int E, int k, const float* logi
 #pragma unroll
         for (int j = 0; j < RT_PER; ++j)
             if (lane + 64 * j == bi) v[j] = NEG_INF;
-        if (lane == 0) ind[(size_t) t * k + r] = bi;
-        w[r] = expf(bv - mx);
-        top += w[r];
+        const float w = expf(bv - mx);
+        top += w;
+        if (lane == r) { mine = w; mine_id = bi; }
     }
-    if (lane == 0)
-        for (int r = 0; r < k; ++r) wt[(size_t) t * k + r] = w[r] / top;
+    if (lane < k) {
+        ind[(size_t) t * k + lane] = mine_id;
+        wt[(size_t) t * k + lane] = mine / top;
+    }
 }
 
 // ---- elementwise --------------------------------------------------------------------------------------------------------

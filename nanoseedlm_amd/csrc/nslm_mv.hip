@@ -14,6 +14,8 @@
 // engine/kernels_moe.cu:239-240).
 //
 // Generic path (k_mv_any): one wave per row, lanes over blocks; every format, any K % 8 == 0, any alignment.
+#include <stdlib.h>
+
 #include "nslm_dev.h"
 
 using namespace nslm;
@@ -348,8 +350,10 @@ int pick_rows_per_wg(int V, int rpi, int ny) {
     const int iters = (V + rpi - 1) / rpi;
     const int want = 3 * cu_count();
     int per = (iters * ny + want - 1) / want;
+    static const char* env = getenv("NSLM_MV_ITERS");   // tuning override: iterations per workgroup
+    if (env && atoi(env) > 0) per = atoi(env);
     if (per < 1) per = 1;
-    if (per > 16) per = 16;
+    if (per > 64) per = 64;
     return per * rpi;
 }
 
