@@ -153,6 +153,20 @@ void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out)
 /* 1: the matvec family stores unrounded f32 instead of BF16-rounded values (for comparison with CPU references that do
  * not round, nslm/lib_cpu_seed4.c).  Process-global like kc_seed_gemm_f32; default 0 = the reference's store. */
 void kc_store_f32(int on);
+/* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
+ * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same
+ * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.
+ * Scratch (caller-owned device memory): logits [T][n_exp], ind / wt [T][top_k] (the routing, also an output), A [T*k][ff],
+ * D [T*k][d], sync: kc_moe_decode_sync_words(T, d) uint32 that must be zero before the first call (the kernel keeps them
+ * consistent from launch to launch; sync[kc_moe_decode_error_word()] != 0 afterwards reports a grid barrier that gave up,
+ * after which the caller must zero sync again).
+ * The grid spans the whole device and its workgroups wait for each other: nothing else may run on the GPU beside it.
+ * Returns 0, or -1 when the shape has no fused kernel (nothing launched: use the separate launchers). */
+size_t kc_moe_decode_sync_words(int T, int d);
+int kc_moe_decode_error_word(void);
+int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
+                  int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
+                  int32_t* ind, float* wt, float* A, float* D, uint32_t* sync);
 /* last launch-configuration error of this library on the calling thread's device: 0 none, else a hipError_t value */
 int kc_last_error(void);
 

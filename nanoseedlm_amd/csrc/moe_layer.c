@@ -20,6 +20,8 @@ struct NslmMoe {
     int32_t *ind, *perm, *ntiles;
     MmTile* tiles;
     int max_tiles;
+    uint32_t* sync;             /* device: the fused decode kernel's barrier words */
+    int fused;                  /* 1: T <= MV_MAXT steps of the softmax composition take kc_moe_decode */
 };
 
 static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
@@ -86,6 +88,8 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     bad |= nh_malloc((void**) &m->perm, 4 * (size_t) P);
     bad |= nh_malloc((void**) &m->tiles, sizeof(MmTile) * (size_t) m->max_tiles);
     bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 3));
+    bad |= nh_malloc((void**) &m->sync, 4 * kc_moe_decode_sync_words(MV_MAXT, c->d));
+    m->fused = 1;
     m->unit_host = (uint8_t*) calloc(1, cur);
     m->eb = (int32_t*) calloc((size_t) m->units * 3, 4);
     if (bad || !m->unit_host || !m->eb) {
@@ -94,6 +98,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
         return NULL;
     }
     nh_memset(m->zero, 0, 4 * (size_t) c->max_rows * c->d);
+    nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(MV_MAXT, c->d));
     nh_memset(m->rb, 0, 2 * (size_t) c->n_layer * c->n_exp);
     return m;
 }
@@ -102,7 +107,7 @@ void nslm_moe_close(NslmMoe* m) {
     if (!m) return;
     void* d[] = {m->arena, m->resident ? NULL : m->pool.vram, m->pool.unit_slot, m->pool.slot_unit, m->pool.slot_last, m->pool.tick,
                  m->pool.stats, m->pool.jobs, m->pool.njobs, m->pool.tab, m->rw, m->rb, m->logit, m->score, m->wt, m->ind, m->A,
-                 m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles};
+                 m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles, m->sync};
     for (size_t i = 0; i < sizeof d / sizeof d[0]; ++i)
         if (d[i]) nh_free(d[i]);
     free(m->unit_host);
@@ -179,6 +184,10 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
     const WSlice* gate = m->pool.tab + ((size_t) layer * 3 + 0) * E;
     const WSlice* up = m->pool.tab + ((size_t) layer * 3 + 1) * E;
     const WSlice* down = m->pool.tab + ((size_t) layer * 3 + 2) * E;
+    if (m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= MV_MAXT &&
+        !kc_moe_decode(s, c->fmt, m->rw + (size_t) layer * E * d, gate, up, down, E, k, d, ff, xn, d, T, io, d, m->logit, m->ind,
+                       m->wt, m->A, m->D, m->sync))
+        return kc_last_error() ? -1 : 0;   /* the whole step in one persistent kernel */
     if (c->router == NSLM_ROUTE_SOFTMAX) {
         WSlice rw;
         memset(&rw, 0, sizeof rw);
@@ -211,6 +220,14 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
     if (c->router == NSLM_ROUTE_SOFTMAX) kq4_moe_combine(s, d, k, m->D, m->wt, m->zero, m->zero, 0, io, T);
     else kc_moe_combine(s, m->D, m->wt, m->zero, io, d, k, T);
     return kc_last_error() ? -1 : 0;
+}
+
+void nslm_moe_set_fused(NslmMoe* m, int on) { m->fused = on; }
+void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }
+int nslm_moe_fused_error(NslmMoe* m) {
+    uint32_t w = 0;
+    if (nh_device_sync() || nh_memcpy_d2h(&w, m->sync + kc_moe_decode_error_word(), 4)) return -1;
+    return (int) w;
 }
 
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {

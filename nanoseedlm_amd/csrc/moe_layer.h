@@ -41,6 +41,11 @@ int nslm_moe_finalize(NslmMoe* m);
  * xn: the layer input [T][d] (device).  io [T][d] (device): softmax composition: receives sum_k wt_k y_k;
  * sigmoid composition: the residual stream, updated in place x = bf16(x + bf16(bf16(sum) + 0)). */
 int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, float* io);
+/* 1 (default): decode steps of the softmax composition with every expert resident run as one persistent kernel
+ * (kc_moe_decode); 0: always the separate launchers.  The results are the same bits either way. */
+void nslm_moe_set_fused(NslmMoe* m, int on);
+/* 0, or non-zero when a grid barrier of the fused kernel gave up since open (synchronises) */
+int nslm_moe_fused_error(NslmMoe* m);
 /* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
 /* the slot table's counters and state (synchronises): hits, misses since open */

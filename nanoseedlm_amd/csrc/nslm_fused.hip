@@ -1,0 +1,394 @@
+// nslm_fused.hip - one persistent kernel for a whole routed-expert decode step at T <= 8 tokens: router logits, softmax
+// top-k, fused gate + up + SwiGLU gather, down gather, weighted combine.  No counterpart in the reference, which launches
+// these as five kernels (engine/qwen4_cuda.c:1023-1083); on MI355X each launch and each dependent global read costs
+// microseconds that a ~20 us step cannot afford, so the phases run inside one grid separated by grid-wide barriers.
+//
+// Arithmetic is the stand-alone kernels', instruction for instruction (k_mv_any's BF16 row dot, k_q4_route's selection
+// and weights, k_mv_seed's chunk products and row-sum order, k_q4_moe_combine's sum), so the fused step returns the same
+// bits as the five launches.
+//
+// Data that one workgroup writes and another reads inside the launch (logits, A, D) moves with agent-scope relaxed
+// atomic stores and loads: on this GPU every XCD has its own L2, and those accesses go through to the coherent level, so
+// no device-scope fence (an L2 write-back / invalidate per workgroup, which costs far more than the step) is needed;
+// ordering against the barrier counters is a workgroup-scope release / acquire, i.e. a wait for outstanding memory
+// operations.
+//
+// Grid barriers: the grid is sized to the number of workgroups the device can hold at once (occupancy query), every
+// workgroup arrives on a counter in caller-provided scratch and spins until all have; the spin is bounded, and a
+// workgroup that gives up sets an error word and runs on to the end, so every wave always exits.
+#include <stdlib.h>
+
+#include "nslm_mv_dev.h"
+
+using namespace nslm;
+
+namespace {
+
+struct FusedArgs {
+    const uint16_t* rw;                 // router weight BF16 [E][d]
+    const WSlice *gate, *up, *down;     // device slice tables [E]
+    const float* x;                     // [T][xs]
+    float* out;                         // [T][os]
+    float *logits, *wt, *A, *D;         // scratch: [T][E], [T][k], [T*k][ff], [T*k][d]
+    int32_t* ind;                       // [T][k]
+    uint32_t* sync;                     // [FUSED_SYNC_WORDS + T * ntile_d], see below
+    int E, k, d, ff, T, xs, os;
+    int Lg, rpig, rows_g, ntile_g;      // gate+up pass: chunks per row, virtual rows per iteration / per item, items per pair
+    int Ld, rpid, rows_d, ntile_d;      // down pass
+    int grid;
+};
+
+// Barrier words (uint32; every counter sits alone on a 128-byte line = 32 words):
+//   [32 g]              arrivals of group g = blockIdx.x % BAR_GROUPS
+//   [32 BAR_GROUPS]     groups that are complete
+//   [32 (BAR_GROUPS+1+g)] group g's sense word: flipped when the barrier opens
+//   [32 (2 BAR_GROUPS+1)] error word
+//   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile)
+// Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
+// counters and only each group's last arrival touches the shared one; waiters poll their own group's sense word.  The
+// barrier is sense-reversing and resets its own counters, so the words need no clean-up between launches.
+#define BAR_GROUPS 32
+#define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
+#define FUSED_SYNC_WORDS (32 * (2 * BAR_GROUPS + 2))
+#define SPIN_LIMIT (1u << 21)
+
+__device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// this workgroup's earlier memory operations have completed / later ones start after this point
+__device__ __forceinline__ void wg_release() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+__device__ __forceinline__ void wg_acquire() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
+
+// every workgroup of the grid arrives and waits (bounded); data written before it by any workgroup is visible after it
+__device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G) {
+    wg_release();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t g = blockIdx.x % BAR_GROUPS, ng = G < BAR_GROUPS ? G : BAR_GROUPS, mine = (G - g + BAR_GROUPS - 1) / BAR_GROUPS;
+        uint32_t* sense = sync + 32 * (BAR_GROUPS + 1 + g);
+        const uint32_t s = ld_agent(sense);   // read before arriving: the barrier cannot open without this arrival
+        if (atomicAdd(sync + 32 * g, 1u) == mine - 1) {
+            st_agent(sync + 32 * g, 0u);
+            if (atomicAdd(sync + 32 * BAR_GROUPS, 1u) == ng - 1) {
+                st_agent(sync + 32 * BAR_GROUPS, 0u);
+                wg_release();   // every counter is back at zero before anyone is let through
+                for (uint32_t i = 0; i < ng; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), s ^ 1u);
+            }
+        }
+        uint32_t spins = 0;
+        while (ld_agent(sense) == s) {
+            __builtin_amdgcn_s_sleep(4);
+            if (++spins > SPIN_LIMIT) {
+                atomicExch(&sync[FUSED_ERR_WORD], 1u);
+                break;
+            }
+        }
+    }
+    __syncthreads();
+    wg_acquire();
+}
+
+// The first chunk of a pass over rows [v0, v1): issued as early as the slices are known, so its latency hides behind
+// whatever comes before the pass (a grid barrier, the staging of the activations).
+template <int P, bool GATEUP>
+__device__ __forceinline__ Chunk first_chunk(const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1) {
+    const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L, vv = v0 + lr;
+    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
+    const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
+    return load_chunk<P>(w, (uint32_t) (GATEUP ? vv >> 1 : vv) * (uint32_t) L + (uint32_t) ch, lr < rpi && vv < v1, al);
+}
+
+// rows [v0, v1) of one pair: the k_mv_seed loop with the activations in LDS (xl, chunk-padded).  emit(row, sum, other)
+// is called by the thread that owns a finished row sum.
+template <int P, bool GATEUP, bool SHFL, typename Emit>
+__device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1,
+                                          const uint32_t* tab, const float* xl, float (*part)[256], Emit emit) {
+    const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
+    const bool active = lr < rpi;
+    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
+    auto fetch = [&](int vv) {
+        const bool ok = active && vv < v1;
+        const int r = GATEUP ? vv >> 1 : vv;
+        const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
+        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
+    };
+    int par = 0;
+    for (int vb = v0; vb < v1; vb += rpi, par ^= 1) {
+        const int v = vb + lr;
+        const Chunk nxt = fetch(v + rpi);
+        float acc[1] = {0.0f};
+        const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
+        if (active && v < v1) chunk_dot<P, 1>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
+        if (SHFL) {
+            float s = acc[0];
+            for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            if (GATEUP) {
+                const float other = __shfl_xor(s, L);
+                if (active && ch == 0 && !(v & 1) && v < v1) emit(v >> 1, s * NSLM_R32, other * NSLM_R32);
+            } else if (active && ch == 0 && v < v1) emit(v, s * NSLM_R32, 0.0f);
+        } else {
+            part[par][tid] = acc[0];
+            __syncthreads();
+            const int nrow = min(rpi, v1 - vb);
+            if (GATEUP) {
+                if (tid < nrow / 2) {
+                    float gs = 0.0f, us = 0.0f;
+                    for (int j = 0; j < L; ++j) gs += part[par][(2 * tid) * L + j];
+                    for (int j = 0; j < L; ++j) us += part[par][(2 * tid + 1) * L + j];
+                    emit((vb >> 1) + tid, gs * NSLM_R32, us * NSLM_R32);
+                }
+            } else if (tid < nrow) {
+                float s = 0.0f;
+                for (int j = 0; j < L; ++j) s += part[par][tid * L + j];
+                emit(vb + tid, s * NSLM_R32, 0.0f);
+            }
+        }
+        cur = nxt;
+    }
+    if (!SHFL) __syncthreads();   // part may be reused by the next pass
+}
+
+// n floats of a row staged chunk-padded into LDS by the whole workgroup; coherent: agent-scope loads (the row was
+// written by other workgroups of this launch)
+__device__ __forceinline__ void stage_row(const float* src, int n, float* xl, bool coherent) {
+    for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = coherent ? ld_agent(src + i) : src[i];
+}
+
+template <int P, bool SHFL_G, bool SHFL_D>
+__global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
+    extern __shared__ float xl[];   // activations of the current pair: max(d, ff) floats, chunk-padded
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    __shared__ float part[2][256];
+    __shared__ __attribute__((aligned(16))) float rv[1024];   // route: the token's logits
+    __shared__ float rw_s[32];      // route: weight by rank
+    __shared__ int ri_s[32];        // route: expert by rank
+    __shared__ WSlice sl_s[3][32];  // route: the chosen experts' gate / up / down slices
+    __shared__ int s_flag;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const uint32_t G = (uint32_t) a.grid;
+    const int P_ = a.T * a.k;
+    // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
+    unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
+#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
+    STAMP(0);
+    load_tables(tab);
+    const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
+    int staged = -1;
+
+    // ---- phase 1: router logits, one wave per (token, expert): k_mv_any's BF16 row dot and BF16 store ----------------
+    for (int item = (int) blockIdx.x * 4 + wv; item < a.T * a.E; item += (int) G * 4) {
+        const int t = item / a.E, e = item - t * a.E;
+        const uint16_t* wr = a.rw + (size_t) e * a.d;
+        const float* xr = a.x + (size_t) t * a.xs;
+        float acc = 0.0f;
+        for (int j = lane; j < a.d / 8; j += 64) {
+            const uint4 q = *(const uint4*) (wr + (size_t) j * 8);
+            const float4 x0 = *(const float4*) (xr + (size_t) j * 8), x1 = *(const float4*) (xr + (size_t) j * 8 + 4);
+            float dd = bf(q.x & 0xFFFFu) * x0.x;
+            dd = fmaf(bf(q.x >> 16), x0.y, dd);
+            dd = fmaf(bf(q.y & 0xFFFFu), x0.z, dd);
+            dd = fmaf(bf(q.y >> 16), x0.w, dd);
+            dd = fmaf(bf(q.z & 0xFFFFu), x1.x, dd);
+            dd = fmaf(bf(q.z >> 16), x1.y, dd);
+            dd = fmaf(bf(q.w & 0xFFFFu), x1.z, dd);
+            dd = fmaf(bf(q.w >> 16), x1.w, dd);
+            acc = fmaf(dd, 1.0f, acc);
+        }
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+        if (lane == 0) st_agent(a.logits + item, bfr(acc));
+    }
+    // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
+    if ((int) blockIdx.x < items_g) {
+        staged = ((int) blockIdx.x / a.ntile_g) / a.k;
+        stage_row(a.x + (size_t) staged * a.xs, a.d, xl, false);
+    }
+    STAMP(1);
+    grid_barrier(a.sync, G);
+    STAMP(2);
+
+    // ---- route: every workgroup ranks the logits of the token it needs (cheap, and saves a grid barrier) ----------------
+    // rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order
+    int routed = -1;
+    auto route = [&](int t) {
+        if (routed == t) return;
+        routed = t;
+        __syncthreads();
+        const int E4 = (a.E + 3) & ~3;
+        for (int e = tid; e < E4; e += 256) rv[e] = e < a.E ? ld_agent(a.logits + (size_t) t * a.E + e) : __uint_as_float(0xFF800000u);
+        __syncthreads();
+        for (int e = tid; e < a.E; e += 256) {
+            const float v = rv[e];
+            int rank = 0;
+#pragma unroll 8
+            for (int o = 0; o < E4; o += 4) {
+                const float4 u = *(const float4*) &rv[o];
+                rank += (u.x > v || (u.x == v && o > e)) ? 1 : 0;
+                rank += (u.y > v || (u.y == v && o + 1 > e)) ? 1 : 0;
+                rank += (u.z > v || (u.z == v && o + 2 > e)) ? 1 : 0;
+                rank += (u.w > v || (u.w == v && o + 3 > e)) ? 1 : 0;
+            }
+            if (rank < a.k) ri_s[rank] = e;
+        }
+        __syncthreads();
+        if (tid < 3 * a.k) {   // the chosen experts' slices, fetched side by side
+            const int which = tid / a.k, j = tid - which * a.k;
+            sl_s[which][j] = (which == 0 ? a.gate : which == 1 ? a.up : a.down)[ri_s[j]];
+        }
+        if (tid < a.k) rw_s[tid] = expf(rv[ri_s[tid]] - rv[ri_s[0]]);
+        __syncthreads();
+        if (tid < a.k) {
+            float top = 0.0f;
+            for (int r = 0; r < a.k; ++r) top += rw_s[r];
+            rw_s[tid] = rw_s[tid] / top;   // every lane has read all k values before any lane writes: one wave, in order
+        }
+        __syncthreads();
+        if (blockIdx.x == (unsigned) t % G && tid < a.k) {   // one writer per token publishes the routing
+            a.ind[(size_t) t * a.k + tid] = ri_s[tid];
+            a.wt[(size_t) t * a.k + tid] = rw_s[tid];
+        }
+    };
+
+    // ---- phase 2: gate + up + SwiGLU, items (pair, row tile) -------------------------------------------------------------
+    for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
+        const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.k, j = p - t * a.k;
+        route(t);
+        const int v0 = tile * a.rows_g, v1 = min(v0 + a.rows_g, 2 * a.ff);
+        const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
+        if (staged != t) {
+            __syncthreads();
+            stage_row(a.x + (size_t) t * a.xs, a.d, xl, false);
+            staged = t;
+            __syncthreads();
+        }
+        float* Ap = a.A + (size_t) p * a.ff;
+        rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
+                                   [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
+    }
+    // tokens whose routing nobody needed here still get published by their designated workgroup
+    for (int t = (int) blockIdx.x; t < a.T; t += (int) G) route(t);
+    STAMP(3);
+
+    // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
+    // the first down item's records do not depend on phase 2: they are fetched before the barrier
+    uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
+    Chunk d0;
+    if ((int) blockIdx.x < items_d) {
+        const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.k, j = p - t * a.k;
+        route(t);
+        d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.rows_d, min(tile * a.rows_d + a.rows_d, a.d));
+    }
+    grid_barrier(a.sync, G);
+    STAMP(4);
+    for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
+        const int p = item / a.ntile_d, tile = item - p * a.ntile_d, t = p / a.k, j = p - t * a.k;
+        route(t);
+        const int v0 = tile * a.rows_d, v1 = min(v0 + a.rows_d, a.d);
+        if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
+        __syncthreads();
+        stage_row(a.A + (size_t) p * a.ff, a.ff, xl, true);
+        staged = -1;
+        __syncthreads();
+        float* Dp = a.D + (size_t) p * a.d;
+        rows_pass<P, false, SHFL_D>(d0, sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1, tab, xl, part,
+                                    [&](int r, float s, float) { st_agent(Dp + r, bfr(s)); });
+        wg_release();
+        __syncthreads();
+        if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.k - 1);
+        __syncthreads();
+        if (s_flag) {   // all k experts' rows of this tile are written: out = 0.5 * 0 + sum_j wt_j D_j, in j order
+            wg_acquire();
+            for (int r = v0 + tid; r < v1; r += 256) {
+                float acc = 0.0f;
+                for (int jj = 0; jj < a.k; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.k + jj) * a.d + r), acc);
+                a.out[(size_t) t * a.os + r] = acc;
+            }
+            if (tid == 0) st_agent(&tick[t * a.ntile_d + tile], 0u);
+        }
+    }
+    STAMP(5);
+#undef STAMP
+}
+
+int cu_count() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        hipDeviceProp_t pr;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) n = pr.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+bool shape_of(int K, bool gateup, int* L, int* rpi, bool* shfl) {
+    if (K % 64 || K / 64 > 128) return false;
+    const int l = K / 64;
+    int r = 256 / l;
+    if (gateup) r &= ~1;
+    if (r < 1) return false;
+    *L = l;
+    *rpi = r;
+    *shfl = (l & (l - 1)) == 0 && l <= (gateup ? 32 : 64);
+    return true;
+}
+
+template <int P>
+int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
+    void (*kern)(FusedArgs) = sg ? (sd ? k_moe_decode<P, true, true> : k_moe_decode<P, true, false>)
+                                 : (sd ? k_moe_decode<P, false, true> : k_moe_decode<P, false, false>);
+    static int cached[2][2] = {{0, 0}, {0, 0}};   // resident workgroups per CU, by kernel variant (same LDS request every call)
+    int& per_cu = cached[sg][sd];
+    if (!per_cu && (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds) != hipSuccess || per_cu < 1)) {
+        per_cu = 0;
+        return -1;
+    }
+    // the grid must be resident at once: all the device holds, but no more than the work can use
+    int grid = (per_cu < 3 ? per_cu : 3) * cu_count();
+    static const char* env = getenv("NSLM_FUSED_WGS_PER_CU");
+    if (env && atoi(env) > 0 && atoi(env) <= per_cu) grid = atoi(env) * cu_count();
+    const int items = a.T * a.k * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
+    if (grid > items) grid = items;
+    if (grid < 1) grid = 1;
+    a.grid = grid;
+    hipLaunchKernelGGL(kern, dim3((unsigned) grid), dim3(256), lds, st, a);
+    host_note_launch();
+    return 0;
+}
+
+}   // namespace
+
+extern "C" {
+
+size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1); }
+int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
+
+int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
+                  int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
+                  int32_t* ind, float* wt, float* A, float* D, uint32_t* sync) {
+    if (T < 1 || T > MV_MAXT || top_k < 1 || top_k > 32 || n_exp > 1024 || n_exp < top_k) return -1;
+    if (fmt != MF_SEED4P4 && fmt != MF_SEED4) return -1;
+    if (host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u)) return -1;
+    FusedArgs a = {};
+    bool sg, sd;
+    if (!shape_of(d, true, &a.Lg, &a.rpig, &sg) || !shape_of(ff, false, &a.Ld, &a.rpid, &sd)) return -1;
+    a.rw = router_w; a.gate = gate; a.up = up; a.down = down; a.x = x; a.out = out; a.logits = logits; a.wt = wt; a.A = A;
+    a.D = D; a.ind = ind; a.sync = sync; a.E = n_exp; a.k = top_k; a.d = d; a.ff = ff; a.T = T; a.xs = xs; a.os = os;
+    // iterations per item: as many as keep every workgroup of a full grid busy in that phase, at most 4
+    const int full = 3 * cu_count(), P_ = T * top_k;
+    const int it_g = (2 * ff + a.rpig - 1) / a.rpig, it_d = (d + a.rpid - 1) / a.rpid;
+    int per_g = P_ * it_g / full, per_d = P_ * it_d / full;
+    per_g = per_g < 1 ? 1 : per_g > 4 ? 4 : per_g;
+    per_d = per_d < 1 ? 1 : per_d > 4 ? 4 : per_d;
+    a.rows_g = per_g * a.rpig;
+    a.ntile_g = (2 * ff + a.rows_g - 1) / a.rows_g;
+    a.rows_d = per_d * a.rpid;
+    a.ntile_d = (d + a.rows_d - 1) / a.rows_d;
+    const int kmax = d > ff ? d : ff;
+    size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
+    static const char* pad = getenv("NSLM_FUSED_LDS");   // experiment: request this much LDS to cap workgroups per CU
+    if (pad && (size_t) atoi(pad) > lds) lds = (size_t) atoi(pad);
+    return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
+}
+
+}   // extern "C"

@@ -141,7 +141,7 @@ __global__ void k_q4_moe_combine(int d, int k, const float* D, const float* wt, 
     const int i = (int) (blockIdx.x * blockDim.x + threadIdx.x), t = (int) blockIdx.y;
     if (i >= d) return;
     float acc = (1.0f / (1.0f + expf(-sg[(size_t) t * sgld]))) * sh[(size_t) t * d + i];
-    for (int j = 0; j < k; ++j) acc += wt[t * k + j] * D[((size_t) t * k + j) * d + i];
+    for (int j = 0; j < k; ++j) acc = fmaf(wt[t * k + j], D[((size_t) t * k + j) * d + i], acc);
     out[(size_t) t * d + i] = acc;
 }
 __global__ void k_pack_input_bf16(const float* x, uint16_t* y, size_t n) {

@@ -16,7 +16,7 @@
 // Generic path (k_mv_any): one wave per row, lanes over blocks; every format, any K % 8 == 0, any alignment.
 #include <stdlib.h>
 
-#include "nslm_dev.h"
+#include "nslm_mv_dev.h"
 
 using namespace nslm;
 
@@ -37,81 +37,6 @@ struct MvArgs {
 };
 
 enum { DENSE = 0, GATHER = 1, GATEUP = 2 };
-
-struct Chunk {
-    uint4 sd, cw;
-    uint32_t codes;
-};
-
-// al: the slice's streams are 16-byte (codes: 4-byte) aligned; otherwise the same records by 2-byte and 1-byte loads
-template <int P>
-__device__ __forceinline__ Chunk load_chunk(const WSlice& w, uint32_t unit, bool ok, bool al) {
-    Chunk c;
-    c.sd = make_uint4(0, 0, 0, 0);
-    c.cw = c.sd;
-    c.codes = 0;
-    if (!ok) return c;
-    if (al) {
-        c.sd = ((const uint4*) w.p[0])[unit];
-        c.cw = ((const uint4*) w.p[1])[unit];
-        if (P == 4) c.codes = ((const uint32_t*) w.p[3])[unit];
-    } else {
-        const uint16_t* sp = (const uint16_t*) w.p[0] + (size_t) unit * 8;
-        const uint16_t* cp = (const uint16_t*) w.p[1] + (size_t) unit * 8;
-        c.sd = make_uint4(sp[0] | (uint32_t) sp[1] << 16, sp[2] | (uint32_t) sp[3] << 16, sp[4] | (uint32_t) sp[5] << 16,
-                          sp[6] | (uint32_t) sp[7] << 16);
-        c.cw = make_uint4(cp[0] | (uint32_t) cp[1] << 16, cp[2] | (uint32_t) cp[3] << 16, cp[4] | (uint32_t) cp[5] << 16,
-                          cp[6] | (uint32_t) cp[7] << 16);
-        if (P == 4) {
-            const uint8_t* ep = (const uint8_t*) w.p[3] + (size_t) unit * 4;
-            c.codes = ep[0] | (uint32_t) ep[1] << 8 | (uint32_t) ep[2] << 16 | (uint32_t) ep[3] << 24;
-        }
-    }
-    return c;
-}
-__device__ __forceinline__ bool streams_aligned(int P, const WSlice& w) {
-    return (((uintptr_t) w.p[0] | (uintptr_t) w.p[1]) & 15u) == 0 && (P != 4 || ((uintptr_t) w.p[3] & 3u) == 0);
-}
-
-__device__ __forceinline__ uint32_t word_of(const uint4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
-
-// One chunk (8 blocks) against NT tokens.  xr: this chunk's activations, token t at xr + t * xstride (registers when
-// NT == 1, LDS otherwise).  acc[t] accumulates 2^(e+0) * sum_c isum_c x_c per block (R32 is applied to the row sum).
-template <int P, int NT>
-__device__ __forceinline__ void chunk_dot(const Chunk& ck, int eb, const uint32_t* tab, const float* xr, int xstride, int nt,
-                                          float (&acc)[NT]) {
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
-        const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
-        const uint32_t seed16 = (b & 1) ? ss >> 16 : ss & 0xFFFFu, word16 = (b & 1) ? cc >> 16 : cc & 0xFFFFu;
-        const uint32_t g = stream_of(tab, seed16);
-        const uint32_t up = (b & 1) ? ss : ss << 16;   // only the upper 16 bits are read
-        int is[8];
-        int code;
-        if (P == 4) {
-            isum_p4(up, g, tab[512 + (word16 & 0xFFu)], tab[512 + (word16 >> 8)], is);
-            code = (int) ((ck.codes >> (4 * b)) & 15u);
-        } else {
-            isum_p3(up, g, tab[512 + ((word16 >> 4) & 0xFFu)], tab[512 + (word16 >> 12)], is);
-            code = (int) (word16 & 15u);
-        }
-        const float e2 = pow2f(eb + code);
-        float w[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) w[c] = (float) is[c];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (NT > 1 && t >= nt) break;
-            const float* xb = xr + t * xstride + 8 * b;
-            float d = w[0] * xb[0];
-#pragma unroll
-            for (int c = 1; c < 8; ++c) d = fmaf(w[c], xb[c], d);
-            acc[t] = fmaf(d, e2, acc[t]);
-        }
-    }
-}
-
-#define XPAD 68   // LDS floats per 64-float chunk: 16-byte reads of 8 consecutive lanes land on 32 distinct banks
 
 // SHFL: L is a power of two <= 64 (<= 32 for GATEUP): row sums by wave shuffles, no barrier.  Otherwise through LDS.
 template <int P, int MODE, int NT, bool SHFL>
@@ -222,45 +147,6 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
 }
 
 // ---- generic path: every format, one wave per row --------------------------------------------------------------------
-// The 8 weights of block j of row r as f32: seeds unscaled integers with *sc = 2^e R32; BF16 / Q8 as BF16 values; Q4 in
-// MLX's matvec form s * q + b unrounded (reference engine/kernels_moe.cu:91-107, 171-189).
-__device__ __forceinline__ void block_weights(int fmt, const WSlice& w, const uint32_t* tab, int r, int K, int j, float (&o)[8],
-                                              float* sc) {
-    const int nbk = K / 8;
-    *sc = 1.0f;
-    if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
-        const size_t g = (size_t) r * nbk + j;
-        const uint32_t seed = ((const uint16_t*) w.p[0])[g], word = ((const uint16_t*) w.p[1])[g];
-        int is[8], code;
-        if (fmt == MF_SEED4P4) {
-            block_isum<4>(tab, seed, word, is);
-            code = (((const uint8_t*) w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
-        } else {
-            block_isum<3>(tab, seed, word, is);
-            code = (int) (word & 15u);
-        }
-#pragma unroll
-        for (int c = 0; c < 8; ++c) o[c] = (float) is[c];
-        *sc = pow2f(w.eb + code) * NSLM_R32;
-    } else if (fmt == MF_BF16) {
-        const uint16_t* v = (const uint16_t*) w.p[0] + (size_t) r * K + (size_t) j * 8;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) o[c] = bf(v[c]);
-    } else {
-        const size_t e0 = (size_t) r * K + (size_t) j * 8, gi = e0 >> group_shift(w);
-        const float s = bf(((const uint16_t*) w.p[1])[gi]), b = bf(((const uint16_t*) w.p[2])[gi]);
-        if (fmt == MF_Q8) {
-            const uint32_t* q = (const uint32_t*) w.p[0] + e0 / 4;
-#pragma unroll
-            for (int c = 0; c < 8; ++c) o[c] = bfr(s * (float) ((q[c >> 2] >> (8 * (c & 3))) & 255u) + b);
-        } else {
-            const uint32_t q = ((const uint32_t*) w.p[0])[e0 / 8];
-#pragma unroll
-            for (int c = 0; c < 8; ++c) o[c] = s * (float) ((q >> (4 * c)) & 15u) + b;
-        }
-    }
-}
-
 template <int MODE>
 __global__ void __launch_bounds__(256) k_mv_any(int fmt, MvArgs a) {
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
@@ -375,6 +261,8 @@ void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t l
 }
 template <int MODE, int NT>
 void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds) {
+    static const char* pad = getenv("NSLM_MV_LDS");   // experiment: request this much LDS to cap workgroups per CU
+    if (pad && (size_t) atoi(pad) > lds) lds = (size_t) atoi(pad);
     if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds);
     else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds);
 }

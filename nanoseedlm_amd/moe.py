@@ -129,6 +129,12 @@ class MoeStack:
             raise RuntimeError("nslm_moe_cache_stats failed")
         return h.value, m.value
 
+    def set_fused(self, on):
+        self.L.nslm_moe_set_fused(self.h, int(on))
+
+    def fused_error(self):
+        return self.L.nslm_moe_fused_error(self.h)
+
     def expert_bytes(self):
         return int(self.L.nslm_moe_expert_bytes(self.h))
 
