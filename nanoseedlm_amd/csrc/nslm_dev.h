@@ -13,6 +13,27 @@
 
 namespace nslm {
 
+// ---- global-memory pointers ---------------------------------------------------------------------------------------------
+// Stream pointers arrive inside structs (WSlice), where the compiler cannot tell that they address global memory and would
+// emit flat loads.  A flat load also counts against the LDS counter, so every LDS wait - and every barrier built on one -
+// would wait for the HBM latency of loads issued steps ahead on purpose.  gp<T>(p) states the address space.
+#define NSLM_GLOBAL __attribute__((address_space(1)))
+template <typename T>
+__device__ __forceinline__ const NSLM_GLOBAL T* gp(const void* p) { return (const NSLM_GLOBAL T*) p; }
+// 16- and 8-byte global loads (uint4 / uint2 are class types and cannot be read through a qualified pointer directly)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <typename P>
+__device__ __forceinline__ uint4 ldg16(P p) {
+    const u32x4 v = *(const NSLM_GLOBAL u32x4*) p;
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+template <typename P>
+__device__ __forceinline__ uint2 ldg8(P p) {
+    const u32x2 v = *(const NSLM_GLOBAL u32x2*) p;
+    return make_uint2(v.x, v.y);
+}
+
 // ---- BF16 (round to nearest even; reference engine/kernels_moe.cu:17-31) ---------------------------------------------
 __device__ __forceinline__ float bfr(float x) {
     uint32_t u = __float_as_uint(x);
@@ -87,9 +108,12 @@ __device__ __forceinline__ uint32_t stream_of(const uint32_t* tab, uint32_t seed
 }
 
 // ---- exact block decode -----------------------------------------------------------------------------------------------
-typedef short short2v __attribute__((ext_vector_type(2)));
+// Written as the three-source encoding: left to itself the compiler prefers the accumulating two-source form, whose
+// destination is tied to the addend, and pays a register move whenever the addend has another use or a different home.
 __device__ __forceinline__ int dot2(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot2(__builtin_bit_cast(short2v, a), __builtin_bit_cast(short2v, b), c, false);
+    int d;
+    asm("v_dot2_i32_i16 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
 }
 // the same with a zero addend: the three-source encoding takes the constant inline, where the accumulating two-source
 // form the compiler picks for dot2(a, b, 0) would first spend a move on zeroing its destination
@@ -136,6 +160,79 @@ __device__ __forceinline__ void isum_p3(uint32_t up, uint32_t g, uint32_t q01, u
         const int third = k2 <= 16 ? dot2z(A[k2], q2) : dot2z(A[k2 - 16], q2hi);
         is[c] = dot2(pr, q01, third);
     }
+}
+
+// Two blocks at once, written in phases (all windows, then all sign flips, all pairings, all products) with the
+// scheduler held to that order: a VALU result is not available to the next instruction slots, and a wave that has a SIMD's
+// vector issue to itself (the GEMM's decoder waves) loses those slots unless dependent instructions sit far apart.  In
+// phase order every operand is at least a dozen instructions old.
+__device__ __forceinline__ void isum2_p4(const uint32_t (&up)[2], const uint32_t (&g)[2], const uint32_t (&q01)[2],
+                                         const uint32_t (&q23)[2], int (&is)[2][8]) {
+    uint32_t A[2][17], lo[2][8], hi[2][8];
+#pragma unroll
+    for (int k = 1; k <= 15; ++k)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) A[h][k] = __builtin_amdgcn_alignbit(g[h], up[h], 16 + k);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k = 1; k <= 16; ++k)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) A[h][k] = (k < 16 ? A[h][k] : g[h]) ^ 0x80008000u;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)   // pair j = states 2j+1, 2j+2 (low halves) and 2j+17, 2j+18 (high halves)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            lo[h][j] = halves(A[h][2 * j + 1], 0, A[h][2 * j + 2], 0);
+            hi[h][j] = halves(A[h][2 * j + 1], 1, A[h][2 * j + 2], 1);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+    int t[2][8];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            t[h][c] = dot2z(lo[h][2 * c + 1], q23[h]);
+            t[h][c + 4] = dot2z(hi[h][2 * c + 1], q23[h]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            is[h][c] = dot2(lo[h][2 * c], q01[h], t[h][c]);
+            is[h][c + 4] = dot2(hi[h][2 * c], q01[h], t[h][c + 4]);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+}
+__device__ __forceinline__ void isum2_p3(const uint32_t (&up)[2], const uint32_t (&g)[2], const uint32_t (&q01)[2],
+                                         const uint32_t (&q2)[2], int (&is)[2][8]) {
+    uint32_t A[2][17], pr[2][8];
+#pragma unroll
+    for (int k = 1; k <= 15; ++k)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) A[h][k] = __builtin_amdgcn_alignbit(g[h], up[h], 16 + k);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int k = 1; k <= 16; ++k)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) A[h][k] = (k < 16 ? A[h][k] : g[h]) ^ 0x80008000u;
+    __builtin_amdgcn_sched_barrier(0);
+    int t[2][8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k0 = 3 * c + 1, k1 = k0 + 1, k2 = k0 + 2;   // state k lives in A[k] low (k <= 16) or A[k-16] high
+            pr[h][c] = halves(A[h][k0 <= 16 ? k0 : k0 - 16], k0 > 16, A[h][k1 <= 16 ? k1 : k1 - 16], k1 > 16);
+            t[h][c] = k2 <= 16 ? dot2z(A[h][k2], q2[h]) : dot2z(A[h][k2 - 16], q2[h] << 16);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) is[h][c] = dot2(pr[h][c], q01[h], t[h][c]);
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // One block of either seed format from its raw fields.  seed16 / word16: the 16-bit seed and coefficient (P = 4) or

@@ -307,12 +307,12 @@ __global__ void __launch_bounds__(256) k_deq(int fmt, WSlice W, int rows_per_hea
     const int nbk = K / 8, row = b / nbk;
     float o[8];
     if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
-        const uint32_t seed = ((const uint16_t*) W.p[0])[b], word = ((const uint16_t*) W.p[1])[b];
-        const int eb = heads ? ((const int32_t*) W.p[2])[row / rows_per_head] : W.eb;
+        const uint32_t seed = gp<uint16_t>(W.p[0])[b], word = gp<uint16_t>(W.p[1])[b];
+        const int eb = heads ? gp<int32_t>(W.p[2])[row / rows_per_head] : W.eb;
         int is[8], code;
         if (fmt == MF_SEED4P4) {
             block_isum<4>(tab, seed, word, is);
-            code = (((const uint8_t*) W.p[3])[b >> 1] >> ((b & 1) * 4)) & 15;
+            code = (gp<uint8_t>(W.p[3])[b >> 1] >> ((b & 1) * 4)) & 15;
         } else {
             block_isum<3>(tab, seed, word, is);
             code = (int) (word & 15u);
@@ -322,14 +322,14 @@ __global__ void __launch_bounds__(256) k_deq(int fmt, WSlice W, int rows_per_hea
         for (int c = 0; c < 8; ++c) o[c] = (float) is[c] * sc;
     } else if (fmt == MF_BF16) {
 #pragma unroll
-        for (int c = 0; c < 8; ++c) o[c] = bf(((const uint16_t*) W.p[0])[(size_t) b * 8 + c]);
+        for (int c = 0; c < 8; ++c) o[c] = bf(gp<uint16_t>(W.p[0])[(size_t) b * 8 + c]);
     } else {
         const size_t e0 = (size_t) b * 8, gi = e0 >> group_shift(W);
-        const float s = bf(((const uint16_t*) W.p[1])[gi]), bb = bf(((const uint16_t*) W.p[2])[gi]);
+        const float s = bf(gp<uint16_t>(W.p[1])[gi]), bb = bf(gp<uint16_t>(W.p[2])[gi]);
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-            const uint32_t q = fmt == MF_Q8 ? (((const uint32_t*) W.p[0])[e0 / 4 + (c >> 2)] >> (8 * (c & 3))) & 255u
-                                            : (((const uint32_t*) W.p[0])[e0 / 8] >> (4 * c)) & 15u;
+            const uint32_t q = fmt == MF_Q8 ? (gp<uint32_t>(W.p[0])[e0 / 4 + (c >> 2)] >> (8 * (c & 3))) & 255u
+                                            : (gp<uint32_t>(W.p[0])[e0 / 8] >> (4 * c)) & 15u;
             o[c] = s * (float) q + bb;
         }
     }

@@ -10,7 +10,11 @@
 // accumulator columns are consecutive output addresses).  f32 accumulation.  In exact mode (kc_seed_gemm_f32) a seed
 // weight is carried as three BF16 terms hi + mid + lo whose sum is the f32 value, three MFMAs per step, as the reference.
 // Other formats (BF16, Q8, Q4) dequantize to BF16 values exactly and take the same path.
-#include "nslm_dev.h"
+#include <stdlib.h>
+
+#include <type_traits>
+
+#include "nslm_mv_dev.h"
 
 using namespace nslm;
 
@@ -25,6 +29,10 @@ struct MmArgs {
     int K, R, T, xs, ys, xdiv, add, f32out;
 };
 
+// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load of the
+// wave, which would serialise the producers' prefetches (issued steps ahead on purpose) with each step.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 #define BM 64           // weight rows per workgroup
 #define BK 32           // K per step
 #define LDW 40          // LDS row stride in BF16 elements (80 bytes: 16-byte fragment reads are conflict-free)
@@ -34,11 +42,11 @@ __device__ __forceinline__ void tile_block(int fmt, const WSlice& w, const uint3
     const int nbk = K / 8;
     if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
         const size_t g = (size_t) r * nbk + j;
-        const uint32_t seed = ((const uint16_t*) w.p[0])[g], word = ((const uint16_t*) w.p[1])[g];
+        const uint32_t seed = gp<uint16_t>(w.p[0])[g], word = gp<uint16_t>(w.p[1])[g];
         int is[8], code;
         if (fmt == MF_SEED4P4) {
             block_isum<4>(tab, seed, word, is);
-            code = (((const uint8_t*) w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
+            code = (gp<uint8_t>(w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
         } else {
             block_isum<3>(tab, seed, word, is);
             code = (int) (word & 15u);
@@ -47,38 +55,59 @@ __device__ __forceinline__ void tile_block(int fmt, const WSlice& w, const uint3
 #pragma unroll
         for (int c = 0; c < 8; ++c) o[c] = (float) is[c] * sc;
     } else if (fmt == MF_BF16) {
-        const uint4 v = *(const uint4*) ((const uint16_t*) w.p[0] + (size_t) r * K + (size_t) j * 8);
+        const uint4 v = ldg16(gp<uint16_t>(w.p[0]) + (size_t) r * K + (size_t) j * 8);
         const uint32_t u[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(u[i] << 16); o[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u); }
     } else {
         const size_t e0 = (size_t) r * K + (size_t) j * 8, gi = e0 >> group_shift(w);
-        const float s = bf(((const uint16_t*) w.p[1])[gi]), b = bf(((const uint16_t*) w.p[2])[gi]);
+        const float s = bf(gp<uint16_t>(w.p[1])[gi]), b = bf(gp<uint16_t>(w.p[2])[gi]);
         if (fmt == MF_Q8) {
-            const uint2 q = *(const uint2*) ((const uint32_t*) w.p[0] + e0 / 4);
+            const uint2 q = ldg8(gp<uint32_t>(w.p[0]) + e0 / 4);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 o[i] = bfr(s * (float) ((q.x >> (8 * i)) & 255u) + b);
                 o[4 + i] = bfr(s * (float) ((q.y >> (8 * i)) & 255u) + b);
             }
         } else {
-            const uint32_t q = ((const uint32_t*) w.p[0])[e0 / 8];
+            const uint32_t q = gp<uint32_t>(w.p[0])[e0 / 8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = bfr(s * (float) ((q >> (4 * i)) & 15u) + b);
         }
     }
 }
 
-// MT: 32-token tiles per wave (the workgroup covers 128 * MT tokens or pairs).  NTERM: BF16 terms per weight.
+// MT: 32-token tiles per consumer wave (the workgroup covers 128 * MT tokens or pairs).  NTERM: BF16 terms per weight.
+//
+// 512 threads: waves 0-3 are consumers (MFMA only: wave w owns tokens [32 MT w, 32 MT (w+1)) x all 64 rows), waves 4-7
+// are producers (each thread decodes one 8-weight block per K step and stages its share of the step's activations).
+// The two LDS buffers alternate per step with one workgroup barrier between steps; producers hold the global loads of
+// the two following steps in registers, so a step's records and activations are requested three steps before the MFMAs
+// read them and the matrix cores never wait on HBM or L2 latency.
+struct MmRec {
+    uint32_t seed, word, code;   // seeds: the block's raw fields
+    uint4 raw[2];                // other formats: the block's packed words, scale and bias
+};
+template <int MT, bool PACKED>
+struct MmX {
+    uint4 v[PACKED ? 2 * MT : 4 * MT];   // this thread's share of a step: MT x 16 activations (BF16, or f32 before rounding)
+};
+
 template <int MT, int NTERM, bool PACKED>
-__global__ void __launch_bounds__(256) k_mm(int fmt, MmArgs a, WSlice wd, const WSlice* ws, const void* Xv, float* Y,
+__global__ void __launch_bounds__(512) k_mm(int fmt, MmArgs a, WSlice wd, const WSlice* ws, const void* Xv, float* Y,
                                             const int32_t* perm, const MmTile* tiles, const int32_t* ntiles) {
     constexpr int BN = 128 * MT;
-    __shared__ __attribute__((aligned(16))) uint16_t Wsm[NTERM][BM][LDW];
-    __shared__ __attribute__((aligned(16))) uint16_t Xsm[BN][LDW];
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    typedef uint16_t WTile[NTERM][BM][LDW];
+    typedef uint16_t XTile[BN][LDW];
+    WTile* Wsm = (WTile*) smem;                               // [2]
+    XTile* Xsm = (XTile*) (smem + 2 * NTERM * BM * LDW);      // [2]
     __shared__ int srow[BN], drow[BN];
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    __shared__ __attribute__((aligned(16))) uint16_t rec_seed[2][BM][32], rec_word[2][BM][32];   // two super-steps of records
+    __shared__ uint32_t rec_code[2][BM][4];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const bool producer = wv >= 4;
     const bool grouped = tiles != nullptr;
     if (grouped && ntiles && (int) blockIdx.y >= *ntiles) return;
     const int r0 = (int) blockIdx.x * BM;
@@ -95,13 +124,181 @@ __global__ void __launch_bounds__(256) k_mm(int fmt, MmArgs a, WSlice wd, const 
         count = min(BN, a.T - start);
     }
     load_tables(tab);
-    for (int i = tid; i < BN; i += 256) {
+    for (int i = tid; i < BN; i += 512) {
         const bool ok = i < count;
         srow[i] = !ok ? -1 : grouped ? perm[start + i] / a.xdiv : start + i;
         drow[i] = !ok ? -1 : grouped ? perm[start + i] : start + i;
     }
     __syncthreads();
+    const int nsteps = a.K / BK;
 
+    // ---- producer side ---------------------------------------------------------------------------------------------------
+    const int ptid = tid - 256, rr = ptid >> 2, jb = ptid & 3, row = r0 + rr, nbk = a.K / 8;
+    const bool seedf = fmt == MF_SEED4P4 || fmt == MF_SEED4;
+    // Seed records reach the decoder through LDS, one "super-step" of 8 K steps (32 blocks a row) at a time: thread
+    // (rr, jb) fetches blocks [8 jb, 8 jb + 8) of the super-step with one 16-byte load of seeds, one of coefficient words
+    // and a dword of codes, a whole super-step (microseconds) before they are decoded - the records stream from HBM
+    // exactly once and nothing downstream may wait on that latency.
+    const bool rec_fast = seedf && nbk % 8 == 0 && streams_aligned(fmt == MF_SEED4P4 ? 4 : 3, wt);
+    auto load_super = [&](int S) {
+        Chunk c;
+        c.sd = c.cw = make_uint4(0, 0, 0, 0);
+        c.codes = 0;
+        const int b0 = 32 * S + 8 * jb;   // first block of this thread's share
+        if (!seedf || row >= a.R || b0 >= nbk) return c;
+        const size_t g = (size_t) row * nbk + b0;
+        if (rec_fast) {
+            c.sd = ldg16(gp<uint16_t>(wt.p[0]) + g);
+            c.cw = ldg16(gp<uint16_t>(wt.p[1]) + g);
+            if (fmt == MF_SEED4P4) c.codes = *(const NSLM_GLOBAL uint32_t*) (gp<uint8_t>(wt.p[3]) + (g >> 1));
+        } else {
+            uint32_t sd[8], cw[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool ok = b0 + i < nbk;
+                sd[i] = ok ? gp<uint16_t>(wt.p[0])[g + i] : 0u;
+                cw[i] = ok ? gp<uint16_t>(wt.p[1])[g + i] : 0u;
+                if (ok && fmt == MF_SEED4P4) c.codes |= ((uint32_t) (gp<uint8_t>(wt.p[3])[(g + i) >> 1] >> (((g + i) & 1) * 4)) & 15u) << (4 * i);
+            }
+            c.sd = make_uint4(sd[0] | sd[1] << 16, sd[2] | sd[3] << 16, sd[4] | sd[5] << 16, sd[6] | sd[7] << 16);
+            c.cw = make_uint4(cw[0] | cw[1] << 16, cw[2] | cw[3] << 16, cw[4] | cw[5] << 16, cw[6] | cw[7] << 16);
+        }
+        return c;
+    };
+    auto store_super = [&](int buf, const Chunk& c) {
+        if (!seedf) return;
+        *(uint4*) &rec_seed[buf][rr][8 * jb] = c.sd;
+        *(uint4*) &rec_word[buf][rr][8 * jb] = c.cw;
+        rec_code[buf][rr][jb] = c.codes;
+    };
+    // other formats: this thread's block of step s straight into registers
+    auto load_rec = [&](int s, MmRec& r) {
+        if (seedf || s >= nsteps || row >= a.R) return;
+        const size_t g = (size_t) row * nbk + s * (BK / 8) + jb;
+        if (fmt == MF_BF16) {
+            r.raw[0] = ldg16(gp<uint16_t>(wt.p[0]) + g * 8);
+        } else {
+            const size_t gi = (g * 8) >> group_shift(wt);
+            r.seed = gp<uint16_t>(wt.p[1])[gi];
+            r.word = gp<uint16_t>(wt.p[2])[gi];
+            if (fmt == MF_Q8) r.raw[0] = make_uint4(gp<uint32_t>(wt.p[0])[g * 2], gp<uint32_t>(wt.p[0])[g * 2 + 1], 0, 0);
+            else r.raw[0] = make_uint4(gp<uint32_t>(wt.p[0])[g], 0, 0, 0);
+        }
+    };
+    auto load_x = [&](int s, MmX<MT, PACKED>& x) {
+        if (s >= nsteps) return;
+        const int k0 = s * BK;
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+            const int i = ptid + 256 * u, n = i >> 1, h = (i & 1) * 16, src = srow[n];
+            if (PACKED) {
+                x.v[2 * u] = x.v[2 * u + 1] = make_uint4(0, 0, 0, 0);
+                if (src >= 0) {
+                    const uint4* xr = (const uint4*) ((const uint16_t*) Xv + (size_t) src * a.xs + k0 + h);
+                    x.v[2 * u] = xr[0];
+                    x.v[2 * u + 1] = xr[1];
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) x.v[4 * u + q] = make_uint4(0, 0, 0, 0);
+                if (src >= 0) {
+                    const uint4* xr = (const uint4*) ((const float*) Xv + (size_t) src * a.xs + k0 + h);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) x.v[4 * u + q] = xr[q];
+                }
+            }
+        }
+    };
+    auto store_step = [&](int buf, int s, const MmRec& r, const MmX<MT, PACKED>& x) {
+        float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (row < a.R) {
+            if (seedf) {
+                const int sb = (s >> 3) & 1, b = 4 * (s & 7) + jb;   // block b of the staged super-step
+                const uint32_t seed = rec_seed[sb][rr][b], word = rec_word[sb][rr][b];
+                int is[8], code;
+                if (fmt == MF_SEED4P4) {
+                    block_isum<4>(tab, seed, word, is);
+                    code = (int) ((rec_code[sb][rr][b >> 3] >> (4 * (b & 7))) & 15u);
+                } else {
+                    block_isum<3>(tab, seed, word, is);
+                    code = (int) (word & 15u);
+                }
+                const float sc = pow2f(wt.eb + code) * NSLM_R32;
+#pragma unroll
+                for (int c = 0; c < 8; ++c) f[c] = (float) is[c] * sc;
+            } else if (fmt == MF_BF16) {
+                const uint32_t u[4] = {r.raw[0].x, r.raw[0].y, r.raw[0].z, r.raw[0].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { f[2 * i] = __uint_as_float(u[i] << 16); f[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u); }
+            } else {
+                const float sc = bf(r.seed), b = bf(r.word);
+                if (fmt == MF_Q8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        f[i] = bfr(sc * (float) ((r.raw[0].x >> (8 * i)) & 255u) + b);
+                        f[4 + i] = bfr(sc * (float) ((r.raw[0].y >> (8 * i)) & 255u) + b);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f[i] = bfr(sc * (float) ((r.raw[0].x >> (4 * i)) & 15u) + b);
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NTERM; ++q) {   // f = hi + mid + lo: each term the BF16 value of what remains (exact)
+            uint32_t h[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { h[i] = tobf(f[i]); f[i] -= bf(h[i]); }
+            *(uint4*) &Wsm[buf][q][rr][jb * 8] = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+        }
+#pragma unroll
+        for (int u = 0; u < MT; ++u) {
+            const int i = ptid + 256 * u, n = i >> 1, h = (i & 1) * 16;
+            if (PACKED) {
+                *(uint4*) &Xsm[buf][n][h] = x.v[2 * u];
+                *(uint4*) &Xsm[buf][n][h + 8] = x.v[2 * u + 1];
+            } else {
+                const uint4 p0 = x.v[4 * u], p1 = x.v[4 * u + 1], p2 = x.v[4 * u + 2], p3 = x.v[4 * u + 3];
+#define F(w) __uint_as_float(w)
+                *(uint4*) &Xsm[buf][n][h] = make_uint4(pack_bf2(F(p0.x), F(p0.y)), pack_bf2(F(p0.z), F(p0.w)), pack_bf2(F(p1.x), F(p1.y)), pack_bf2(F(p1.z), F(p1.w)));
+                *(uint4*) &Xsm[buf][n][h + 8] = make_uint4(pack_bf2(F(p2.x), F(p2.y)), pack_bf2(F(p2.z), F(p2.w)), pack_bf2(F(p3.x), F(p3.y)), pack_bf2(F(p3.z), F(p3.w)));
+#undef F
+            }
+        }
+    };
+
+    // ---- the pipeline: each role runs its own loop (same barrier count) so neither carries the other's registers -----------
+    // Step ps is produced into buffer ps & 1 while the consumers multiply step ps - 1 out of the other buffer.
+    if (producer) {
+        MmRec ra = {}, rb = {};
+        MmX<MT, PACKED> xa, xb;
+        load_x(0, xa);
+        load_x(1, xb);
+        load_rec(0, ra);
+        load_rec(1, rb);
+        Chunk rec = load_super(0);
+        store_super(0, rec);
+        rec = load_super(1);
+        lds_barrier();   // super-step 0's records are in LDS
+        for (int ps = 0; ps < nsteps; ps += 2) {
+            if ((ps & 7) == 0) {   // the next super-step's records (fetched 8 steps ago) go to LDS, the one after is requested
+                store_super(((ps >> 3) + 1) & 1, rec);
+                rec = load_super((ps >> 3) + 2);
+            }
+            store_step(0, ps, ra, xa);
+            load_x(ps + 2, xa);
+            load_rec(ps + 2, ra);
+            lds_barrier();
+            if (ps + 1 >= nsteps) break;
+            store_step(1, ps + 1, rb, xb);
+            load_x(ps + 3, xb);
+            load_rec(ps + 3, rb);
+            lds_barrier();
+        }
+        return;
+    }
+
+    // ---- consumer side ---------------------------------------------------------------------------------------------------
     f32x16 acc[MT][2];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
@@ -109,60 +306,30 @@ __global__ void __launch_bounds__(256) k_mm(int fmt, MmArgs a, WSlice wd, const 
         for (int n = 0; n < 2; ++n)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[m][n][i] = 0.0f;
-    const int wtok = wv * 32 * MT;          // this wave's first token of the tile
-    const bool wave_live = wtok < count;    // a wave whose tokens are all padding only helps to decode
+    const int wtok = wv * 32 * MT;          // this consumer wave's first token of the tile
+    const bool wave_live = wtok < count;    // a consumer whose tokens are all padding has nothing to multiply
     const int frow = lane & 31, fk = (lane >> 5) * 8;
-
-    for (int k0 = 0; k0 < a.K; k0 += BK) {
-        {   // weights: 64 rows x 4 blocks, one block per thread
-            const int rr = tid >> 2, jb = tid & 3, row = r0 + rr;
-            float f[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (row < a.R) tile_block(fmt, wt, tab, row, a.K, k0 / 8 + jb, f);
+    auto consume = [&](int buf) {
+        if (!wave_live) return;
 #pragma unroll
-            for (int q = 0; q < NTERM; ++q) {   // f = hi + mid + lo: each term the BF16 value of what remains (exact)
-                uint32_t h[8];
+        for (int kk = 0; kk < BK; kk += 16) {
+            bf16x8 af[MT];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) { h[i] = tobf(f[i]); f[i] -= bf(h[i]); }
-                *(uint4*) &Wsm[q][rr][jb * 8] = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
-            }
-        }
-        // activations: BN tokens x 32 k, 16 per thread per pass
-        for (int i = tid; i < BN * 2; i += 256) {
-            const int n = i >> 1, h = (i & 1) * 16, src = srow[n];
-            uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
-            if (src >= 0) {
-                if (PACKED) {
-                    const uint4* xr = (const uint4*) ((const uint16_t*) Xv + (size_t) src * a.xs + k0 + h);
-                    v0 = xr[0];
-                    v1 = xr[1];
-                } else {
-                    const float4* xr = (const float4*) ((const float*) Xv + (size_t) src * a.xs + k0 + h);
-                    const float4 x0 = xr[0], x1 = xr[1], x2 = xr[2], x3 = xr[3];
-                    v0 = make_uint4(pack_bf2(x0.x, x0.y), pack_bf2(x0.z, x0.w), pack_bf2(x1.x, x1.y), pack_bf2(x1.z, x1.w));
-                    v1 = make_uint4(pack_bf2(x2.x, x2.y), pack_bf2(x2.z, x2.w), pack_bf2(x3.x, x3.y), pack_bf2(x3.z, x3.w));
+            for (int m = 0; m < MT; ++m) af[m] = *(const bf16x8*) &Xsm[buf][wtok + 32 * m + frow][kk + fk];
+#pragma unroll
+            for (int q = 0; q < NTERM; ++q)   // the largest term first
+#pragma unroll
+                for (int n = 0; n < 2; ++n) {
+                    const bf16x8 bfrag = *(const bf16x8*) &Wsm[buf][q][32 * n + frow][kk + fk];
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[m], bfrag, acc[m][n], 0, 0, 0);
                 }
-            }
-            *(uint4*) &Xsm[n][h] = v0;
-            *(uint4*) &Xsm[n][h + 8] = v1;
         }
-        __syncthreads();
-        if (wave_live) {
-#pragma unroll
-            for (int kk = 0; kk < BK; kk += 16) {
-                bf16x8 af[MT];
-#pragma unroll
-                for (int m = 0; m < MT; ++m) af[m] = *(const bf16x8*) &Xsm[wtok + 32 * m + frow][kk + fk];
-#pragma unroll
-                for (int q = 0; q < NTERM; ++q)   // the largest term first
-#pragma unroll
-                    for (int n = 0; n < 2; ++n) {
-                        const bf16x8 bfrag = *(const bf16x8*) &Wsm[q][32 * n + frow][kk + fk];
-#pragma unroll
-                        for (int m = 0; m < MT; ++m) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[m], bfrag, acc[m][n], 0, 0, 0);
-                    }
-            }
-        }
-        __syncthreads();
+    };
+    lds_barrier();   // pairs with the producers' barrier after the first records
+    for (int s = 0; s < nsteps; ++s) {
+        lds_barrier();   // step s is in buffer s & 1
+        consume(s & 1);
     }
     if (!wave_live) return;
     // accumulator element v of lane l: token row 8 * (v / 4) + 4 * (l / 32) + v % 4, weight column l % 32
@@ -172,19 +339,368 @@ __global__ void __launch_bounds__(256) k_mm(int fmt, MmArgs a, WSlice wd, const 
         for (int n = 0; n < 2; ++n)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int tok = wtok + 32 * m + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), row = r0 + 32 * n + (lane & 31);
+                const int tok = wtok + 32 * m + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), orow = r0 + 32 * n + (lane & 31);
                 const int dst = drow[tok];
-                if (dst < 0 || row >= a.R) continue;
-                store_y(Y + (size_t) dst * a.ys + row, acc[m][n][v], a.add, a.f32out);
+                if (dst < 0 || orow >= a.R) continue;
+                store_y(Y + (size_t) dst * a.ys + orow, acc[m][n][v], a.add, a.f32out);
             }
 }
+
+// a kernel that asks for more dynamic LDS than the default limit has the limit raised to what it needs, once
+template <typename Kern>
+void allow_big_lds(Kern k, size_t bytes) {
+    static const hipError_t once = bytes > 48 * 1024 ? hipFuncSetAttribute((const void*) k, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes)
+                                                     : hipSuccess;
+    (void) once;
+}
+template <int MT, int NTERM>
+constexpr size_t mm_lds() { return (size_t) (2 * NTERM * BM * LDW + 2 * 128 * MT * LDW) * sizeof(uint16_t); }
 
 template <int MT, bool PACKED>
 void launch_mm(hipStream_t st, int fmt, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
                const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
     const bool exact = g_seed_exact && (fmt == MF_SEED4 || fmt == MF_SEED4P4);
-    if (exact) hipLaunchKernelGGL((k_mm<MT, 3, PACKED>), grid, dim3(256), 0, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
-    else hipLaunchKernelGGL((k_mm<MT, 1, PACKED>), grid, dim3(256), 0, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
+    if (exact) {
+        const size_t lds = mm_lds<MT, 3>();
+        allow_big_lds(k_mm<MT, 3, PACKED>, lds);
+        hipLaunchKernelGGL((k_mm<MT, 3, PACKED>), grid, dim3(512), lds, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
+    } else {
+        const size_t lds = mm_lds<MT, 1>();
+        allow_big_lds(k_mm<MT, 1, PACKED>, lds);
+        hipLaunchKernelGGL((k_mm<MT, 1, PACKED>), grid, dim3(512), lds, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
+    }
+    host_note_launch();
+}
+
+// ---- the streamed kernel: BF16 activations go from global memory straight into LDS -----------------------------------------
+//
+// For packed (BF16) activations and one BF16 term per weight.  512 threads: waves 0-3 are consumers, waves 4-7 producers.
+//   * Weights move in steps of 64 K: producer thread (rr, jb) decodes blocks 2 jb and 2 jb + 1 of row rr (two independent
+//     chains in one instruction stream) into one of two LDS tiles; one workgroup barrier per step hands the tile over.
+//     The thread's records (a dword of seeds, a dword of coefficient words, a byte of codes) are requested four steps
+//     before they are decoded and wait in registers; the four threads of a row read 16 consecutive bytes of each stream,
+//     so every line comes from HBM once.
+//   * Activations never touch a register on their way in: consumer wave w owns tokens [32 MT w, 32 MT (w + 1)) and fetches
+//     its own rows with global_load_lds_dwordx4 (each lane lands 16 bytes at consecutive LDS addresses) into a ring of
+//     four 32-K stages, three stages ahead of the MFMAs.  Only the owning wave reads those rows back, so the ring needs
+//     no barrier - the wave waits on its own vector-memory counter.
+//   * The 16-byte slots of a row (4 per 64-byte row) are stored XOR-swizzled by the row number so that the fragment reads
+//     (32 rows x one slot per half wave) spread over all banks although the rows are unpadded; the swizzle is applied on
+//     the global side, where every lane is free to pick the address it loads.
+#define WK 64            // K per weight step
+#define LDW2 72          // weight tile row stride in BF16 elements (144 bytes)
+#define XCHUNK 2048      // BF16 elements of an activation chunk: 32 tokens x 64 K
+#define RECD 4           // weight steps between a record's request and its decode
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {   // v_cvt_pk_bf16_f32: both round to nearest even
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ int x_swizzle(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+struct MmRec2 {
+    uint4 raw[2];      // BF16: the two blocks; Q8: raw[0]; Q4: raw[0].xy
+    uint32_t u, v, c;  // seeds: two seeds, two coefficient words, the codes byte; Q8 / Q4: the group's scale and bias bits
+};
+
+#ifdef NSLM_MM_STAMPS   // development builds only: wall-clock stamps of every workgroup behind the T x ys results
+#define MM_STAMP(t, step, slot) do { } while (0)
+#define MM_WG_STAMP(t, slot) do { if (tid == (t)) ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define MM_STAMP(t, step, slot) do { } while (0)
+#define MM_WG_STAMP(t, slot) do { } while (0)
+#endif
+#ifndef NSLM_MM_ABLATE   // development builds only: 1 no activation loads, 2 no decode, 4 no MFMA
+#define NSLM_MM_ABLATE 0
+#endif
+template <int CT, int NCW, int FMT>
+__global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice wd, const WSlice* ws, const uint16_t* X, float* Y,
+                                                   const int32_t* perm, const MmTile* tiles, const int32_t* ntiles) {
+    constexpr int BN = 32 * CT * NCW, NTHR = 64 * (NCW + 4), XCH = 32 / NCW;   // XCH: chunks in a consumer wave's ring (128 KB in all)
+    constexpr bool seedf = FMT == MF_SEED4P4 || FMT == MF_SEED4;
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    uint16_t* Xs = smem;                                   // [NCW waves][XCH chunks][32 rows][64 K], slots swizzled
+    typedef uint16_t WTile[BM][LDW2];
+    WTile* Wsm = (WTile*) (smem + NCW * XCH * XCHUNK);          // [2]
+    __shared__ int srow[BN], drow[BN];
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    MM_WG_STAMP(0, 0);
+    const bool producer = wv >= NCW;
+    const bool grouped = tiles != nullptr;
+    if (grouped && ntiles && (int) blockIdx.y >= *ntiles) return;
+    const int r0 = (int) blockIdx.x * BM;
+    int start, count;
+    WSlice wt;
+    if (grouped) {
+        const MmTile tl = tiles[blockIdx.y];
+        wt = ws[tl.slice];
+        start = tl.start;
+        count = tl.count;
+    } else {
+        wt = wd;
+        start = (int) blockIdx.y * BN;
+        count = min(BN, a.T - start);
+    }
+    if (count < 1) return;
+    if (seedf) load_tables(tab);
+    for (int i = tid; i < BN; i += NTHR) {
+        const bool ok = i < count;
+        const int j = start + (ok ? i : 0);   // padding rows load the tile's first row; their results are never stored
+        srow[i] = grouped ? perm[j] / a.xdiv : j;
+        drow[i] = !ok ? -1 : grouped ? perm[j] : j;
+    }
+    __syncthreads();
+    const int nsteps = a.K / WK;
+
+    if (producer) {
+        const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = r0 + rr, nbk = a.K / 8;
+        const bool live = row < a.R;
+        const bool al4 = (((uintptr_t) wt.p[0] | (uintptr_t) wt.p[1]) & 3u) == 0;
+        // this thread's two blocks of step s
+        auto load_rec = [&](int s, MmRec2& r) {
+            if (s >= nsteps || !live) return;
+            if (seedf) {
+                const size_t g = (size_t) row * nbk + (size_t) s * (WK / 8) + 2 * jb;   // even: the pair shares a dword and a codes byte
+                const NSLM_GLOBAL uint16_t *sp = gp<uint16_t>(wt.p[0]) + g, *cp = gp<uint16_t>(wt.p[1]) + g;
+                if (al4) {
+                    r.u = *(const NSLM_GLOBAL uint32_t*) sp;
+                    r.v = *(const NSLM_GLOBAL uint32_t*) cp;
+                } else {
+                    r.u = sp[0] | (uint32_t) sp[1] << 16;
+                    r.v = cp[0] | (uint32_t) cp[1] << 16;
+                }
+                if (FMT == MF_SEED4P4) r.c = gp<uint8_t>(wt.p[3])[g >> 1];
+                return;
+            }
+            const size_t e0 = (size_t) row * a.K + (size_t) s * WK + 16 * jb;   // first of 16 elements
+            if (FMT == MF_BF16) {
+                r.raw[0] = ldg16(gp<uint16_t>(wt.p[0]) + e0);
+                r.raw[1] = ldg16(gp<uint16_t>(wt.p[0]) + e0 + 8);
+            } else {
+                const size_t gi = e0 >> group_shift(wt);
+                r.u = gp<uint16_t>(wt.p[1])[gi];
+                r.v = gp<uint16_t>(wt.p[2])[gi];
+                if (FMT == MF_Q8) r.raw[0] = ldg16(gp<uint8_t>(wt.p[0]) + e0);
+                else r.raw[0] = make_uint4(gp<uint32_t>(wt.p[0])[e0 / 8], gp<uint32_t>(wt.p[0])[e0 / 8 + 1], 0, 0);
+            }
+        };
+        // seeds: the table reads of a step's two blocks are issued one step early (its records are in registers by then)
+        struct Look { uint32_t g[2], qa[2], qb[2]; };
+        auto lookup = [&](const MmRec2& r, Look& k) {
+            if (!seedf) return;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t seed = h ? r.u >> 16 : r.u & 0xFFFFu, word = h ? r.v >> 16 : r.v & 0xFFFFu;
+                k.g[h] = stream_of(tab, seed);
+                k.qa[h] = FMT == MF_SEED4P4 ? tab[512 + (word & 0xFFu)] : tab[512 + ((word >> 4) & 0xFFu)];
+                k.qb[h] = FMT == MF_SEED4P4 ? tab[512 + (word >> 8)] : tab[512 + (word >> 12)];
+            }
+        };
+        auto produce = [&](int s, const MmRec2& r, const Look& k) {
+            float f[2][8];   // rows past R decode their zeroed records: harmless, their outputs are never stored
+            {
+                if (NSLM_MM_ABLATE & 2) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) f[0][c] = f[1][c] = __uint_as_float(r.u);
+                } else if (seedf) {
+                    const uint32_t up[2] = {r.u << 16, r.u}, word[2] = {r.v & 0xFFFFu, r.v >> 16};
+                    int is[2][8];
+                    if (FMT == MF_SEED4P4) isum2_p4(up, k.g, k.qa, k.qb, is);
+                    else isum2_p3(up, k.g, k.qa, k.qb, is);
+                    float sc[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int code = FMT == MF_SEED4P4 ? (int) ((r.c >> (4 * h)) & 15u) : (int) (word[h] & 15u);
+                        sc[h] = pow2f(wt.eb + code) * NSLM_R32;
+                    }
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) f[h][c] = (float) is[h][c];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) f[h][c] *= sc[h];
+                    __builtin_amdgcn_sched_barrier(0);
+                } else if (FMT == MF_BF16) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const uint32_t u[4] = {r.raw[h].x, r.raw[h].y, r.raw[h].z, r.raw[h].w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { f[h][2 * i] = __uint_as_float(u[i] << 16); f[h][2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u); }
+                    }
+                } else {
+                    const float sc = bf(r.u), b = bf(r.v);
+                    const uint32_t u[4] = {r.raw[0].x, r.raw[0].y, r.raw[0].z, r.raw[0].w};
+                    if (FMT == MF_Q8) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) f[i >> 3][i & 7] = bfr(sc * (float) ((u[i >> 2] >> (8 * (i & 3))) & 255u) + b);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) f[i >> 3][i & 7] = bfr(sc * (float) ((u[i >> 3] >> (4 * (i & 7))) & 15u) + b);
+                    }
+                }
+            }
+            MM_STAMP(256, s, 10);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                *(uint4*) &Wsm[s & 1][rr][16 * jb + 8 * h] = make_uint4(cvt_pk_bf16(f[h][0], f[h][1]), cvt_pk_bf16(f[h][2], f[h][3]),
+                                                                       cvt_pk_bf16(f[h][4], f[h][5]), cvt_pk_bf16(f[h][6], f[h][7]));
+        };
+        MmRec2 rec[RECD] = {};
+        Look look[2] = {};
+#pragma unroll
+        for (int u = 0; u < RECD; ++u) load_rec(u, rec[u]);
+        lookup(rec[0], look[0]);
+        for (int s0 = 0; s0 < nsteps; s0 += RECD) {
+#pragma unroll
+            for (int u = 0; u < RECD; ++u) {
+                if (s0 + u >= nsteps) break;
+                lookup(rec[(u + 1) % RECD], look[(u + 1) & 1]);   // the next step's table reads travel under this step's decode
+                produce(s0 + u, rec[u], look[u & 1]);
+                load_rec(s0 + u + RECD, rec[u]);
+                MM_STAMP(256, s0 + u, 8);
+                lds_barrier();
+                MM_STAMP(256, s0 + u, 9);
+            }
+        }
+        return;
+    }
+
+    // ---- consumer side ---------------------------------------------------------------------------------------------------
+    const int wtok = wv * 32 * CT;          // this wave's first token of the tile
+    if (wtok >= count) {                    // a wave whose tokens are all padding has nothing to multiply
+        for (int s = 0; s < nsteps; ++s) lds_barrier();
+        return;
+    }
+    __builtin_amdgcn_s_setprio(2);   // the matrix pipeline's instruction stream goes first when both roles are ready
+    f32x16 acc[CT][2];
+#pragma unroll
+    for (int m = 0; m < CT; ++m)
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[m][n][i] = 0.0f;
+    // Chunk c = s MT + m is the 32 tokens of m-tile m x the 64 K of weight step s: 4 KB, four instructions, instruction i
+    // landing rows 8 i + lane / 8, slot lane % 8 (whole 128-byte lines per row).  The wave's ring holds XCH chunks.
+    // Offsets from X are 32-bit where the host has checked that they fit (MT > 1), so the loads take the scalar base +
+    // vector offset form and cost no address arithmetic.
+    typedef typename std::conditional<CT == 1, size_t, uint32_t>::type xoff_t;
+    xoff_t xoff[4 * CT];
+#pragma unroll
+    for (int i = 0; i < 4 * CT; ++i) {
+        const int row = 8 * (i & 3) + (lane >> 3), n = wtok + 32 * (i >> 2) + row, piece = (lane & 7) ^ x_swizzle(row);
+        xoff[i] = (xoff_t) (((size_t) srow[n] * (size_t) a.xs + 8u * (size_t) piece) * 2u);
+    }
+    uint16_t* ring = Xs + wv * (XCH * XCHUNK);
+    auto fetch = [&](int sf, int mf, int slot) {   // chunk (sf, mf) -> ring slot (past the end: a harmless reload of the last step)
+        if (NSLM_MM_ABLATE & 1) return;
+        const char* src = (const char*) X + (size_t) min(sf, nsteps - 1) * WK * 2;
+        uint16_t* dst = ring + slot * XCHUNK;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (src + xoff[4 * mf + i]),
+                                             (__attribute__((address_space(3))) void*) (dst + i * 512), 16, 0, 0);
+    };
+    const int frow = lane & 31, fhi = lane >> 5, fsw = x_swizzle(frow);
+    auto load_a = [&](int slot, bf16x8 (&af)[4]) {
+        const uint16_t* ch = ring + slot * XCHUNK + frow * 64;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) af[kk] = *(const bf16x8*) (ch + ((2 * kk + fhi) ^ fsw) * 8);
+    };
+    // One weight step: chunk m multiplies out of fragment set (m even ? fa : fb) while the next chunk's fragments travel
+    // into the other set; with MT odd the sets have swapped roles when the step ends.
+    auto step = [&](int s, bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
+        MM_STAMP(0, s, 0);
+        lds_barrier();   // weight step s is in tile s & 1
+        MM_STAMP(0, s, 1);
+        bf16x8 bq[4][2];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+            for (int n = 0; n < 2; ++n) bq[kk][n] = *(const bf16x8*) &Wsm[s & 1][32 * n + frow][16 * kk + 8 * fhi];
+#pragma unroll
+        for (int m = 0; m < CT; ++m) {
+            const int c = s * CT + m;
+            fetch(s + (m + XCH - 1) / CT, (m + XCH - 1) % CT, (c + XCH - 1) % XCH);   // into the slot chunk c - 1 just left
+            wait_vm<4 * (XCH - 2)>();   // chunks up to c + 1 have landed
+            load_a((c + 1) % XCH, (m & 1) ? fa : fb);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int n = 0; n < 2; ++n)
+                    if (!(NSLM_MM_ABLATE & 4)) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(((m & 1) ? fb : fa)[kk], bq[kk][n], acc[m][n], 0, 0, 0);
+            MM_STAMP(0, s, 2 + m);
+        }
+    };
+    MM_WG_STAMP(0, 1);
+    if (nsteps > 0) {
+#pragma unroll
+        for (int c = 0; c < XCH - 1; ++c) fetch(c / CT, c % CT, c);
+    }
+    bf16x8 f0[4], f1[4];
+    wait_vm<4 * (XCH - 2)>();   // chunk 0 has landed
+    load_a(0, f0);
+    for (int s = 0; s < nsteps; s += 2) {
+        step(s, f0, f1);
+        if (s + 1 >= nsteps) break;
+        if (CT & 1) step(s + 1, f1, f0);
+        else step(s + 1, f0, f1);
+    }
+    wait_vm<0>();
+    MM_WG_STAMP(0, 2);
+    // accumulator element v of lane l: token row 8 * (v / 4) + 4 * (l / 32) + v % 4, weight column l % 32
+    const bool plain = !a.add && !a.f32out;
+#pragma unroll
+    for (int m = 0; m < CT; ++m)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int tok = wtok + 32 * m + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+            const int dst = drow[tok];
+            if (dst < 0) continue;
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                const int orow = r0 + 32 * n + (lane & 31);
+                if (orow >= a.R) continue;
+                float* yo = Y + (size_t) dst * a.ys + orow;
+                if (plain) __builtin_nontemporal_store(bfr(acc[m][n][v]), yo);
+                else store_y(yo, acc[m][n][v], a.add, a.f32out);
+            }
+        }
+    MM_WG_STAMP(0, 3);
+}
+constexpr size_t mm_stream_lds() { return (size_t) (32 * XCHUNK + 2 * BM * LDW2) * sizeof(uint16_t); }
+// the streamed kernel takes BF16 activations in 16-byte aligned rows, one BF16 term per weight, K in whole weight steps
+// (xrows > 0: the row count, for the variants that address rows by 32-bit byte offsets)
+bool stream_ok(int fmt, int K, int xs, const void* x, long long xrows) {
+    const bool exact = g_seed_exact && (fmt == MF_SEED4 || fmt == MF_SEED4P4);
+    return !exact && K % WK == 0 && xs % 8 == 0 && ((uintptr_t) x & 15u) == 0 && (xrows * xs + K) * 2 < (1ll << 32);
+}
+template <int CT, int NCW, int FMT>
+void launch_mm_stream_f(hipStream_t st, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
+                        const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
+    const size_t lds = mm_stream_lds();
+    auto kern = k_mm_stream<CT, NCW, FMT>;
+    allow_big_lds(kern, lds);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * (NCW + 4)), lds, st, a, wd, ws, (const uint16_t*) X, Y, perm, tiles, ntiles);
+    host_note_launch();
+}
+template <int CT, int NCW>
+void launch_mm_stream(hipStream_t st, int fmt, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
+                      const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
+    switch (fmt) {
+        case MF_SEED4P4: launch_mm_stream_f<CT, NCW, MF_SEED4P4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_SEED4: launch_mm_stream_f<CT, NCW, MF_SEED4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_BF16: launch_mm_stream_f<CT, NCW, MF_BF16>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_Q8: launch_mm_stream_f<CT, NCW, MF_Q8>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        default: launch_mm_stream_f<CT, NCW, MF_Q4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+    }
 }
 
 template <bool PACKED>
@@ -192,6 +708,12 @@ void mm_dense(hipStream_t st, int fmt, WSlice w, int K, int R, const void* x, in
     if (T < 1 || R < 1) return;
     MmArgs a = {K, R, T, xs, ys, 1, add, host_store_f32()};
     const unsigned gx = (unsigned) (R + BM - 1) / BM;
+    if (PACKED && stream_ok(fmt, K, xs, x, T)) {
+        if (T > 256) launch_mm_stream<2, 8>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
+        else if (T > 128) launch_mm_stream<2, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
+        else launch_mm_stream<1, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
+        return;
+    }
     if (T > 256) launch_mm<4, PACKED>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
     else if (T > 128) launch_mm<2, PACKED>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
     else launch_mm<1, PACKED>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
@@ -202,6 +724,10 @@ void mm_grouped(hipStream_t st, int fmt, const WSlice* ws, int K, int R, const v
     if (grid_tiles < 1 || R < 1) return;
     MmArgs a = {K, R, 0, xs, ys, xdiv, 0, host_store_f32()};
     WSlice none = {};
+    if (PACKED && stream_ok(fmt, K, xs, x, 0)) {
+        launch_mm_stream<1, 4>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
+        return;
+    }
     launch_mm<1, PACKED>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
 }
 

@@ -19,18 +19,18 @@ __device__ __forceinline__ Chunk load_chunk(const WSlice& w, uint32_t unit, bool
     c.codes = 0;
     if (!ok) return c;
     if (al) {
-        c.sd = ((const uint4*) w.p[0])[unit];
-        c.cw = ((const uint4*) w.p[1])[unit];
-        if (P == 4) c.codes = ((const uint32_t*) w.p[3])[unit];
+        c.sd = ldg16(gp<uint4>(w.p[0]) + unit);
+        c.cw = ldg16(gp<uint4>(w.p[1]) + unit);
+        if (P == 4) c.codes = gp<uint32_t>(w.p[3])[unit];
     } else {
-        const uint16_t* sp = (const uint16_t*) w.p[0] + (size_t) unit * 8;
-        const uint16_t* cp = (const uint16_t*) w.p[1] + (size_t) unit * 8;
+        const NSLM_GLOBAL uint16_t* sp = gp<uint16_t>(w.p[0]) + (size_t) unit * 8;
+        const NSLM_GLOBAL uint16_t* cp = gp<uint16_t>(w.p[1]) + (size_t) unit * 8;
         c.sd = make_uint4(sp[0] | (uint32_t) sp[1] << 16, sp[2] | (uint32_t) sp[3] << 16, sp[4] | (uint32_t) sp[5] << 16,
                           sp[6] | (uint32_t) sp[7] << 16);
         c.cw = make_uint4(cp[0] | (uint32_t) cp[1] << 16, cp[2] | (uint32_t) cp[3] << 16, cp[4] | (uint32_t) cp[5] << 16,
                           cp[6] | (uint32_t) cp[7] << 16);
         if (P == 4) {
-            const uint8_t* ep = (const uint8_t*) w.p[3] + (size_t) unit * 4;
+            const NSLM_GLOBAL uint8_t* ep = gp<uint8_t>(w.p[3]) + (size_t) unit * 4;
             c.codes = ep[0] | (uint32_t) ep[1] << 8 | (uint32_t) ep[2] << 16 | (uint32_t) ep[3] << 24;
         }
     }
@@ -88,11 +88,11 @@ __device__ __forceinline__ void block_weights(int fmt, const WSlice& w, const ui
     *sc = 1.0f;
     if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
         const size_t g = (size_t) r * nbk + j;
-        const uint32_t seed = ((const uint16_t*) w.p[0])[g], word = ((const uint16_t*) w.p[1])[g];
+        const uint32_t seed = gp<uint16_t>(w.p[0])[g], word = gp<uint16_t>(w.p[1])[g];
         int is[8], code;
         if (fmt == MF_SEED4P4) {
             block_isum<4>(tab, seed, word, is);
-            code = (((const uint8_t*) w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
+            code = (gp<uint8_t>(w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
         } else {
             block_isum<3>(tab, seed, word, is);
             code = (int) (word & 15u);
@@ -101,18 +101,18 @@ __device__ __forceinline__ void block_weights(int fmt, const WSlice& w, const ui
         for (int c = 0; c < 8; ++c) o[c] = (float) is[c];
         *sc = pow2f(w.eb + code) * NSLM_R32;
     } else if (fmt == MF_BF16) {
-        const uint16_t* v = (const uint16_t*) w.p[0] + (size_t) r * K + (size_t) j * 8;
+        const NSLM_GLOBAL uint16_t* v = gp<uint16_t>(w.p[0]) + (size_t) r * K + (size_t) j * 8;
 #pragma unroll
         for (int c = 0; c < 8; ++c) o[c] = bf(v[c]);
     } else {
         const size_t e0 = (size_t) r * K + (size_t) j * 8, gi = e0 >> group_shift(w);
-        const float s = bf(((const uint16_t*) w.p[1])[gi]), b = bf(((const uint16_t*) w.p[2])[gi]);
+        const float s = bf(gp<uint16_t>(w.p[1])[gi]), b = bf(gp<uint16_t>(w.p[2])[gi]);
         if (fmt == MF_Q8) {
-            const uint32_t* q = (const uint32_t*) w.p[0] + e0 / 4;
+            const NSLM_GLOBAL uint32_t* q = gp<uint32_t>(w.p[0]) + e0 / 4;
 #pragma unroll
             for (int c = 0; c < 8; ++c) o[c] = bfr(s * (float) ((q[c >> 2] >> (8 * (c & 3))) & 255u) + b);
         } else {
-            const uint32_t q = ((const uint32_t*) w.p[0])[e0 / 8];
+            const uint32_t q = gp<uint32_t>(w.p[0])[e0 / 8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) o[c] = s * (float) ((q >> (4 * c)) & 15u) + b;
         }
