@@ -409,7 +409,7 @@ struct MmRec2 {
 
 #ifdef NSLM_MM_STAMPS   // development builds only: wall-clock stamps of every workgroup behind the T x ys results
 #define MM_STAMP(t, step, slot) do { } while (0)
-#define MM_WG_STAMP(t, slot) do { if (tid == (t)) ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#define MM_WG_STAMP(t, slot) do { if (tid == (t)) { ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + (slot)] = wall_clock64(); ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + 4 + (slot)] = clock64(); } } while (0)
 #else
 #define MM_STAMP(t, step, slot) do { } while (0)
 #define MM_WG_STAMP(t, slot) do { } while (0)
