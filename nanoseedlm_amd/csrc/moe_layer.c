@@ -16,6 +16,7 @@ struct NslmMoe {
     uint8_t* unit_host;         /* staging for one unit */
     int32_t* eb;                /* host: [units][3] exponent biases */
     uint16_t *rw, *rb;          /* device: router weights [layer][n_exp][d], biases [layer][n_exp] */
+    uint16_t* px;               /* device: BF16 view of the step's activations [max_rows][d] (batched path) */
     float *logit, *score, *wt, *A, *G, *U, *D, *zero;
     int32_t *ind, *perm, *ntiles;
     MmTile* tiles;
@@ -82,6 +83,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     bad |= nh_malloc((void**) &m->ind, 4 * (size_t) P);
     bad |= nh_malloc((void**) &m->A, 4 * (size_t) P * c->ff);
     bad |= nh_malloc((void**) &m->G, 4 * (size_t) P * c->ff);
+    bad |= nh_malloc((void**) &m->px, 2 * (size_t) c->max_rows * c->d);
     bad |= nh_malloc((void**) &m->U, 4 * (size_t) P * c->ff);
     bad |= nh_malloc((void**) &m->D, 4 * (size_t) P * c->d);
     bad |= nh_malloc((void**) &m->zero, 4 * (size_t) c->max_rows * c->d);
@@ -107,7 +109,7 @@ void nslm_moe_close(NslmMoe* m) {
     if (!m) return;
     void* d[] = {m->arena, m->resident ? NULL : m->pool.vram, m->pool.unit_slot, m->pool.slot_unit, m->pool.slot_last, m->pool.tick,
                  m->pool.stats, m->pool.jobs, m->pool.njobs, m->pool.tab, m->rw, m->rb, m->logit, m->score, m->wt, m->ind, m->A,
-                 m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles, m->sync};
+                 m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles, m->sync, m->px};
     for (size_t i = 0; i < sizeof d / sizeof d[0]; ++i)
         if (d[i]) nh_free(d[i]);
     free(m->unit_host);
@@ -211,11 +213,24 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         kc_mv_gu(s, c->fmt, gate, up, d, ff, xn, d, m->A, ff, m->ind, P, k, NULL);
         kc_mv_sel(s, c->fmt, down, ff, d, m->A, ff, m->D, d, m->ind, P, 1, NULL);
     } else {              /* batched: pairs grouped by expert, three grouped GEMMs (engine/mova_cuda.c:1308-1317) */
+        /* BF16 views of the activations feed the MFMA path, as the reference's packed_layer() case does
+           (engine/mova_cuda.c:1012-1035,1229,1308-1317): SwiGLU has consumed G, so G's storage holds A's view */
+        const int packed = d % 8 == 0 && ff % 8 == 0;
         kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
-        kc_mm_grouped_dev(s, c->fmt, gate, d, ff, xn, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
-        kc_mm_grouped_dev(s, c->fmt, up, d, ff, xn, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
-        kc_swiglu(s, m->G, m->U, m->A, P * ff);
-        kc_mm_grouped_dev(s, c->fmt, down, ff, d, m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+        if (packed) {
+            kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);
+            kc_mm_grouped_packed(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+            kc_mm_grouped_packed(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+            kc_swiglu(s, m->G, m->U, m->A, P * ff);
+            kc_pack_input_bf16(s, m->A, (uint16_t*) m->G, (size_t) P * ff);
+            kc_mm_grouped_packed(s, c->fmt, down, ff, d, (const uint16_t*) m->G, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
+                                 m->max_tiles, NULL);
+        } else {
+            kc_mm_grouped_dev(s, c->fmt, gate, d, ff, xn, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+            kc_mm_grouped_dev(s, c->fmt, up, d, ff, xn, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+            kc_swiglu(s, m->G, m->U, m->A, P * ff);
+            kc_mm_grouped_dev(s, c->fmt, down, ff, d, m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+        }
     }
     if (c->router == NSLM_ROUTE_SOFTMAX) kq4_moe_combine(s, d, k, m->D, m->wt, m->zero, m->zero, 0, io, T);
     else kc_moe_combine(s, m->D, m->wt, m->zero, io, d, k, T);

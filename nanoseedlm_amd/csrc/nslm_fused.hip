@@ -155,6 +155,9 @@ __device__ __forceinline__ void stage_row(const float* src, int n, float* xl, bo
     for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = coherent ? ld_agent(src + i) : src[i];
 }
 
+#ifdef NSLM_FUSED_STAMPS
+__device__ unsigned long long g_fstamp[1024 * 8];
+#endif
 template <int P, bool SHFL_G, bool SHFL_D>
 __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     extern __shared__ float xl[];   // activations of the current pair: max(d, ff) floats, chunk-padded
@@ -170,7 +173,12 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     const int P_ = a.T * a.k;
     // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
     unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
+#ifdef NSLM_FUSED_STAMPS   // development builds: every workgroup's timeline
+#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 8 + (i)] = wall_clock64(); } } while (0)
+    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 8 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+#else
 #define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
+#endif
     STAMP(0);
     load_tables(tab);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
@@ -392,3 +400,9 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
 }
 
 }   // extern "C"
+
+#ifdef NSLM_FUSED_STAMPS
+extern "C" int kc_moe_decode_stamps(unsigned long long* host) {
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 8);
+}
+#endif

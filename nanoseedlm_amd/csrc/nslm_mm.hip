@@ -417,10 +417,10 @@ struct MmRec2 {
 #ifndef NSLM_MM_ABLATE   // development builds only: 1 no activation loads, 2 no decode, 4 no MFMA
 #define NSLM_MM_ABLATE 0
 #endif
-template <int CT, int NCW, int FMT>
+template <int CT, int NCW, int XCH, int FMT>
 __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice wd, const WSlice* ws, const uint16_t* X, float* Y,
                                                    const int32_t* perm, const MmTile* tiles, const int32_t* ntiles) {
-    constexpr int BN = 32 * CT * NCW, NTHR = 64 * (NCW + 4), XCH = 32 / NCW;   // XCH: chunks in a consumer wave's ring (128 KB in all)
+    constexpr int BN = 32 * CT * NCW, NTHR = 64 * (NCW + 4);   // XCH: chunks in a consumer wave's ring
     constexpr bool seedf = FMT == MF_SEED4P4 || FMT == MF_SEED4;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     uint16_t* Xs = smem;                                   // [NCW waves][XCH chunks][32 rows][64 K], slots swizzled
@@ -675,31 +675,32 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         }
     MM_WG_STAMP(0, 3);
 }
-constexpr size_t mm_stream_lds() { return (size_t) (32 * XCHUNK + 2 * BM * LDW2) * sizeof(uint16_t); }
+template <int NCW, int XCH>
+constexpr size_t mm_stream_lds() { return (size_t) (NCW * XCH * XCHUNK + 2 * BM * LDW2) * sizeof(uint16_t); }
 // the streamed kernel takes BF16 activations in 16-byte aligned rows, one BF16 term per weight, K in whole weight steps
 // (xrows > 0: the row count, for the variants that address rows by 32-bit byte offsets)
 bool stream_ok(int fmt, int K, int xs, const void* x, long long xrows) {
     const bool exact = g_seed_exact && (fmt == MF_SEED4 || fmt == MF_SEED4P4);
     return !exact && K % WK == 0 && xs % 8 == 0 && ((uintptr_t) x & 15u) == 0 && (xrows * xs + K) * 2 < (1ll << 32);
 }
-template <int CT, int NCW, int FMT>
+template <int CT, int NCW, int XCH, int FMT>
 void launch_mm_stream_f(hipStream_t st, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
                         const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
-    const size_t lds = mm_stream_lds();
-    auto kern = k_mm_stream<CT, NCW, FMT>;
+    const size_t lds = mm_stream_lds<NCW, XCH>();
+    auto kern = k_mm_stream<CT, NCW, XCH, FMT>;
     allow_big_lds(kern, lds);
     hipLaunchKernelGGL(kern, grid, dim3(64 * (NCW + 4)), lds, st, a, wd, ws, (const uint16_t*) X, Y, perm, tiles, ntiles);
     host_note_launch();
 }
-template <int CT, int NCW>
+template <int CT, int NCW, int XCH>
 void launch_mm_stream(hipStream_t st, int fmt, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
                       const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
     switch (fmt) {
-        case MF_SEED4P4: launch_mm_stream_f<CT, NCW, MF_SEED4P4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
-        case MF_SEED4: launch_mm_stream_f<CT, NCW, MF_SEED4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
-        case MF_BF16: launch_mm_stream_f<CT, NCW, MF_BF16>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
-        case MF_Q8: launch_mm_stream_f<CT, NCW, MF_Q8>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
-        default: launch_mm_stream_f<CT, NCW, MF_Q4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_SEED4P4: launch_mm_stream_f<CT, NCW, XCH, MF_SEED4P4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_SEED4: launch_mm_stream_f<CT, NCW, XCH, MF_SEED4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_BF16: launch_mm_stream_f<CT, NCW, XCH, MF_BF16>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        case MF_Q8: launch_mm_stream_f<CT, NCW, XCH, MF_Q8>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
+        default: launch_mm_stream_f<CT, NCW, XCH, MF_Q4>(st, a, wd, ws, X, Y, perm, tiles, ntiles, grid); break;
     }
 }
 
@@ -709,9 +710,9 @@ void mm_dense(hipStream_t st, int fmt, WSlice w, int K, int R, const void* x, in
     MmArgs a = {K, R, T, xs, ys, 1, add, host_store_f32()};
     const unsigned gx = (unsigned) (R + BM - 1) / BM;
     if (PACKED && stream_ok(fmt, K, xs, x, T)) {
-        if (T > 256) launch_mm_stream<2, 8>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
-        else if (T > 128) launch_mm_stream<2, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
-        else launch_mm_stream<1, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
+        if (T > 256) launch_mm_stream<2, 8, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
+        else if (T > 128) launch_mm_stream<2, 4, 8>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
+        else launch_mm_stream<1, 4, 8>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, 1));
         return;
     }
     if (T > 256) launch_mm<4, PACKED>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
@@ -725,7 +726,8 @@ void mm_grouped(hipStream_t st, int fmt, const WSlice* ws, int K, int R, const v
     MmArgs a = {K, R, 0, xs, ys, xdiv, 0, host_store_f32()};
     WSlice none = {};
     if (PACKED && stream_ok(fmt, K, xs, x, 0)) {
-        launch_mm_stream<1, 4>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
+        // grouped tiles are mostly a few pairs of one expert: decode-bound, so a short ring buys two workgroups a CU
+        launch_mm_stream<1, 4, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
         return;
     }
     launch_mm<1, PACKED>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
