@@ -202,6 +202,146 @@ __global__ void __launch_bounds__(256) k_mv_any(int fmt, MvArgs a) {
     }
 }
 
+// ---- BF16 / Q8 / Q4 rows: HBM-bound, so the point is bytes in flight -------------------------------------------------------
+// Same arithmetic and lane assignment as k_mv_any (lane l owns blocks l, l + 64, ...; an FMA chain per block; the wave's
+// xor-shuffle sum), hence the same bits - but the activations are staged once per workgroup in LDS instead of being
+// re-read from global memory for every row, a block's weights arrive as one 16 / 8 / 4-byte load, a wave walks its rows
+// with a grid stride and keeps the loads of four blocks in flight, and many small workgroups share a CU.
+template <int FMT>
+struct WideRaw {
+    uint4 q;         // BF16: 8 weights; Q8: q.xy; Q4: q.x
+    uint32_t s, b;   // Q8 / Q4: the group's scale and bias bits
+};
+// al: the slice's weight words are 16-byte aligned; otherwise the same words by 2- and 4-byte loads
+template <int FMT>
+__device__ __forceinline__ WideRaw<FMT> wide_load(const WSlice& w, int r, int K, int j, bool al) {
+    WideRaw<FMT> v;
+    const size_t e0 = (size_t) r * K + (size_t) j * 8;
+    if (FMT == MF_BF16) {
+        if (al) {
+            v.q = ldg16(gp<uint16_t>(w.p[0]) + e0);
+        } else {
+            const NSLM_GLOBAL uint16_t* p = gp<uint16_t>(w.p[0]) + e0;
+            v.q = make_uint4(p[0] | (uint32_t) p[1] << 16, p[2] | (uint32_t) p[3] << 16, p[4] | (uint32_t) p[5] << 16,
+                             p[6] | (uint32_t) p[7] << 16);
+        }
+    } else {
+        const size_t gi = e0 >> group_shift(w);
+        v.s = gp<uint16_t>(w.p[1])[gi];
+        v.b = gp<uint16_t>(w.p[2])[gi];
+        if (FMT == MF_Q8) {
+            if (al) {
+                const uint2 q = ldg8(gp<uint8_t>(w.p[0]) + e0);
+                v.q = make_uint4(q.x, q.y, 0, 0);
+            } else {
+                const NSLM_GLOBAL uint8_t* p = gp<uint8_t>(w.p[0]) + e0;
+                v.q = make_uint4(p[0] | (uint32_t) p[1] << 8 | (uint32_t) p[2] << 16 | (uint32_t) p[3] << 24,
+                                 p[4] | (uint32_t) p[5] << 8 | (uint32_t) p[6] << 16 | (uint32_t) p[7] << 24, 0, 0);
+            }
+        } else {
+            if (al) {
+                v.q = make_uint4(gp<uint32_t>(w.p[0])[e0 / 8], 0, 0, 0);
+            } else {
+                const NSLM_GLOBAL uint8_t* p = gp<uint8_t>(w.p[0]) + e0 / 2;
+                v.q = make_uint4(p[0] | (uint32_t) p[1] << 8 | (uint32_t) p[2] << 16 | (uint32_t) p[3] << 24, 0, 0, 0);
+            }
+        }
+    }
+    return v;
+}
+// BF16 / Q8 as their BF16 values, Q4 in the matvec form s q + b unrounded: block_weights' values
+template <int FMT>
+__device__ __forceinline__ void wide_weights(const WideRaw<FMT>& v, float (&o)[8]) {
+    if (FMT == MF_BF16) {
+        const uint32_t u[4] = {v.q.x, v.q.y, v.q.z, v.q.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(u[i] << 16); o[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u); }
+    } else {
+        const float s = bf(v.s), b = bf(v.b);
+        if (FMT == MF_Q8) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) o[c] = bfr(s * (float) (((c < 4 ? v.q.x : v.q.y) >> (8 * (c & 3))) & 255u) + b);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) o[c] = s * (float) ((v.q.x >> (4 * c)) & 15u) + b;
+        }
+    }
+}
+__device__ __forceinline__ float wide_dot(const float (&w)[8], const float* xb) {
+    const float4 x0 = *(const float4*) xb, x1 = *(const float4*) (xb + 4);
+    float d = w[0] * x0.x;
+    d = fmaf(w[1], x0.y, d);
+    d = fmaf(w[2], x0.z, d);
+    d = fmaf(w[3], x0.w, d);
+    d = fmaf(w[4], x1.x, d);
+    d = fmaf(w[5], x1.y, d);
+    d = fmaf(w[6], x1.z, d);
+    return fmaf(w[7], x1.w, d);
+}
+template <int FMT, int MODE>
+__global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float xw[];   // [nt][K]
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int pair = MODE == DENSE ? 0 : (int) blockIdx.y;
+    WSlice wA = a.wd, wB = a.wd;
+    if (MODE != DENSE) {
+        const int sl = a.sel[pair];
+        wA = a.ws[sl];
+        if (MODE == GATEUP) wB = a.wu[sl];
+    }
+    const float* xrow = a.x + (size_t) (MODE == DENSE ? 0 : pair / a.xdiv) * a.xs;
+    const int nbk = a.K / 8, nt = MODE == DENSE ? a.nt : 1;
+    const bool alA = ((uintptr_t) wA.p[0] & 15u) == 0, alB = ((uintptr_t) wB.p[0] & 15u) == 0;
+    for (int t = 0; t < nt; ++t)
+        for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[(size_t) t * (a.K / 4) + i] = ((const float4*) (xrow + (size_t) t * a.xs))[i];
+    __syncthreads();
+    for (int r = (int) blockIdx.x * 4 + wv; r < a.R; r += (int) gridDim.x * 4) {
+        float acc[MV_MAXT], accu = 0.0f;
+#pragma unroll
+        for (int t = 0; t < MV_MAXT; ++t) acc[t] = 0.0f;
+        for (int j0 = lane; j0 < nbk; j0 += 256) {   // four blocks' loads in flight, then their arithmetic in block order
+            WideRaw<FMT> ra[4], rb[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + 64 * u;
+                if (j < nbk) {
+                    ra[u] = wide_load<FMT>(wA, r, a.K, j, alA);
+                    if (MODE == GATEUP) rb[u] = wide_load<FMT>(wB, r, a.K, j, alB);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + 64 * u;
+                if (j >= nbk) break;
+                float w[8];
+                wide_weights<FMT>(ra[u], w);
+#pragma unroll
+                for (int t = 0; t < MV_MAXT; ++t) {
+                    if (t >= nt) break;
+                    acc[t] = fmaf(wide_dot(w, xw + (size_t) t * a.K + (size_t) j * 8), 1.0f, acc[t]);
+                }
+                if (MODE == GATEUP) {
+                    wide_weights<FMT>(rb[u], w);
+                    accu = fmaf(wide_dot(w, xw + (size_t) j * 8), 1.0f, accu);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MV_MAXT; ++t) {
+            if (t >= nt) break;
+            float s = acc[t];
+            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            if (MODE == GATEUP) {
+                float u = accu;
+                for (int o = 32; o > 0; o >>= 1) u += __shfl_xor(u, o);
+                if (lane == 0) a.y[(size_t) pair * a.ys + r] = a.f32out ? (s / (1.0f + expf(-s))) * u : bfr(silu_bf(bfr(s)) * bfr(u));
+            } else if (lane == 0) {
+                store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + r, s, a.add, a.f32out);
+            }
+        }
+    }
+}
+
 // ---- host side ----------------------------------------------------------------------------------------------------------
 bool aligned16(const void* p) { return ((uintptr_t) p & 15u) == 0; }
 
@@ -267,6 +407,30 @@ void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 g
     else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds);
 }
 
+// the wide path: BF16 / Q8 / Q4, whole blocks, 16-byte aligned activations and weights, staged activations within LDS
+bool wide_ok(int fmt, int K, const void* x, int xs, int nt) {
+    return (fmt == MF_BF16 || fmt == MF_Q8 || fmt == MF_Q4) && K % 8 == 0 && ((uintptr_t) x & 15u) == 0 && xs % 4 == 0 &&
+           (size_t) nt * K * sizeof(float) <= 128 * 1024;
+}
+template <int MODE>
+void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
+    const size_t lds = (size_t) (MODE == DENSE ? a.nt : 1) * a.K * sizeof(float);
+    // about 8 small workgroups a CU when the rows allow it; a wave then walks its rows with a grid stride
+    int gx = (a.R + 3) / 4;
+    const int cap = (8 * cu_count() + ny - 1) / ny;
+    if (gx > cap) gx = cap < 1 ? 1 : cap;
+    const dim3 grid((unsigned) gx, (unsigned) ny);
+#define NSLM_WIDE(F)                                                                         \
+    do {                                                                                     \
+        if (lds > 48 * 1024) allow_big_lds(k_mv_wide<F, MODE>);                              \
+        hipLaunchKernelGGL((k_mv_wide<F, MODE>), grid, dim3(256), lds, st, a);               \
+    } while (0)
+    if (fmt == MF_BF16) NSLM_WIDE(MF_BF16);
+    else if (fmt == MF_Q8) NSLM_WIDE(MF_Q8);
+    else NSLM_WIDE(MF_Q4);
+#undef NSLM_WIDE
+}
+
 void note_launch() { nslm::host_note_launch(); }
 
 #define MV_TG 4   // tokens per pass of the multi-token fast path (activations staged in LDS)
@@ -318,7 +482,8 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         return;
     }
     a.nt = T;
-    hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, a);
+    if (T <= MV_MAXT && wide_ok(fmt, K, x, xs, T)) launch_wide<DENSE>(st, fmt, a, 1);
+    else hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, a);
     note_launch();
 }
 
@@ -340,7 +505,8 @@ void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const flo
         note_launch();
         return;
     }
-    hipLaunchKernelGGL(k_mv_any<GATHER>, dim3((unsigned) (R + 3) / 4, (unsigned) P), dim3(256), 0, st, fmt, a);
+    if (wide_ok(fmt, K, x, xs, 1)) launch_wide<GATHER>(st, fmt, a, P);
+    else hipLaunchKernelGGL(k_mv_any<GATHER>, dim3((unsigned) (R + 3) / 4, (unsigned) P), dim3(256), 0, st, fmt, a);
     note_launch();
 }
 
@@ -362,7 +528,8 @@ void kc_mv_gu(kc_stream_t s, int fmt, const WSlice* wg, const WSlice* wu, int K,
         note_launch();
         return;
     }
-    hipLaunchKernelGGL(k_mv_any<GATEUP>, dim3((unsigned) (R + 3) / 4, (unsigned) P), dim3(256), 0, st, fmt, a);
+    if (wide_ok(fmt, K, x, xs, 1)) launch_wide<GATEUP>(st, fmt, a, P);
+    else hipLaunchKernelGGL(k_mv_any<GATEUP>, dim3((unsigned) (R + 3) / 4, (unsigned) P), dim3(256), 0, st, fmt, a);
     note_launch();
 }
 
