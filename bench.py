@@ -32,6 +32,15 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
+def traffic_of(workload):
+    """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 --pmc summary (or None)."""
+    try:
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")) as f:
+            return json.load(f).get(workload, {}).get("hbm_bytes_per_launch")
+    except OSError:
+        return None
+
+
 def moe_workload(name, steps, warmup, n_layers, no_graph):
     from nanoseedlm_amd import backend, moe, packs
     cfgs = {"c2": dict(E=128, k=8, d=2048, ff=768, fmt=packs.MF_SEED4P4), "c3": dict(E=64, k=4, d=2880, ff=2880, fmt=packs.MF_SEED4)}
@@ -120,8 +129,10 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
                     achieved=kbytes / kms / 1e6, frac=kbytes / kms / 1e6 / HBM_PEAK_GBS)
         # The timed step is ONE launch of the persistent decode kernel (router, top-k, gate + up + SwiGLU, down, combine),
         # so that kernel is the dominant one: its algorithmic bytes are the step's, its duration the step's event time.
+        # Its launch duration is the step's event time: HIP events over the timed region on the launch stream (launches are
+        # queued back to back, so there is no gap between them unless the step is wrapped in a graph).
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=None, kernel="k_moe_decode (one launch per step)",
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=traffic_of(name), kernel="k_moe_decode (one launch per step)",
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part)
         ind.free(); A.free()
     else:
@@ -197,7 +208,7 @@ def dense_workload(name, steps, warmup):
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
     else:
         res["roofline"] = dict(bound="mfma", achieved=flops / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                               frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, traffic=None, kernel="k_mm_stream<2, 8> (BF16 activations, 512-token tile)",
+                               frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, traffic=traffic_of(name), kernel="k_mm_stream<2, 8> (BF16 activations, 512-token tile)",
                                launch_us=ms * 1e3, algorithmic_flops=flops)
     res["config"] = {"workload": desc, "launch": "stream"}
     res["cpu_sample"] = sample
@@ -268,14 +279,21 @@ def main():
     ap.add_argument("--workload", default="c2b1")
     ap.add_argument("--layers", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="plain stream launches even for multi-launch steps")
+    ap.add_argument("--graph", action="store_true", help="one hipGraph per step even when the step is a single launch")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="after the workload, run 20 device-to-device copies of this size: a copy kernel of known traffic "
+                         "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build measures one GPU (one process, one MI355X, no collectives); run with --gpus 1")
     from nanoseedlm_amd import backend
     backend.require_gpu()
     if a.workload[:2] in ("c2", "c3"):
-        r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph)
+        # A decode step of up to 8 tokens is ONE kernel launch: a graph around it only adds its launch gap.  Batched steps
+        # (bucket + grouped GEMMs + glue, about ten launches) are captured into one graph per step.
+        single = int(a.workload[3:]) <= 8
+        r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or (single and not a.graph))
     else:
         r = dense_workload(a.workload, a.steps, a.warmup)
     gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6
@@ -288,6 +306,14 @@ def main():
         "roofline": r["roofline"],
     }
     line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(r["cpu_sample"])
+    if a.calibrate_copy > 0:
+        from nanoseedlm_amd import moe
+        n = a.calibrate_copy << 20
+        src, dst = moe.DevBuf(n), moe.DevBuf(n)
+        for _ in range(20):
+            backend.check(backend.hip().nh_memcpy_d2d(dst.ptr, src.ptr, C.c_size_t(n)), "nh_memcpy_d2d")
+        moe.device_sync()
+        src.free(); dst.free()
     print(json.dumps(line))
 
 

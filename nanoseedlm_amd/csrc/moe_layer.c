@@ -198,8 +198,14 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         memset(&qc, 0, sizeof qc);
         qc.n_exp = E;
         qc.top_k = k;
-        if (T <= MV_MAXT) kc_mv(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
-        else kc_mm(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+        if (T <= MV_MAXT) {
+            kc_mv(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+        } else if (d % 8 == 0 && ff % 8 == 0) {   /* the batched path's BF16 view of xn, made once and used three times */
+            kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);
+            kc_mm_packed(s, MF_BF16, rw, d, E, m->px, d, m->logit, E, T, 0, NULL);
+        } else {
+            kc_mm(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+        }
         kq4_route(s, &qc, m->logit, m->ind, m->wt, T);
     } else {
         RouterArgs ra = {d, E, k, d / 2, c->route_scale};
@@ -218,7 +224,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         const int packed = d % 8 == 0 && ff % 8 == 0;
         kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
         if (packed) {
-            kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);
+            if (c->router != NSLM_ROUTE_SOFTMAX) kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);   /* else: made for the router */
             kc_mm_grouped_packed(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
             kc_mm_grouped_packed(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
             kc_swiglu(s, m->G, m->U, m->A, P * ff);
