@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """bench.py - the SeedLM decode-in-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1|c3b16] [--no-cpu]
 
 A step is one pass of the workload over one batch of seeded synthetic input already resident in HBM:
   c2b1 (default; the configuration the metric is quoted on): one MoE decode layer step at batch 1 - 128 experts seeded
@@ -11,7 +11,8 @@ A step is one pass of the workload over one batch of seeded synthetic input alre
   c2b8 / c2b32: the same at 8 and 32 tokens (32: grouping + grouped MFMA GEMMs).
   c0:   dense GEMV, W 4096x4096 P=4, batch 1, rotating over 64 matrices (604 MB).
   c1:   prefill GEMM, W 14336x4096 P=4, X bf16 [512 x 4096].
-  c3b1: 64 experts P=3 top-4, hidden 2880, intermediate 2880, batch 1.
+  c3b1 / c3b16: the mixed-format layer - 64 experts P=3 top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880
+        Q4-g64 projections (q, k, v, o and the shared expert's gate / up / down) - at batch 1 and 16.
 Prints ONE JSON line: value = effective GB/s of compressed weight bytes (whole job), with the dominant kernel's roofline
 (timed live with HIP events on the launch stream) and the CPU baseline (the reference's own lib_cpu_seed4 when the
 compiled reference is present, else this repository's restatement) on a bounded sample of the same workload."""
@@ -41,6 +42,61 @@ def traffic_of(workload):
         return None
 
 
+class Q4Projections:
+    """Config 3's affine-int4 side of the layer: q / k / v / o and the shared expert's gate / up / down, each d x d, Q4
+    group 64 (BF16 scale ~U(0.005, 0.02), zero point uniform [0, 15] stored as bias = -z * scale).  BASELINE gives no
+    shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs up to 8 tokens, the packed
+    MFMA GEMM above (as the reference's enc_dense / enc_dense_packed choose, engine/mova_cuda.c:1020-1028)."""
+
+    def __init__(self, rng, n_layers, d, T):
+        from nanoseedlm_amd import backend, moe, packs
+        self.L, self.d, self.T, self.keep = backend.hip(), d, T, []
+        self.layers = []
+        for _ in range(n_layers):
+            pk = packs.affine(rng, 7, d, d, bits=4, group=64)
+            bufs = [moe.DevBuf.from_array(pk[k]) for k in ("words", "scales", "biases")]
+            self.keep += bufs
+            arr = (backend.WSlice * 7)()
+            for i in range(7):
+                arr[i].p[0] = bufs[0].ptr.value + i * d * d // 2
+                arr[i].p[1] = bufs[1].ptr.value + i * d * (d // 64) * 2
+                arr[i].p[2] = bufs[2].ptr.value + i * d * (d // 64) * 2
+                arr[i].gs = 6
+            tab = moe.DevBuf(C.sizeof(arr))
+            backend.check(self.L.nh_memcpy_h2d(tab.ptr, arr, C.c_size_t(C.sizeof(arr))), "nh_memcpy_h2d")
+            self.keep.append(tab)
+            self.layers.append((arr, tab))
+        self.bytes_per_layer = 7 * (d * d // 2 + 2 * d * (d // 64) * 2)
+        f = lambda n: moe.DevBuf(4 * n)
+        self.q, self.kk, self.v, self.o, self.a, self.g, self.u, self.sh = (f(T * d) for _ in range(8))
+        self.px, self.pa = moe.DevBuf(2 * T * d), moe.DevBuf(2 * T * d)
+        self.sel0 = moe.DevBuf.from_array(np.zeros(max(T, 1), dtype=np.int32))
+
+    def run(self, stream, layer, x_ptr):
+        from nanoseedlm_amd import packs
+        L, d, T, Q4 = self.L, self.d, self.T, packs.MF_Q4
+        arr, tab = self.layers[layer]
+        if T <= 8:
+            for i, y in enumerate((self.q, self.kk, self.v)):
+                L.kc_mv(stream, Q4, arr[i], d, d, x_ptr, d, y.ptr, d, T, 0, None)
+            L.kc_mv(stream, Q4, arr[3], d, d, self.q.ptr, d, self.o.ptr, d, T, 0, None)
+            # shared expert: the gather entry points with every pair on slice 0 (as engine/qwen4_cuda.c:1029 does)
+            L.kc_mv_gu(stream, Q4, tab.at(4 * C.sizeof(arr[0])), tab.at(5 * C.sizeof(arr[0])), d, d, x_ptr, d, self.a.ptr, d,
+                       self.sel0.ptr, T, 1, None)
+            L.kc_mv(stream, Q4, arr[6], d, d, self.a.ptr, d, self.sh.ptr, d, T, 0, None)
+        else:
+            L.kc_pack_input_bf16(stream, x_ptr, self.px.ptr, C.c_size_t(T * d))
+            for i, y in enumerate((self.q, self.kk, self.v)):
+                L.kc_mm_packed(stream, Q4, arr[i], d, d, self.px.ptr, d, y.ptr, d, T, 0, None)
+            L.kc_pack_input_bf16(stream, self.q.ptr, self.pa.ptr, C.c_size_t(T * d))
+            L.kc_mm_packed(stream, Q4, arr[3], d, d, self.pa.ptr, d, self.o.ptr, d, T, 0, None)
+            L.kc_mm_packed(stream, Q4, arr[4], d, d, self.px.ptr, d, self.g.ptr, d, T, 0, None)
+            L.kc_mm_packed(stream, Q4, arr[5], d, d, self.px.ptr, d, self.u.ptr, d, T, 0, None)
+            L.kc_swiglu(stream, self.g.ptr, self.u.ptr, self.a.ptr, T * d)
+            L.kc_pack_input_bf16(stream, self.a.ptr, self.pa.ptr, C.c_size_t(T * d))
+            L.kc_mm_packed(stream, Q4, arr[6], d, d, self.pa.ptr, d, self.sh.ptr, d, T, 0, None)
+
+
 def moe_workload(name, steps, warmup, n_layers, no_graph):
     from nanoseedlm_amd import backend, moe, packs
     cfgs = {"c2": dict(E=128, k=8, d=2048, ff=768, fmt=packs.MF_SEED4P4), "c3": dict(E=64, k=4, d=2880, ff=2880, fmt=packs.MF_SEED4)}
@@ -56,6 +112,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         st.set_layer(l, gate, up, down, rw)
         del gate, up, down
     st.finalize()
+    q4 = Q4Projections(rng, n_layers, d, T) if name[:2] == "c3" else None
     NX = 16
     xs = [moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))) for _ in range(NX)]
     out = moe.DevBuf(4 * T * d)
@@ -65,8 +122,21 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     if not no_graph:
         for l, xi in combos[:2]:
             st.step(stream, l, xs[xi].ptr, T, out.ptr)          # warm every kernel before capture
+            if q4:
+                q4.run(stream, l, xs[xi].ptr)
         moe.device_sync()
-        graphs = [st.graph_of_step(stream, l, xs[xi].ptr, T, out.ptr) for l, xi in combos]
+
+        def capture(l, xi):
+            if not q4:
+                return st.graph_of_step(stream, l, xs[xi].ptr, T, out.ptr)
+            backend.check(st.L.nslm_graph_begin(stream), "nslm_graph_begin")
+            st.step(stream, l, xs[xi].ptr, T, out.ptr)
+            q4.run(stream, l, xs[xi].ptr)
+            g = C.c_void_p(st.L.nslm_graph_end(stream))
+            if not g:
+                raise RuntimeError("graph capture failed")
+            return g
+        graphs = [capture(l, xi) for l, xi in combos]
 
     def run(i):
         l, xi = combos[i % len(combos)]
@@ -74,6 +144,8 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
             st.launch(graphs[i % len(combos)], stream)
         else:
             st.step(stream, l, xs[xi].ptr, T, out.ptr)
+            if q4:
+                q4.run(stream, l, xs[xi].ptr)
 
     for i in range(warmup):
         run(i)
@@ -97,9 +169,9 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         ind, _ = st.last_routing(T)
         uniq.append(len(set(ind.reshape(-1).tolist())))
     eb = st.expert_bytes()
-    bytes_step = float(np.mean(uniq)) * eb + E * d * 2
+    bytes_step = float(np.mean(uniq)) * eb + E * d * 2 + (q4.bytes_per_layer if q4 else 0)
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T,
-               flops_per_step=2.0 * T * k * 3 * d * ff)
+               flops_per_step=2.0 * T * k * 3 * d * ff + (2.0 * T * 7 * d * d if q4 else 0.0))
 
     # dominant kernel alone, timed with events on its stream
     P = T * k
@@ -143,7 +215,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
                                kernel="k_mm_stream<1, 4, 3> grouped (three launches of the step, with its glue kernels)",
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
     desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",
-            "c3": "C3 MoE decode layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880"}[name[:2]]
+            "c3": "C3 mixed-format layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880 Q4-g64 projections (q, k, v, o, shared gate / up / down)"}[name[:2]]
     res["config"] = {"workload": f"{desc}, batch {T}", "layers_rotated": n_layers, "inputs_rotated": NX,
                      "launch": "stream" if no_graph else "hipGraph per step"}
     res["cpu_sample"] = dict(shapes=[(ff, d), (ff, d), (d, ff)], reps=k, fmt=fmt)
@@ -295,7 +367,7 @@ def main():
     if a.workload[:2] in ("c2", "c3"):
         # A decode step of up to 8 tokens is ONE kernel launch: a graph around it only adds its launch gap.  Batched steps
         # (bucket + grouped GEMMs + glue, about ten launches) are captured into one graph per step.
-        single = int(a.workload[3:]) <= 8
+        single = int(a.workload[3:]) <= 8 and a.workload[:2] == "c2"
         r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or (single and not a.graph))
     else:
         r = dense_workload(a.workload, a.steps, a.warmup)

@@ -353,8 +353,6 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     }
     // the grid must be resident at once: all the device holds, but no more than the work can use
     int grid = (per_cu < 3 ? per_cu : 3) * cu_count();
-    static const char* env = getenv("NSLM_FUSED_WGS_PER_CU");
-    if (env && atoi(env) > 0 && atoi(env) <= per_cu) grid = atoi(env) * cu_count();
     const int items = a.T * a.k * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     if (grid > items) grid = items;
     if (grid < 1) grid = 1;
@@ -394,8 +392,6 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
     a.ntile_d = (d + a.rows_d - 1) / a.rows_d;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
-    static const char* pad = getenv("NSLM_FUSED_LDS");   // experiment: request this much LDS to cap workgroups per CU
-    if (pad && (size_t) atoi(pad) > lds) lds = (size_t) atoi(pad);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
 }
 

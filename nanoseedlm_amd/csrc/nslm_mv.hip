@@ -376,8 +376,6 @@ int pick_rows_per_wg(int V, int rpi, int ny) {
     const int iters = (V + rpi - 1) / rpi;
     const int want = 3 * cu_count();
     int per = (iters * ny + want - 1) / want;
-    static const char* env = getenv("NSLM_MV_ITERS");   // tuning override: iterations per workgroup
-    if (env && atoi(env) > 0) per = atoi(env);
     if (per < 1) per = 1;
     if (per > 64) per = 64;
     return per * rpi;
@@ -401,8 +399,6 @@ void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t l
 }
 template <int MODE, int NT>
 void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds) {
-    static const char* pad = getenv("NSLM_MV_LDS");   // experiment: request this much LDS to cap workgroups per CU
-    if (pad && (size_t) atoi(pad) > lds) lds = (size_t) atoi(pad);
     if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds);
     else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds);
 }
