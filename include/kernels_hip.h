@@ -153,6 +153,22 @@ void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out)
 /* 1: the matvec family stores unrounded f32 instead of BF16-rounded values (for comparison with CPU references that do
  * not round, nslm/lib_cpu_seed4.c).  Process-global like kc_seed_gemm_f32; default 0 = the reference's store. */
 void kc_store_f32(int on);
+/* ---- the small kernels either side of the seed matmuls in a full decode step ------------------------------------------ */
+/* engine/kernels_cuda.h:74-75, engine/kernels_moe.cu:676-692,2302-2304.  x[t][:] = the embedding row ids[t] of w as BF16
+ * values: BF16, Q8, Q4 (bf16(s q + b)) and, as tests/kernel_backend.h:141-142 asks of a backend, seed rows (the BF16-rounded
+ * exact weights).  d % 8 == 0. */
+void kc_embed(kc_stream_t s, int fmt, WSlice w, int d, const int32_t* ids, float* x, int T);
+/* engine/kernels_cuda.h:76-77, engine/kernels_moe.cu:694-713.  Grouped RMSNorm, 2 groups of d / 2:
+ * y = bf16(w * (x * rsqrt(mean_group(x^2) + eps))), w BF16 [d]. */
+void kc_gnorm(kc_stream_t s, int d, float eps, const float* x, const uint16_t* w, float* y, int T);
+/* engine/kernels_qwen4.h:24-25, engine/kernels_qwen4.cu:205-236 (nslm/lib_qwen4_ops.c:11-18).  y[t] = x r (1 + w) per
+ * group of g values of a row of len (g == len: the plain RMSNorm of a full model), f32 weights, no rounding; y may be x. */
+void kq4_norm1p(kc_stream_t s, const float* x, int len, int g, const float* w, float eps, float* y, int T);
+/* engine/kernels_cuda.h:177-178, engine/kernels_moe.cu:2115-2151,2714-2719.  Greedy arg-max of n rows of V logits (ties:
+ * the lowest index), and with its softmax probability 1 / sum exp(l - max). */
+void kc_argmax(kc_stream_t s, const float* logits, int32_t* out, int V, int n);
+void kc_argmax_p(kc_stream_t s, const float* logits, int32_t* out, float* prob, int V, int n);
+
 /* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
  * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same
  * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.

@@ -268,6 +268,49 @@ def kt_q4_combine(D, wt, sh, sg):
     return out
 
 
+def kt_gnorm(x, w_bits, eps):
+    x, w_bits = _c(x, np.float32), _c(w_bits, np.uint16)
+    T, d = x.shape
+    y = np.zeros_like(x)
+    _chk(kt().kt_gnorm(d, C.c_float(eps), _p(x), _p(w_bits), _p(y), T), "kt_gnorm")
+    return y
+
+
+def kt_q4_norm1p(x, g, w, eps):
+    x, w = _c(x, np.float32), _c(w, np.float32)
+    T, ln = x.shape
+    y = np.zeros_like(x)
+    _chk(kt().kt_q4_norm1p(_p(x), ln, g, _p(w), C.c_float(eps), _p(y), T), "kt_q4_norm1p")
+    return y
+
+
+def kt_embed(p, ids):
+    """Rows ids of slice 0 of a BF16 / Q8 / Q4 / seed pack as BF16-valued f32 [n, K]."""
+    ids = _c(ids, np.int32)
+    x = np.zeros((ids.size, p["K"]), dtype=np.float32)
+    if p["fmt"] in (packs.MF_SEED4P4, packs.MF_SEED4):
+        _chk(kt().kt_embed_seed(C.byref(kt_weight(p)), _p(ids), ids.size, _p(x)), "kt_embed_seed")
+    elif p["fmt"] == packs.MF_BF16:
+        E = _c(p["w"][0], np.uint16)
+        _chk(kt().kt_embed(packs.MF_BF16, _p(E), None, None, None, p["R"], p["K"], _p(ids), ids.size, _p(x)), "kt_embed")
+    else:
+        q, s_, b = _c(p["words"][0], np.uint32), _c(p["scales"][0], np.uint16), _c(p["biases"][0], np.uint16)
+        _chk(kt().kt_embed(p["fmt"], None, _p(q), _p(s_), _p(b), p["R"], p["K"], _p(ids), ids.size, _p(x)), "kt_embed")
+    return x
+
+
+def kt_argmax(logits, with_prob=False):
+    logits = _c(logits, np.float32)
+    n, V = logits.shape
+    out = np.zeros(n, dtype=np.int32)
+    if not with_prob:
+        _chk(kt().kt_argmax(_p(logits), V, n, _p(out)), "kt_argmax")
+        return out
+    prob = np.zeros(n, dtype=np.float32)
+    _chk(kt().kt_argmax_p(_p(logits), V, n, _p(out), _p(prob)), "kt_argmax_p")
+    return out, prob
+
+
 def kt_slice_deq(p, s=0):
     out = np.zeros((p["R"], p["K"]), dtype=np.uint16)
     _chk(kt().kt_slice_deq(C.byref(kt_weight(p)), s, _p(out)), "kt_slice_deq")

@@ -53,6 +53,14 @@ int kt_swiglu(const float* g, const float* u, float* a, int n);
 int kt_combine(const float* D, const float* w, const float* shared, float* x, int d, int k, int T);
 int kt_q4_combine(int d, int k, const float* D, const float* wt, const float* sh, const float* sg, int sgld, float* out, int T);
 /* slice `slice` of w decoded to BF16 bits [R][K] (kc_slice_deq) */
+/* the small kernels of a full decode step (tests/kernel_backend.h:51,139-143,155) */
+int kt_gnorm(int d, float eps, const float* x, const uint16_t* w, float* y, int T);
+int kt_q4_norm1p(const float* x, int len, int g, const float* w, float eps, float* y, int T);
+int kt_embed(int fmt, const uint16_t* E, const uint32_t* q8, const uint16_t* s8, const uint16_t* b8, int V, int d,
+             const int32_t* ids, int n, float* x);
+int kt_embed_seed(const KtWeight* w, const int32_t* ids, int n, float* x);   /* 1 for formats this backend lacks */
+int kt_argmax(const float* logits, int V, int n, int32_t* out);
+int kt_argmax_p(const float* logits, int V, int n, int32_t* out, float* prob);   /* ours: kc_argmax_p has no kt_ in the reference */
 int kt_slice_deq(const KtWeight* w, int slice, uint16_t* out);
 /* a SEED4P4 / Q8 / Q4 per-head map [H][O][I] decoded to BF16 (kc_heads_deq); seeds: ebias one per head */
 int kt_heads_deq(int fmt, int H, int O, int I, const void* p0, size_t n0, const void* p1, size_t n1, const int32_t* ebias,

@@ -239,6 +239,58 @@ int kt_q4_combine(int d, int k, const float* D, const float* wt, const float* sh
     if (!g_bad) kq4_moe_combine(0, d, k, dD, dw, ds, dg, sgld, dout, T);
     return done("kq4_moe_combine", out, dout, 4 * (size_t) T * d);
 }
+int kt_gnorm(int d, float eps, const float* x, const uint16_t* w, float* y, int T) {
+    const float* dx = (const float*) dev(x, 4 * (size_t) T * d);
+    const uint16_t* dw = (const uint16_t*) dev(w, 2 * (size_t) d);
+    float* dy = (float*) dev(NULL, 4 * (size_t) T * d);
+    if (!g_bad) kc_gnorm(0, d, eps, dx, dw, dy, T);
+    return done("kc_gnorm", y, dy, 4 * (size_t) T * d);
+}
+int kt_q4_norm1p(const float* x, int len, int g, const float* w, float eps, float* y, int T) {
+    const float* dx = (const float*) dev(x, 4 * (size_t) T * len), *dw = (const float*) dev(w, 4 * (size_t) len);
+    float* dy = (float*) dev(NULL, 4 * (size_t) T * len);
+    if (!g_bad) kq4_norm1p(0, dx, len, g, dw, eps, dy, T);
+    return done("kq4_norm1p", y, dy, 4 * (size_t) T * len);
+}
+int kt_embed(int fmt, const uint16_t* E, const uint32_t* q8, const uint16_t* s8, const uint16_t* b8, int V, int d,
+             const int32_t* ids, int n, float* x) {
+    WSlice w;
+    memset(&w, 0, sizeof w);
+    if (fmt == MF_BF16) {
+        w.p[0] = dev(E, 2 * (size_t) V * d);
+    } else {   /* Q8 (or Q4) with one group per 64 values */
+        const size_t per = fmt == MF_Q8 ? 4 : 8;
+        w.p[0] = dev(q8, 4 * (size_t) V * d / per);
+        w.p[1] = dev(s8, 2 * (size_t) V * d / 64);
+        w.p[2] = dev(b8, 2 * (size_t) V * d / 64);
+    }
+    const int32_t* di = (const int32_t*) dev(ids, 4 * (size_t) n);
+    float* dx = (float*) dev(NULL, 4 * (size_t) n * d);
+    if (!g_bad) kc_embed(0, fmt, w, d, di, dx, n);
+    return done("kc_embed", x, dx, 4 * (size_t) n * d);
+}
+int kt_embed_seed(const KtWeight* w, const int32_t* ids, int n, float* x) {
+    if (w->S > MAXS || (w->fmt != MF_SEED4P4 && w->fmt != MF_SEED4)) return 1;
+    slices(w, g_ws);
+    const int32_t* di = (const int32_t*) dev(ids, 4 * (size_t) n);
+    float* dx = (float*) dev(NULL, 4 * (size_t) n * w->K);
+    if (!g_bad) kc_embed(0, w->fmt, g_ws[0], w->K, di, dx, n);
+    return done("kc_embed", x, dx, 4 * (size_t) n * w->K);
+}
+int kt_argmax(const float* logits, int V, int n, int32_t* out) {
+    const float* dl = (const float*) dev(logits, 4 * (size_t) V * n);
+    int32_t* dout = (int32_t*) dev(NULL, 4 * (size_t) n);
+    if (!g_bad) kc_argmax(0, dl, dout, V, n);
+    return done("kc_argmax", out, dout, 4 * (size_t) n);
+}
+int kt_argmax_p(const float* logits, int V, int n, int32_t* out, float* prob) {
+    const float* dl = (const float*) dev(logits, 4 * (size_t) V * n);
+    int32_t* dout = (int32_t*) dev(NULL, 4 * (size_t) n);
+    float* dp = (float*) dev(NULL, 4 * (size_t) n);
+    if (!g_bad) kc_argmax_p(0, dl, dout, dp, V, n);
+    if (fetch("kc_argmax_p", prob, dp, 4 * (size_t) n)) return -1;
+    return done("kc_argmax_p", out, dout, 4 * (size_t) n);
+}
 int kt_slice_deq(const KtWeight* w, int slice, uint16_t* out) {
     if (w->S > MAXS || slice >= w->S) return -1;
     slices(w, g_ws);

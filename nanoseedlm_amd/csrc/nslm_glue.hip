@@ -1,0 +1,162 @@
+// nslm_glue.hip - the small kernels that sit either side of the seed matmuls in a full decode step: embedding rows,
+// the two RMSNorm forms, greedy arg-max over the vocabulary.  They replace the reference's k_embed, k_gnorm
+// (engine/kernels_moe.cu:676-713), k_argmax (:2115-2151) and k_q4_norm1p (engine/kernels_qwen4.cu:205-236) behind the same
+// launchers.  All of them move a few hundred KB at most per token: what matters is one pass over the data with wide
+// loads, 64-lane reductions and no second kernel.
+#include "nslm_mv_dev.h"
+
+using namespace nslm;
+
+namespace {
+
+// x[t][c] = the BF16 value of weight (ids[t], c): BF16 rows as stored, Q8 / Q4 as bf16(s q + b), seed rows as the
+// BF16-rounded exact weight.  One thread per 8-weight block.
+__global__ void __launch_bounds__(256) k_embed(int fmt, WSlice w, int d, const int32_t* ids, float* x) {
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    const bool seedf = fmt == MF_SEED4P4 || fmt == MF_SEED4;
+    if (seedf) {
+        load_tables(tab);
+        __syncthreads();
+    }
+    const int j = (int) (blockIdx.x * 256 + threadIdx.x), t = (int) blockIdx.y;
+    if (j >= d / 8) return;
+    const int row = ids[t];
+    float o[8], sc;
+    if (fmt == MF_Q4) {   // block_weights gives Q4 in the unrounded matvec form; the embedding is the dequantized value
+        const size_t e0 = (size_t) row * d + (size_t) j * 8, gi = e0 >> group_shift(w);
+        const float s = bf(gp<uint16_t>(w.p[1])[gi]), b = bf(gp<uint16_t>(w.p[2])[gi]);
+        const uint32_t q = gp<uint32_t>(w.p[0])[e0 / 8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o[c] = bfr(s * (float) ((q >> (4 * c)) & 15u) + b);
+        sc = 1.0f;
+    } else {
+        block_weights(fmt, w, tab, row, d, j, o, &sc);
+    }
+    float* xo = x + (size_t) t * d + (size_t) j * 8;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) xo[c] = seedf ? bfr(o[c] * sc) : o[c];
+}
+
+// the sum of v over the workgroup's 256 threads, the same value in every thread
+__device__ __forceinline__ float wg_sum(float v, float* red) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads();   // red may still be read from a previous call
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// One workgroup per (token, group): y = f(x * rsqrt(mean_group(x^2) + eps), w).  The group's values stay in registers
+// between the sum and the scaling when the group is at most 256 * NR long; longer groups read x twice.
+// MODE 0: the MoVA grouped norm, BF16 weights, y = bf16(w * (x * r));  MODE 1: the Qwen form, f32 weights, y = x r (1 + w).
+#define NR 16
+template <int MODE>
+__global__ void __launch_bounds__(256) k_rmsnorm(const float* x, int len, int g, const void* wv, float eps, float* y) {
+    __shared__ float red[4];
+    const int groups = len / g, t = (int) blockIdx.x / groups, a = ((int) blockIdx.x % groups) * g, tid = threadIdx.x;
+    const float* xi = x + (size_t) t * len + a;
+    float* yi = y + (size_t) t * len + a;
+    auto out = [&](int k, float v, float r) {
+        if (MODE == 0) yi[k] = bfr(bf(((const uint16_t*) wv)[a + k]) * (v * r));
+        else yi[k] = v * r * (1.0f + ((const float*) wv)[a + k]);
+    };
+    if (g <= 256 * NR) {
+        float v[NR], ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NR; ++j) {
+            const int k = tid + j * 256;
+            v[j] = k < g ? xi[k] : 0.0f;
+            ss = fmaf(v[j], v[j], ss);
+        }
+        const float r = rsqrtf(wg_sum(ss, red) / (float) g + eps);
+#pragma unroll
+        for (int j = 0; j < NR; ++j)
+            if (tid + j * 256 < g) out(tid + j * 256, v[j], r);
+    } else {
+        float ss = 0.0f;
+        for (int k = tid; k < g; k += 256) ss = fmaf(xi[k], xi[k], ss);
+        const float r = rsqrtf(wg_sum(ss, red) / (float) g + eps);
+        for (int k = tid; k < g; k += 256) out(k, xi[k], r);
+    }
+}
+
+// Greedy arg-max of row t (ties: the lowest index; NaNs never win), optionally with its softmax probability
+// 1 / sum exp(l - max).  One workgroup of 1024 per row, 16-byte loads where the row allows them.
+__device__ __forceinline__ void take(float v, int i, float& best, int& idx) {
+    if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+}
+__global__ void __launch_bounds__(1024) k_argmax(const float* logits, int32_t* out, float* prob, int V) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const int t = (int) blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const float* l = logits + (size_t) t * V;
+    const bool vec = (((uintptr_t) l) & 15u) == 0;
+    const int V4 = vec ? V / 4 : 0;
+    float best = -INFINITY;
+    int idx = V;   // "nothing yet": any real index is lower
+    for (int i = tid; i < V4; i += 1024) {
+        const float4 q = ((const float4*) l)[i];
+        take(q.x, 4 * i, best, idx);
+        take(q.y, 4 * i + 1, best, idx);
+        take(q.z, 4 * i + 2, best, idx);
+        take(q.w, 4 * i + 3, best, idx);
+    }
+    for (int i = 4 * V4 + tid; i < V; i += 1024) take(l[i], i, best, idx);
+    for (int o = 32; o > 0; o >>= 1) take(__shfl_xor(best, o), __shfl_xor(idx, o), best, idx);
+    if (lane == 0) { bv[wv] = best; bi[wv] = idx; }
+    __syncthreads();
+    best = bv[0];
+    idx = bi[0];
+#pragma unroll
+    for (int s = 1; s < 16; ++s) take(bv[s], bi[s], best, idx);
+    if (idx >= V) idx = 0;   // a row of NaNs or -inf: the reference answers 0
+    if (tid == 0) out[t] = idx;
+    if (!prob) return;
+    float s = 0.0f;
+    for (int i = tid; i < V4; i += 1024) {
+        const float4 q = ((const float4*) l)[i];
+        s += __expf(q.x - best) + __expf(q.y - best) + __expf(q.z - best) + __expf(q.w - best);
+    }
+    for (int i = 4 * V4 + tid; i < V; i += 1024) s += __expf(l[i] - best);
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    __syncthreads();   // every thread has read bv
+    if (lane == 0) bv[wv] = s;
+    __syncthreads();
+    if (tid == 0) {
+        float tot = 0.0f;
+        for (int w = 0; w < 16; ++w) tot += bv[w];
+        prob[t] = 1.0f / tot;
+    }
+}
+
+}   // namespace
+
+extern "C" {
+
+void kc_embed(kc_stream_t s, int fmt, WSlice w, int d, const int32_t* ids, float* x, int T) {
+    if (T < 1 || d < 8) return;
+    hipLaunchKernelGGL(k_embed, dim3((unsigned) (d / 8 + 255) / 256, (unsigned) T), dim3(256), 0, (hipStream_t) s, fmt, w, d, ids, x);
+    host_note_launch();
+}
+void kc_gnorm(kc_stream_t s, int d, float eps, const float* x, const uint16_t* w, float* y, int T) {
+    if (T < 1 || d < 2) return;
+    hipLaunchKernelGGL(k_rmsnorm<0>, dim3((unsigned) (2 * T)), dim3(256), 0, (hipStream_t) s, x, d, d / 2, (const void*) w, eps, y);
+    host_note_launch();
+}
+void kq4_norm1p(kc_stream_t s, const float* x, int len, int g, const float* w, float eps, float* y, int T) {
+    if (T < 1 || g < 1 || len < g) return;
+    hipLaunchKernelGGL(k_rmsnorm<1>, dim3((unsigned) (T * (len / g))), dim3(256), 0, (hipStream_t) s, x, len, g, (const void*) w, eps, y);
+    host_note_launch();
+}
+void kc_argmax(kc_stream_t s, const float* logits, int32_t* out, int V, int n) {
+    if (n < 1 || V < 1) return;
+    hipLaunchKernelGGL(k_argmax, dim3((unsigned) n), dim3(1024), 0, (hipStream_t) s, logits, out, (float*) nullptr, V);
+    host_note_launch();
+}
+void kc_argmax_p(kc_stream_t s, const float* logits, int32_t* out, float* prob, int V, int n) {
+    if (n < 1 || V < 1) return;
+    hipLaunchKernelGGL(k_argmax, dim3((unsigned) n), dim3(1024), 0, (hipStream_t) s, logits, out, prob, V);
+    host_note_launch();
+}
+
+}   // extern "C"

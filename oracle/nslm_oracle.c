@@ -20,6 +20,11 @@
  *   or_route_sigmoid / or_topk_sigmoid   brute-force k-round arg-max with ties to the lowest id incl. a many-ties case
  *                        (tests/test_mova_kernels.c:376-445).
  *   or_swiglu / or_moe_combine / or_q4_moe_combine   closed forms recomputed in numpy float64 with BF16 rounding.
+ *   or_gnorm             the reference test's own closed form (tests/test_mova_kernels.c:361-374): per-group double sum, within
+ *                        its close_bf(1e-6) of bf16(w * (x * r)); a constant row has r = 1 / sqrt(c^2 + eps) exactly.
+ *   or_norm1p            compiled reference qwen4_norm1p (live); closed form on a constant row; g == len and g < len.
+ *   or_argmax            the reference test's vector: lg[123456] = lg[200000] = 50 -> 123456, lg[V + 99] = 60 -> 99
+ *                        (tests/test_mova_kernels.c:563-572); prob against numpy's softmax in float64.
  *   or_bucket            host regrouping is the definition (tests/test_qwen4_engine.c:33-61): stable sort by expert.
  *   or_cache_admit       invariants (every selected unit resident afterwards, LRU victim = smallest tick, ties to the
  *                        lowest slot); the reference holds no standalone vector for it.
@@ -490,4 +495,48 @@ int or_cache_admit(int32_t* unit_slot, int32_t* slot_unit, uint32_t* slot_last, 
     }
     free(need);
     return nj;
+}
+
+/* ------------------------------------------------------------------------------------------------------------------ */
+/* the small kernels either side of the matmuls                                                                        */
+
+void or_gnorm(int d, float eps, const float* x, const uint16_t* w, float* y, int T) {
+    const int hw = d / 2;
+    for (int t = 0; t < T; ++t) {
+        const float* xr = x + (size_t) t * d;
+        double a = 0, b = 0;
+        for (int c = 0; c < d; ++c) {
+            if (c < hw) a += (double) xr[c] * xr[c];
+            else b += (double) xr[c] * xr[c];
+        }
+        const float r0 = (float) (1.0 / sqrt(a / hw + eps)), r1 = (float) (1.0 / sqrt(b / hw + eps));
+        for (int c = 0; c < d; ++c) y[(size_t) t * d + c] = or_bfr(or_bf2f(w[c]) * (xr[c] * (c < hw ? r0 : r1)));
+    }
+}
+
+void or_norm1p(const float* x, int len, int g, const float* w, float eps, float* y, int T) {
+    for (int t = 0; t < T; ++t)
+        for (int a = 0; a + g <= len; a += g) {
+            const float* xi = x + (size_t) t * len + a;
+            double ss = 0;
+            for (int k = 0; k < g; ++k) ss += (double) xi[k] * xi[k];
+            const double s = 1.0 / sqrt(ss / g + eps);
+            for (int k = 0; k < g; ++k) y[(size_t) t * len + a + k] = (float) (xi[k] * s * (1.0 + w[a + k]));
+        }
+}
+
+void or_argmax(const float* logits, int V, int n, int32_t* out, double* prob) {
+    for (int t = 0; t < n; ++t) {
+        const float* l = logits + (size_t) t * V;
+        float best = -INFINITY;
+        int idx = 0;
+        for (int i = 0; i < V; ++i)
+            if (l[i] > best) { best = l[i]; idx = i; }   /* strict: the first of equal maxima stays */
+        out[t] = idx;
+        if (prob) {
+            double s = 0;
+            for (int i = 0; i < V; ++i) s += exp((double) l[i] - (double) best);
+            prob[t] = 1.0 / s;
+        }
+    }
 }

@@ -83,6 +83,14 @@ void or_moe_combine(const float* D, const float* w, const float* shared, float* 
 void or_q4_moe_combine(int d, int k, const float* D, const float* wt, const float* sh, const float* sg, int sgld,
                        float* out, int T);
 
+/* ---- the small kernels either side of the matmuls ---- */
+/* grouped RMSNorm, 2 groups (nslm/lib_mova_ref.c:158-168): sums in double, r as float, y = bf16(w * (x * r)) */
+void or_gnorm(int d, float eps, const float* x, const uint16_t* w, float* y, int T);
+/* y = x r (1 + w) per group of g (nslm/lib_qwen4_ops.c:11-18): all in double, one rounding to float */
+void or_norm1p(const float* x, int len, int g, const float* w, float eps, float* y, int T);
+/* greedy arg-max, ties to the lowest index (engine/kernels_moe.cu:2115-2136), and prob = 1 / sum exp(l - max) (:2137-2150) */
+void or_argmax(const float* logits, int V, int n, int32_t* out, double* prob);
+
 /* ---- grouping (engine/kernels_moe.cu:527-573; tests/test_qwen4_engine.c:33-61 host regrouping) ----
  * tiles: int32 quads {slice,start,count,0}; returns the tile count */
 int or_bucket(const int32_t* inds, int count, int n, int bn, int32_t* perm, int32_t* tiles);

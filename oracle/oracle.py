@@ -284,3 +284,32 @@ def cache_admit(unit_slot, slot_unit, slot_last, tick, per_layer, sl, inds, prot
                               C.c_int(per_layer), C.c_int(sl), _p(inds), C.c_int(inds.size), C.c_int(protect_prev),
                               _p(jobs), C.byref(hits), C.byref(misses))
     return jobs[:nj].copy(), hits.value, misses.value
+
+
+def gnorm(x, w_bits, eps):
+    """Grouped RMSNorm (2 groups): x [T, d] f32, w BF16 bits [d]."""
+    x = _c(x, np.float32)
+    w_bits = _c(w_bits, np.uint16)
+    T, d = x.shape
+    y = np.zeros_like(x)
+    lib().or_gnorm(C.c_int(d), C.c_float(eps), _p(x), _p(w_bits), _p(y), C.c_int(T))
+    return y
+
+
+def norm1p(x, g, w, eps):
+    """y = x r (1 + w) per group of g values of each row of x [T, len]."""
+    x = _c(x, np.float32)
+    w = _c(w, np.float32)
+    T, ln = x.shape
+    y = np.zeros_like(x)
+    lib().or_norm1p(_p(x), C.c_int(ln), C.c_int(g), _p(w), C.c_float(eps), _p(y), C.c_int(T))
+    return y
+
+
+def argmax(logits, with_prob=False):
+    logits = _c(logits, np.float32)
+    n, V = logits.shape
+    out = np.zeros(n, dtype=np.int32)
+    prob = np.zeros(n, dtype=np.float64)
+    lib().or_argmax(_p(logits), C.c_int(V), C.c_int(n), _p(out), _p(prob) if with_prob else None)
+    return (out, prob) if with_prob else out

@@ -49,6 +49,8 @@ void ref_qwen4_route(int n_exp, int top_k, const float* logits, int32_t* ind, fl
     qwen4_route(&c, logits, ind, wt);
 }
 
+void ref_norm1p(const float* x, int len, int g, const float* w, float eps, float* y) { qwen4_norm1p(x, len, g, w, eps, y); }
+
 /* the tiled CPU mat-vec / mat-mul as the reference's own bench drives it (harness/nslm-cpu-seed-bench.c:50-75) */
 void* ref_tile4(const uint16_t* seeds, const uint16_t* coefs, const uint8_t* codes, int bias, int rows, int kb) {
     CpuSeed4Tiled* t = (CpuSeed4Tiled*) malloc(sizeof *t);

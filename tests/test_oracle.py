@@ -421,3 +421,70 @@ def test_cache_admit_lru(oracle):
     slot_last = np.zeros(per_layer, dtype=np.uint32)
     jobs, h, m = oracle.cache_admit(unit_slot, slot_unit, slot_last, tick, per_layer, 0, [1, 2, 3])
     assert jobs.size == 0 and (h, m) == (3, 0)
+
+
+def test_gnorm_closed_form(oracle):
+    # tests/test_mova_kernels.c:355-374: per-group double sum, close_bf(1e-6) of bf16(w * (x * r))
+    rng = np.random.default_rng(7)
+    T, d = 3, 256
+    x = packs.round_bf16((rng.standard_normal((T, d)) * 3).astype(np.float32))
+    wb = packs.f32_to_bf16_bits((1 + 0.3 * rng.standard_normal(d)).astype(np.float32))
+    y = oracle.gnorm(x, wb, 1e-6)
+    w = packs.bf16_bits_to_f32(wb).astype(np.float64)
+    for t in range(T):
+        for g in range(2):
+            sl = slice(g * d // 2, (g + 1) * d // 2)
+            r = 1.0 / np.sqrt(np.mean(x[t, sl].astype(np.float64) ** 2) + 1e-6)
+            want = w[sl] * (x[t, sl].astype(np.float64) * r)
+            # one BF16 ulp (2^-8 relative) around the unrounded value, plus the f32 slack of the inner product
+            assert np.all(np.abs(y[t, sl] - want) <= np.abs(want) * (2.0 ** -8 + 1e-6) + 1e-30)
+            assert np.array_equal(y[t, sl], packs.round_bf16(y[t, sl]))           # every output is a BF16 value
+    # a constant row: r = 1 / sqrt(c^2 + eps) exactly, so y = bf16(w * fl(c * fl(r)))
+    c = np.float32(0.5)
+    xc = np.full((1, d), c, dtype=np.float32)
+    r = np.float32(1.0 / np.sqrt(float(c) ** 2 + 1e-6))
+    want = packs.round_bf16((packs.bf16_bits_to_f32(wb) * (c * r)).astype(np.float32))
+    assert np.array_equal(oracle.gnorm(xc, wb, 1e-6)[0], want)
+
+
+def test_norm1p(oracle):
+    rng = np.random.default_rng(8)
+    T, ln = 3, 512
+    x = rng.standard_normal((T, ln)).astype(np.float32)
+    w = (0.1 * rng.standard_normal(ln)).astype(np.float32)
+    for g in (ln, 128):
+        y = oracle.norm1p(x, g, w, 1e-6)
+        xs = x.astype(np.float64).reshape(T, ln // g, g)
+        r = 1.0 / np.sqrt((xs ** 2).mean(-1, keepdims=True) + 1e-6)
+        want = (xs * r).reshape(T, ln) * (1.0 + w.astype(np.float64))
+        assert np.allclose(y, want, rtol=1e-6, atol=0)
+    # a row of ones with w = 0: y = 1 / sqrt(1 + eps)
+    y = oracle.norm1p(np.ones((1, 64), np.float32), 64, np.zeros(64, np.float32), 1e-6)
+    assert np.all(y == np.float32(1.0 / np.sqrt(1.0 + 1e-6)))
+
+
+def test_norm1p_vs_reference(oracle, ref):
+    rng = np.random.default_rng(9)
+    ln = 768
+    x = rng.standard_normal(ln).astype(np.float32)
+    w = (0.2 * rng.standard_normal(ln)).astype(np.float32)
+    for g in (768, 256, 64):
+        y = np.zeros(ln, dtype=np.float32)
+        ref.ref_norm1p(x.ctypes.data_as(C.c_void_p), ln, g, w.ctypes.data_as(C.c_void_p), C.c_float(1e-6), y.ctypes.data_as(C.c_void_p))
+        assert np.array_equal(oracle.norm1p(x[None], g, w, 1e-6)[0].view(np.uint32), y.view(np.uint32))
+
+
+def test_argmax_reference_vector(oracle):
+    # tests/test_mova_kernels.c:563-572: a tie goes to the lowest id
+    rng = np.random.default_rng(10)
+    V = 250624
+    lg = packs.round_bf16((rng.standard_normal((2, V)) * 3).astype(np.float32))
+    lg[0, 123456] = 50
+    lg[0, 200000] = 50
+    lg[1, 99] = 60
+    out, prob = oracle.argmax(lg, with_prob=True)
+    assert out.tolist() == [123456, 99]
+    z = lg.astype(np.float64)
+    want = 1.0 / np.exp(z - z.max(1, keepdims=True)).sum(1)
+    assert np.allclose(prob, want, rtol=1e-12)
+    assert oracle.argmax(np.full((1, 17), -np.inf, dtype=np.float32)).tolist() == [0]
