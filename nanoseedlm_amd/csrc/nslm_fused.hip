@@ -354,6 +354,9 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // the grid must be resident at once: all the device holds, but no more than the work can use
     int grid = (per_cu < 3 ? per_cu : 3) * cu_count();
     const int items = a.T * a.k * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
+    // A phase with a few items more than workgroups would leave stragglers a whole second item long (C2 at one token:
+    // 784 down-row items on 768 workgroups); when the device can hold them, a few extra workgroups cost less.
+    if (items > grid && items <= grid + grid / 8 && items <= per_cu * cu_count()) grid = items;
     if (grid > items) grid = items;
     if (grid < 1) grid = 1;
     a.grid = grid;
@@ -380,12 +383,23 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
     if (!shape_of(d, true, &a.Lg, &a.rpig, &sg) || !shape_of(ff, false, &a.Ld, &a.rpid, &sd)) return -1;
     a.rw = router_w; a.gate = gate; a.up = up; a.down = down; a.x = x; a.out = out; a.logits = logits; a.wt = wt; a.A = A;
     a.D = D; a.ind = ind; a.sync = sync; a.E = n_exp; a.k = top_k; a.d = d; a.ff = ff; a.T = T; a.xs = xs; a.os = os;
-    // iterations per item: as many as keep every workgroup of a full grid busy in that phase, at most 4
+    // Iterations per item (an item = one pair's row tile): the count that gives the busiest workgroup of a full grid the
+    // fewest iterations, an item's set-up priced at a third of an iteration; a few items over the grid count as one round
+    // (the launch adds workgroups for them).
     const int full = 3 * cu_count(), P_ = T * top_k;
     const int it_g = (2 * ff + a.rpig - 1) / a.rpig, it_d = (d + a.rpid - 1) / a.rpid;
-    int per_g = P_ * it_g / full, per_d = P_ * it_d / full;
-    per_g = per_g < 1 ? 1 : per_g > 4 ? 4 : per_g;
-    per_d = per_d < 1 ? 1 : per_d > 4 ? 4 : per_d;
+    auto pick = [&](int iters) {
+        int best = 1;
+        long best_cost = -1;
+        for (int per = 1; per <= 8; ++per) {
+            const long items = (long) P_ * ((iters + per - 1) / per);
+            const long rounds = items <= full + full / 8 ? 1 : (items + full - 1) / full;
+            const long cost = rounds * (3 * per + 1);
+            if (best_cost < 0 || cost < best_cost) { best = per; best_cost = cost; }
+        }
+        return best;
+    };
+    const int per_g = pick(it_g), per_d = pick(it_d);
     a.rows_g = per_g * a.rpig;
     a.ntile_g = (2 * ff + a.rows_g - 1) / a.rows_g;
     a.rows_d = per_d * a.rpid;
