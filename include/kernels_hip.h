@@ -169,6 +169,52 @@ void kq4_norm1p(kc_stream_t s, const float* x, int len, int g, const float* w, f
 void kc_argmax(kc_stream_t s, const float* logits, int32_t* out, int V, int n);
 void kc_argmax_p(kc_stream_t s, const float* logits, int32_t* out, float* prob, int V, int n);
 
+/* ---- decode attention over a latent KV cache (absorbed MLA) ------------------------------------------------------------ */
+/* The KV cache view, engine/kernels_cuda.h:57-72: per layer, positions [0, nv) in segment a and [nv, ...) in segment b
+ * (row 0 of b = position nv).  MLA: k holds the RoPE key, v the latent; BF16 (u16 values), or FP8 (nslm/kvq.h: E4M3 codes
+ * in k / v, one E8M0 scale byte per 32 values in ks / vs).  KV_Q8 and KV_FP4 are not built (the launchers refuse them). */
+enum { KV_BF16 = 0, KV_Q8 = 1, KV_FP8 = 2, KV_FP4 = 3 };
+typedef struct {
+    void* k;
+    void* v;
+    float* ks; /* FP8: the block scale bytes [rows][n / 32] */
+    float* vs;
+} KvSeg;
+typedef struct {
+    KvSeg a, b;
+    int32_t nv, fmt;
+} KvView;
+typedef struct { int pos, kv0; int pad[2]; } RowInfo; /* kv0: the cache row of the sequence slot's position 0 (kernels_moe.metal:86) */
+#define ATT_HD 128
+/* engine/kernels_moe.metal:100-104.  chunk: target keys per split; each row splits its own 0..pos into
+ * min(n_splits, ceil((pos + 1) / chunk)) parts.  pad[0] (ours; the reference leaves it 0): the RoPE key's width, 64 or 128,
+ * 0 = 128 (the reference hard-codes ATT_HD).  pad[2] > 0: at most 32 splits, as the reference's one-pass kernel takes it. */
+typedef struct {
+    int n_head, r, chunk, n_splits;
+    float scale;
+    int pad[3];
+} MlaArgs;
+/* per-head maps, engine/kernels_moe.metal:112-115: y[t][h][o] = W_h[o] . x[t * xs + h * hs ..] */
+typedef struct {
+    int H, O, I, xs, hs, gate;
+    int pad[2];
+} HmvArgs;
+/* engine/kernels_cuda.h:136-142, engine/kernels_moe.cu:1147-1176,2437-2440.  y[t][h][o] = bf16(W_h[o] . x), with g (y's layout)
+ * bf16(that * bf16(softplus_ln2(g))).  W stacked [H][O][I] in fmt; SEED4P4 takes head h's exponent bias from W.p[2][h]. */
+void kc_heads_mv(kc_stream_t s, HmvArgs a, int fmt, WSlice W, const uint32_t* G, const float* x, const float* g, float* y, int T);
+/* engine/kernels_cuda.h:154-156, engine/kernels_moe.cu:1177-1208.  RoPE of the query RoPE parts qr [T][n_head][rope] (in place,
+ * BF16-rounded) and of kr [T][rope] into kv.k; the latent c [T][r] into kv.v, at cache row ri[t].kv0 + ri[t].pos. */
+void kc_mla_rope(kc_stream_t s, MlaArgs a, float* qr, const float* kr, const float* c, KvView kv, const RowInfo* ri,
+                 const float* inv, int T);
+/* engine/kernels_cuda.h:157-161, engine/kernels_moe.cu:1217-1323,2459-2489.  olat[t][h] = bf16(sum_p softmax_p(scale (ql_th .
+ * c_p + qr_th . k_p)) c_p) over p <= pos_t; n_splits > 1 splits the keys (partials in part: T x n_head x n_splits x (r + 2)
+ * floats) and reduces.  r % 8 == 0, r <= 1024. */
+void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part,
+                 float* olat, int T);
+/* engine/kernels_cuda.h:173-176.  y[i] = value i of `rows` cache rows of n values in fmt (KV_BF16 / KV_FP8): the decode the
+ * attention reads, for tests */
+void kc_kv_f32(kc_stream_t s, int fmt, const uint8_t* codes, const uint8_t* scales, int n, int rows, float* y);
+
 /* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
  * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same
  * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.

@@ -18,6 +18,18 @@ class WSlice(C.Structure):
     _fields_ = [("p", C.c_void_p * 4), ("eb", C.c_int32), ("gs", C.c_int32), ("pad", C.c_int32 * 2)]
 
 
+class RowInfo(C.Structure):
+    _fields_ = [("pos", C.c_int), ("kv0", C.c_int), ("pad", C.c_int * 2)]
+
+
+class MlaArgs(C.Structure):
+    _fields_ = [("n_head", C.c_int), ("r", C.c_int), ("chunk", C.c_int), ("n_splits", C.c_int), ("scale", C.c_float),
+                ("pad", C.c_int * 3)]
+
+
+KV_BF16, KV_FP8 = 0, 2
+
+
 class RouterArgs(C.Structure):
     _fields_ = [("d", C.c_int), ("n", C.c_int), ("top_k", C.c_int), ("hw", C.c_int), ("scale", C.c_float)]
 
@@ -309,6 +321,58 @@ def kt_argmax(logits, with_prob=False):
     prob = np.zeros(n, dtype=np.float32)
     _chk(kt().kt_argmax_p(_p(logits), V, n, _p(out), _p(prob)), "kt_argmax_p")
     return out, prob
+
+
+def kt_heads_w(p, H, O, I, x, xs, hs, g=None, ebias=None):
+    """Per-head maps with W = slice 0 of pack p (R = H * O, K = I): y [T, H, O]."""
+    x = _c(x, np.float32)
+    T = x.shape[0]
+    y = np.zeros((T, H, O), dtype=np.float32)
+    gg = _c(g, np.float32) if g is not None else None
+    eb = _c(ebias, np.int32) if ebias is not None else None
+    _chk(kt().kt_heads_w(C.byref(kt_weight(p)), H, O, I, _p(eb) if eb is not None else None, _p(x), xs, hs,
+                         _p(gg) if gg is not None else None, _p(y), T), "kt_heads_w")
+    return y
+
+
+def _ri(pos, kv0):
+    ri = (RowInfo * len(pos))()
+    for i, (a, b) in enumerate(zip(pos, kv0)):
+        ri[i].pos, ri[i].kv0 = int(a), int(b)
+    return ri
+
+
+def kt_mla_rope(n_head, r, rope, fmt, qr, kr, c, cache, pos, kv0, inv):
+    """cache = dict(k, v[, ks, vs]) of npos positions, updated in place; returns the rotated qr."""
+    qr = np.array(qr, dtype=np.float32, copy=True)
+    kr, c, inv = _c(kr, np.float32), _c(c, np.float32), _c(inv, np.float32)
+    T = kr.shape[0]
+    a = MlaArgs(n_head, r, 128, 1, 0.0)
+    a.pad[0] = rope
+    npos = cache["k"].shape[0]
+    _chk(kt().kt_mla_rope_f(a, fmt, _p(qr), _p(kr), _p(c), _p(cache["k"]), _p(cache["v"]), _p(cache["ks"]) if fmt == KV_FP8 else None,
+                            _p(cache["vs"]) if fmt == KV_FP8 else None, npos, _ri(pos, kv0), _p(inv), T), "kt_mla_rope_f")
+    return qr
+
+
+def kt_mla_attn(n_head, r, rope, fmt, ql, qr, cache, pos, kv0, scale, chunk, n_splits, long_from=0):
+    ql, qr = _c(ql, np.float32), _c(qr, np.float32)
+    T = len(pos)
+    a = MlaArgs(n_head, r, chunk, n_splits, scale)
+    a.pad[0], a.pad[2] = rope, long_from
+    npos = cache["k"].shape[0]
+    o = np.zeros((T, n_head, r), dtype=np.float32)
+    _chk(kt().kt_mla_attn_f(a, fmt, _p(ql), _p(qr), _p(cache["k"]), _p(cache["v"]), _p(cache["ks"]) if fmt == KV_FP8 else None,
+                            _p(cache["vs"]) if fmt == KV_FP8 else None, npos, _ri(pos, kv0), _p(o), T), "kt_mla_attn_f")
+    return o
+
+
+def kt_kv_f32(fmt, codes, scales):
+    codes = np.ascontiguousarray(codes)
+    rows, n = codes.shape
+    y = np.zeros((rows, n), dtype=np.float32)
+    _chk(kt().kt_kv_f32(fmt, _p(codes), _p(np.ascontiguousarray(scales)) if scales is not None else None, n, rows, _p(y)), "kt_kv_f32")
+    return y
 
 
 def kt_slice_deq(p, s=0):

@@ -61,6 +61,17 @@ int kt_embed(int fmt, const uint16_t* E, const uint32_t* q8, const uint16_t* s8,
 int kt_embed_seed(const KtWeight* w, const int32_t* ids, int n, float* x);   /* 1 for formats this backend lacks */
 int kt_argmax(const float* logits, int V, int n, int32_t* out);
 int kt_argmax_p(const float* logits, int V, int n, int32_t* out, float* prob);   /* ours: kc_argmax_p has no kt_ in the reference */
+/* MLA decode attention (tests/kernel_backend.h:79-104,123-137).  The reference splits these by format (kt_heads_mv /
+ * kt_heads_q / kt_heads_seed, kt_mla_rope / kt_mla_rope_q, kt_mla_attn / kt_mla_attn_q); here the format is an argument:
+ * per-head maps with W = slice 0 of w (R = H * O, K = I; ebias: a seed map's exponent bias per head, or NULL); caches of
+ * npos positions in fmt KV_BF16 (k, v: u16) or KV_FP8 (k, v: codes, ks, vs: scale bytes), all in one segment. */
+int kt_heads_w(const KtWeight* w, int H, int O, int I, const int32_t* ebias, const float* x, int xs, int hs, const float* g,
+               float* y, int T);
+int kt_mla_rope_f(MlaArgs a, int fmt, float* qr, const float* kr, const float* c, void* k, void* v, void* ks, void* vs, int npos,
+                  const RowInfo* ri, const float* inv, int T);
+int kt_mla_attn_f(MlaArgs a, int fmt, const float* ql, const float* qr, void* k, void* v, void* ks, void* vs, int npos,
+                  const RowInfo* ri, float* olat, int T);
+int kt_kv_f32(int fmt, const uint8_t* codes, const uint8_t* scales, int len, int rows, float* y);
 int kt_slice_deq(const KtWeight* w, int slice, uint16_t* out);
 /* a SEED4P4 / Q8 / Q4 per-head map [H][O][I] decoded to BF16 (kc_heads_deq); seeds: ebias one per head */
 int kt_heads_deq(int fmt, int H, int O, int I, const void* p0, size_t n0, const void* p1, size_t n1, const int32_t* ebias,

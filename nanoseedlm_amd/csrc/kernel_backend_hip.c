@@ -291,6 +291,77 @@ int kt_argmax_p(const float* logits, int V, int n, int32_t* out, float* prob) {
     if (fetch("kc_argmax_p", prob, dp, 4 * (size_t) n)) return -1;
     return done("kc_argmax_p", out, dout, 4 * (size_t) n);
 }
+/* ---- MLA decode attention (tests/kernel_backend.h:79-81,97-104,123-137) ---- */
+int kt_heads_w(const KtWeight* w, int H, int O, int I, const int32_t* ebias, const float* x, int xs, int hs, const float* g,
+               float* y, int T) {
+    /* W stacked [H][O][I] = slice 0 of w with R = H * O, K = I; seed maps: an exponent bias per head */
+    if (w->S > MAXS) return -1;
+    slices(w, g_ws);
+    WSlice W = g_ws[0];
+    if (w->fmt == MF_SEED4P4 && ebias) W.p[2] = dev(ebias, 4 * (size_t) H);
+    else if (w->fmt == MF_SEED4P4) {   /* one bias for every head: the slice's own */
+        int32_t eb[64];
+        if (H > 64) return -1;
+        for (int h = 0; h < H; ++h) eb[h] = g_ws[0].eb;
+        W.p[2] = dev(eb, 4 * (size_t) H);
+    }
+    const size_t xn = (size_t) (T - 1) * xs + (size_t) (H - 1) * hs + I;
+    const float* dx = (const float*) dev(x, 4 * xn);
+    const float* dg = g ? (const float*) dev(g, 4 * (size_t) T * H * O) : NULL;
+    float* dy = (float*) dev(NULL, 4 * (size_t) T * H * O);
+    HmvArgs a = {H, O, I, xs, hs, g != NULL, {0, 0}};
+    if (!g_bad) kc_heads_mv(0, a, w->fmt, W, NULL, dx, dg, dy, T);
+    return done("kc_heads_mv", y, dy, 4 * (size_t) T * H * O);
+}
+/* caches of npos positions: BF16 (Kc / Vc as u16) or FP8 (codes + scale bytes); fmt KV_BF16 / KV_FP8 */
+static KvView mla_view(int fmt, int r, int rope, int npos, void* k, void* v, void* ks, void* vs, void** dk, void** dv, void** dks, void** dvs) {
+    KvView kv;
+    memset(&kv, 0, sizeof kv);
+    const size_t e = fmt == KV_BF16 ? 2 : 1;
+    *dk = dev(k, e * (size_t) npos * rope);
+    *dv = dev(v, e * (size_t) npos * r);
+    *dks = fmt == KV_FP8 ? dev(ks, (size_t) npos * rope / 32) : NULL;
+    *dvs = fmt == KV_FP8 ? dev(vs, (size_t) npos * r / 32) : NULL;
+    kv.a.k = *dk; kv.a.v = *dv; kv.a.ks = (float*) *dks; kv.a.vs = (float*) *dvs;
+    kv.nv = npos;   /* everything in segment a */
+    kv.fmt = fmt;
+    return kv;
+}
+int kt_mla_rope_f(MlaArgs a, int fmt, float* qr, const float* kr, const float* c, void* k, void* v, void* ks, void* vs, int npos,
+                  const RowInfo* ri, const float* inv, int T) {
+    const int rope = a.pad[0] > 0 ? a.pad[0] : ATT_HD;
+    void *dk, *dv, *dks, *dvs;
+    const KvView kv = mla_view(fmt, a.r, rope, npos, k, v, ks, vs, &dk, &dv, &dks, &dvs);
+    float* dq = (float*) dev(qr, 4 * (size_t) T * a.n_head * rope);
+    const float* dkr = (const float*) dev(kr, 4 * (size_t) T * rope), *dc = (const float*) dev(c, 4 * (size_t) T * a.r);
+    const RowInfo* dri = (const RowInfo*) dev(ri, sizeof(RowInfo) * (size_t) T);
+    const float* dinv = (const float*) dev(inv, 4 * (size_t) (rope / 2));
+    if (!g_bad) kc_mla_rope(0, a, dq, dkr, dc, kv, dri, dinv, T);
+    const size_t e = fmt == KV_BF16 ? 2 : 1;
+    if (fetch("kc_mla_rope", k, dk, e * (size_t) npos * rope) || fetch("kc_mla_rope", v, dv, e * (size_t) npos * a.r)) return -1;
+    if (fmt == KV_FP8 && (fetch("kc_mla_rope", ks, dks, (size_t) npos * rope / 32) || fetch("kc_mla_rope", vs, dvs, (size_t) npos * a.r / 32)))
+        return -1;
+    return done("kc_mla_rope", qr, dq, 4 * (size_t) T * a.n_head * rope);
+}
+int kt_mla_attn_f(MlaArgs a, int fmt, const float* ql, const float* qr, void* k, void* v, void* ks, void* vs, int npos,
+                  const RowInfo* ri, float* olat, int T) {
+    const int rope = a.pad[0] > 0 ? a.pad[0] : ATT_HD;
+    void *dk, *dv, *dks, *dvs;
+    const KvView kv = mla_view(fmt, a.r, rope, npos, k, v, ks, vs, &dk, &dv, &dks, &dvs);
+    const float* dql = (const float*) dev(ql, 4 * (size_t) T * a.n_head * a.r), *dqr = (const float*) dev(qr, 4 * (size_t) T * a.n_head * rope);
+    const RowInfo* dri = (const RowInfo*) dev(ri, sizeof(RowInfo) * (size_t) T);
+    float* part = (float*) dev(NULL, 4 * (size_t) T * a.n_head * a.n_splits * (a.r + 2));
+    float* dol = (float*) dev(NULL, 4 * (size_t) T * a.n_head * a.r);
+    if (!g_bad) kc_mla_attn(0, a, dql, dqr, kv, dri, part, dol, T);
+    return done("kc_mla_attn", olat, dol, 4 * (size_t) T * a.n_head * a.r);
+}
+int kt_kv_f32(int fmt, const uint8_t* codes, const uint8_t* scales, int len, int rows, float* y) {
+    const uint8_t* dc = (const uint8_t*) dev(codes, (fmt == KV_BF16 ? 2 : 1) * (size_t) len * rows);
+    const uint8_t* ds = fmt == KV_FP8 ? (const uint8_t*) dev(scales, (size_t) rows * len / 32) : NULL;
+    float* dy = (float*) dev(NULL, 4 * (size_t) len * rows);
+    if (!g_bad) kc_kv_f32(0, fmt, dc, ds, len, rows, dy);
+    return done("kc_kv_f32", y, dy, 4 * (size_t) len * rows);
+}
 int kt_slice_deq(const KtWeight* w, int slice, uint16_t* out) {
     if (w->S > MAXS || slice >= w->S) return -1;
     slices(w, g_ws);

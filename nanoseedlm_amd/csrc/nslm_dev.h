@@ -252,5 +252,6 @@ __device__ __forceinline__ int group_shift(const WSlice& w) { return w.gs ? w.gs
 // process-wide switches and launch-error bookkeeping (defined in nslm_mv.hip)
 int host_store_f32();
 void host_note_launch();
+void host_note_unsupported();   // a launcher refused its arguments: kc_last_error() reports an invalid value
 
 }   // namespace nslm

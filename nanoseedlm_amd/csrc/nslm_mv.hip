@@ -435,6 +435,7 @@ void note_launch() { nslm::host_note_launch(); }
 
 namespace nslm {
 int host_store_f32() { return g_store_f32; }
+void host_note_unsupported() { g_last_error = (int) hipErrorInvalidValue; }
 void host_note_launch() {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) g_last_error = (int) e;

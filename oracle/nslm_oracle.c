@@ -25,6 +25,12 @@
  *   or_norm1p            compiled reference qwen4_norm1p (live); closed form on a constant row; g == len and g < len.
  *   or_argmax            the reference test's vector: lg[123456] = lg[200000] = 50 -> 123456, lg[V + 99] = 60 -> 99
  *                        (tests/test_mova_kernels.c:563-572); prob against numpy's softmax in float64.
+ *   or_e4m3_* / or_fp8_*  every finite E4M3 code round-trips and decodes exactly to BF16, 0x7E = 448, 0x01 = 2^-9, 0xB8 = -1,
+ *                        midpoints go to the even code (tests/test_kvq.c:30-45); the scale is the smallest power of two s
+ *                        with 448 s >= amax (nslm/kvq.h:4-5); bit-compared with the compiled reference's kvq.h (live).
+ *   or_heads_map / or_rope_pair / or_mla_attn   the reference tests' own double-precision forms
+ *                        (tests/test_mova_kernels.c:800-812, 962-979, 1004-1031); softmax of equal scores gives the mean
+ *                        latent; one position gives that position's latent.
  *   or_bucket            host regrouping is the definition (tests/test_qwen4_engine.c:33-61): stable sort by expert.
  *   or_cache_admit       invariants (every selected unit resident afterwards, LRU victim = smallest tick, ties to the
  *                        lowest slot); the reference holds no standalone vector for it.
@@ -539,4 +545,91 @@ void or_argmax(const float* logits, int V, int n, int32_t* out, double* prob) {
             prob[t] = 1.0 / s;
         }
     }
+}
+
+/* ------------------------------------------------------------------------------------------------------------------ */
+/* FP8 KV cache codec (nslm/kvq.h)                                                                                     */
+
+float or_e4m3_dec(uint8_t c) {
+    const int e = (c >> 3) & 15, m = c & 7;
+    const float v = e ? ldexpf(1.0f + (float) m / 8, e - 7) : ldexpf((float) m, -9);
+    return c & 0x80 ? -v : v;
+}
+uint8_t or_e4m3_enc_abs(float a) {
+    if (!(a < 448.0f)) return 0x7E;
+    if (a < 0.015625f) return (uint8_t) rintf(a * 512.0f);
+    int e;
+    const float f = frexpf(a, &e);
+    int E = e - 1, m = (int) rintf((2 * f - 1) * 8);
+    if (m == 8) { ++E; m = 0; }
+    const int c = ((E + 7) << 3) | m;
+    return (uint8_t) (c > 0x7E ? 0x7E : c);
+}
+uint8_t or_fp8_scale(float amax) {
+    if (!(amax > 0)) return 127;
+    int k;
+    frexpf(amax, &k);
+    int e = amax <= ldexpf(448.0f, k - 9) ? k - 9 : k - 8;
+    if (e < -126) e = -126;
+    if (e > 127) e = 127;
+    return (uint8_t) (e + 127);
+}
+void or_fp8_row(const float* x, int n, uint8_t* codes, uint8_t* scales) {
+    for (int b = 0; b < n; b += 32) {
+        float amax = 0;
+        for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(x[b + i]));
+        scales[b / 32] = or_fp8_scale(amax);
+        const int e = (int) scales[b / 32] - 127;
+        for (int i = 0; i < 32; ++i) {
+            const uint8_t c = or_e4m3_enc_abs(ldexpf(fabsf(x[b + i]), -e));
+            codes[b + i] = (uint8_t) (c && x[b + i] < 0 ? c | 0x80 : c);
+        }
+    }
+}
+float or_fp8_get(const uint8_t* codes, const uint8_t* scales, int i) { return ldexpf(or_e4m3_dec(codes[i]), (int) scales[i / 32] - 127); }
+
+/* ------------------------------------------------------------------------------------------------------------------ */
+/* MLA decode attention                                                                                                */
+
+static float or_softplus_gate(float g) {   /* softplus(x, beta = ln 2) in f32, then BF16 */
+    const float gx = g * 0.69314718055994531f;
+    return or_bfr((fmaxf(gx, 0.0f) + logf(1.0f + expf(-fabsf(gx)))) / 0.69314718055994531f);
+}
+void or_heads_map(int H, int O, int I, const float* W, const float* x, int xs, int hs, const float* g, float* y, int T) {
+    for (int t = 0; t < T; ++t)
+        for (int h = 0; h < H; ++h)
+            for (int o = 0; o < O; ++o) {
+                double s = 0;
+                for (int i = 0; i < I; ++i) s += (double) W[((size_t) h * O + o) * I + i] * x[(size_t) t * xs + (size_t) h * hs + i];
+                const size_t yi = ((size_t) t * H + h) * O + o;
+                float v = or_bfr((float) s);
+                if (g) v = or_bfr(v * or_softplus_gate(g[yi]));
+                y[yi] = v;
+            }
+}
+void or_rope_pair(double x0, double x1, int pos, float inv, double* y0, double* y1) {
+    const double th = (double) (float) ((float) pos * inv), cs = cos(th), sn = sin(th);
+    *y0 = x0 * cs - x1 * sn;
+    *y1 = x1 * cs + x0 * sn;
+}
+void or_mla_attn(int r, int rope, double scale, const float* ql, const float* qr, const float* lat, const float* kr, int pos,
+                 float* olat) {
+    double* s = (double*) malloc(sizeof(double) * (size_t) (pos + 1));
+    double* acc = (double*) calloc((size_t) r, sizeof(double));
+    double m = -INFINITY, l = 0;
+    for (int p = 0; p <= pos; ++p) {
+        double v = 0;
+        for (int i = 0; i < r; ++i) v += (double) ql[i] * lat[(size_t) p * r + i];
+        for (int i = 0; i < rope; ++i) v += (double) qr[i] * kr[(size_t) p * rope + i];
+        s[p] = v * scale;
+        if (s[p] > m) m = s[p];
+    }
+    for (int p = 0; p <= pos; ++p) {
+        const double e = exp(s[p] - m);
+        l += e;
+        for (int i = 0; i < r; ++i) acc[i] += e * lat[(size_t) p * r + i];
+    }
+    for (int i = 0; i < r; ++i) olat[i] = or_bfr((float) (acc[i] / l));
+    free(s);
+    free(acc);
 }

@@ -91,6 +91,24 @@ void or_norm1p(const float* x, int len, int g, const float* w, float eps, float*
 /* greedy arg-max, ties to the lowest index (engine/kernels_moe.cu:2115-2136), and prob = 1 / sum exp(l - max) (:2137-2150) */
 void or_argmax(const float* logits, int V, int n, int32_t* out, double* prob);
 
+/* ---- FP8 KV cache codec (nslm/kvq.h:19-34,48-57,70-79,109-111): E4M3 codes, one E8M0 scale byte per 32 values ---- */
+float or_e4m3_dec(uint8_t c);
+uint8_t or_e4m3_enc_abs(float a);              /* a >= 0: round to nearest even, saturated at 448 */
+uint8_t or_fp8_scale(float amax);              /* the smallest 2^e with 448 2^e >= amax, as byte e + 127 */
+void or_fp8_row(const float* x, int n, uint8_t* codes, uint8_t* scales);   /* n a multiple of 32 */
+float or_fp8_get(const uint8_t* codes, const uint8_t* scales, int i);
+
+/* ---- MLA decode attention (nslm/lib_mova_ref.c:280-345; engine/kernels_moe.cu:1147-1323) ---- */
+/* per-head maps y[t][h][o] = bf16(W_h[o] . x[t*xs + h*hs ..]) over exact weights W [H*O][I] given as f32 rows; with g:
+ * bf16(that * bf16(softplus_ln2(g))) (engine/kernels_moe.cu:215-218,1170-1174).  Sums in double. */
+void or_heads_map(int H, int O, int I, const float* W, const float* x, int xs, int hs, const float* g, float* y, int T);
+/* RoPE of pair (p, p + rope/2) at angle (float) pos * inv[p] (engine/kernels_moe.cu:1188-1196), in double */
+void or_rope_pair(double x0, double x1, int pos, float inv, double* y0, double* y1);
+/* latent attention of one (row, head) over positions 0..pos: lat [npos][r], kr [npos][rope] as f32 values; olat[r] =
+ * bf16(sum softmax(scale (ql . c + qr . k)) c), all sums in double */
+void or_mla_attn(int r, int rope, double scale, const float* ql, const float* qr, const float* lat, const float* kr, int pos,
+                 float* olat);
+
 /* ---- grouping (engine/kernels_moe.cu:527-573; tests/test_qwen4_engine.c:33-61 host regrouping) ----
  * tiles: int32 quads {slice,start,count,0}; returns the tile count */
 int or_bucket(const int32_t* inds, int count, int n, int bn, int32_t* perm, int32_t* tiles);

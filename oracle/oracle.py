@@ -313,3 +313,53 @@ def argmax(logits, with_prob=False):
     prob = np.zeros(n, dtype=np.float64)
     lib().or_argmax(_p(logits), C.c_int(V), C.c_int(n), _p(out), _p(prob) if with_prob else None)
     return (out, prob) if with_prob else out
+
+
+def fp8_row(x):
+    """FP8 cache rows of x [rows, n] (n a multiple of 32): codes u8 [rows, n], scales u8 [rows, n / 32]."""
+    x = _c(x, np.float32)
+    rows, n = x.shape
+    codes = np.zeros((rows, n), dtype=np.uint8)
+    scales = np.zeros((rows, n // 32), dtype=np.uint8)
+    for i in range(rows):
+        lib().or_fp8_row(_p(x[i]), C.c_int(n), codes[i].ctypes.data_as(C.c_void_p), scales[i].ctypes.data_as(C.c_void_p))
+    return codes, scales
+
+
+def fp8_decode(codes, scales):
+    codes = _c(codes, np.uint8)
+    scales = _c(scales, np.uint8)
+    lib().or_fp8_get.restype = C.c_float
+    rows, n = codes.shape
+    y = np.zeros((rows, n), dtype=np.float32)
+    for i in range(rows):
+        for j in range(n):
+            y[i, j] = lib().or_fp8_get(codes[i].ctypes.data_as(C.c_void_p), scales[i].ctypes.data_as(C.c_void_p), C.c_int(j))
+    return y
+
+
+def heads_map(W, x, H, O, I, xs, hs, g=None):
+    """W f32 [H * O, I] (exact weights), x [T, xs] -> y [T, H, O]."""
+    W = _c(W, np.float32)
+    x = _c(x, np.float32)
+    T = x.shape[0]
+    y = np.zeros((T, H, O), dtype=np.float32)
+    gg = _c(g, np.float32) if g is not None else None
+    lib().or_heads_map(C.c_int(H), C.c_int(O), C.c_int(I), _p(W), _p(x), C.c_int(xs), C.c_int(hs), _p(gg) if gg is not None else None,
+                       _p(y), C.c_int(T))
+    return y
+
+
+def rope_pair(x0, x1, pos, inv):
+    y0, y1 = C.c_double(0), C.c_double(0)
+    lib().or_rope_pair(C.c_double(x0), C.c_double(x1), C.c_int(pos), C.c_float(inv), C.byref(y0), C.byref(y1))
+    return y0.value, y1.value
+
+
+def mla_attn(ql, qr, lat, kr, pos, scale):
+    """One (row, head): ql [r], qr [rope], lat [npos, r], kr [npos, rope] (f32 values) -> olat [r]."""
+    ql, qr, lat, kr = _c(ql, np.float32), _c(qr, np.float32), _c(lat, np.float32), _c(kr, np.float32)
+    r, rope = ql.size, qr.size
+    o = np.zeros(r, dtype=np.float32)
+    lib().or_mla_attn(C.c_int(r), C.c_int(rope), C.c_double(scale), _p(ql), _p(qr), _p(lat), _p(kr), C.c_int(pos), _p(o))
+    return o

@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include "cpu_seed4.h"
+#include "kvq.h"
 #include "lfsr.h"
 #include "qwen4_ops.h"
 #include "rows.h"
@@ -48,6 +49,12 @@ void ref_qwen4_route(int n_exp, int top_k, const float* logits, int32_t* ind, fl
     c.n_exp = n_exp; c.top_k = top_k;
     qwen4_route(&c, logits, ind, wt);
 }
+
+float ref_e4m3_dec(uint8_t c) { return kvq_e4m3_dec(c); }
+uint8_t ref_e4m3_enc_abs(float a) { return kvq_e4m3_enc_abs(a); }
+uint8_t ref_fp8_scale(float amax) { return kvq_fp8_scale(amax); }
+void ref_fp8_row(const float* x, int n, uint8_t* codes, uint8_t* scales) { kvq_row(x, n, n, codes, scales); }
+float ref_fp8_get(const uint8_t* codes, const uint8_t* scales, int i) { return kvq_fp8_get(codes, scales, i); }
 
 void ref_norm1p(const float* x, int len, int g, const float* w, float eps, float* y) { qwen4_norm1p(x, len, g, w, eps, y); }
 

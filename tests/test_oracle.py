@@ -488,3 +488,92 @@ def test_argmax_reference_vector(oracle):
     want = 1.0 / np.exp(z - z.max(1, keepdims=True)).sum(1)
     assert np.allclose(prob, want, rtol=1e-12)
     assert oracle.argmax(np.full((1, 17), -np.inf, dtype=np.float32)).tolist() == [0]
+
+
+def test_fp8_codec(oracle):
+    L = oracle.lib()
+    L.or_e4m3_dec.restype = C.c_float
+    L.or_e4m3_enc_abs.restype = C.c_uint8
+    L.or_fp8_scale.restype = C.c_uint8
+    dec = [L.or_e4m3_dec(C.c_uint8(c)) for c in range(256)]
+    # tests/test_kvq.c:30-35: every finite code round-trips and is exact in BF16; three hand values
+    for c in range(0x7F):
+        assert L.or_e4m3_enc_abs(C.c_float(dec[c])) == c
+        assert packs.round_bf16(np.float32(dec[c])) == np.float32(dec[c])
+    assert dec[0x7E] == 448 and dec[0x01] == 0.001953125 and dec[0xB8] == -1
+    # the closed form of the value table: (1 + m / 8) 2^(e - 7), subnormals m 2^-9
+    for c in range(0x7F):
+        e, m = c >> 3, c & 7
+        assert dec[c] == ((1 + m / 8) * 2.0 ** (e - 7) if e else m * 2.0 ** -9)
+    # rounding: nearest value, midpoints to the even code (:36-45), saturation at 448
+    rng = np.random.default_rng(5)
+    vals = np.array(dec[:0x7F], dtype=np.float64)
+    for a in np.concatenate([rng.uniform(0, 500, 2000), rng.uniform(0, 0.05, 500), (vals[:-1] + vals[1:]) / 2]).astype(np.float32):
+        got = L.or_e4m3_enc_abs(C.c_float(float(a)))
+        if a >= 448:
+            assert got == 0x7E
+            continue
+        d = np.abs(vals - float(a))
+        best = np.flatnonzero(d == d.min())
+        want = best[0] if len(best) == 1 else [b for b in best if b % 2 == 0][0]
+        assert got == want, (a, got, want)
+    # the scale: the smallest power of two s with 448 s >= amax
+    for amax in np.concatenate([rng.uniform(1e-6, 1e4, 500), 448.0 * 2.0 ** np.arange(-20, 20)]).astype(np.float32):
+        e = L.or_fp8_scale(C.c_float(float(amax))) - 127
+        assert 448.0 * 2.0 ** e >= amax and 448.0 * 2.0 ** (e - 1) < amax
+    assert L.or_fp8_scale(C.c_float(0.0)) == 127
+    # a row: decode(encode(x)) within half a step of the block's E4M3 grid
+    x = rng.standard_normal((3, 96)).astype(np.float32)
+    codes, scales = oracle.fp8_row(x)
+    y = oracle.fp8_decode(codes, scales)
+    assert np.all(np.abs(y - x) <= np.abs(x) * 2.0 ** -4 + 2.0 ** (scales.repeat(32, 1).astype(np.float64) - 127 - 10))
+
+
+def test_fp8_codec_vs_reference(oracle, ref):
+    L = oracle.lib()
+    for f in (L.or_e4m3_dec, ref.ref_e4m3_dec, ref.ref_fp8_get):
+        f.restype = C.c_float
+    for f in (L.or_e4m3_enc_abs, ref.ref_e4m3_enc_abs, L.or_fp8_scale, ref.ref_fp8_scale):
+        f.restype = C.c_uint8
+    rng = np.random.default_rng(6)
+    for c in range(256):
+        assert L.or_e4m3_dec(C.c_uint8(c)) == ref.ref_e4m3_dec(C.c_uint8(c))
+    for a in np.abs(np.concatenate([rng.standard_normal(3000) * 100, rng.standard_normal(1000) * 0.01])).astype(np.float32):
+        assert L.or_e4m3_enc_abs(C.c_float(float(a))) == ref.ref_e4m3_enc_abs(C.c_float(float(a)))
+        assert L.or_fp8_scale(C.c_float(float(a))) == ref.ref_fp8_scale(C.c_float(float(a)))
+    x = (rng.standard_normal((4, 128)) * rng.uniform(0.01, 50, (4, 1))).astype(np.float32)
+    codes, scales = oracle.fp8_row(x)
+    for i in range(4):
+        rc, rs = np.zeros(128, np.uint8), np.zeros(4, np.uint8)
+        ref.ref_fp8_row(x[i].ctypes.data_as(C.c_void_p), 128, rc.ctypes.data_as(C.c_void_p), rs.ctypes.data_as(C.c_void_p))
+        assert np.array_equal(rc, codes[i]) and np.array_equal(rs, scales[i])
+
+
+def test_mla_reference_forms(oracle):
+    rng = np.random.default_rng(12)
+    r, rope, npos = 64, 64, 9
+    lat = packs.round_bf16(rng.standard_normal((npos, r)).astype(np.float32))
+    kr = packs.round_bf16(rng.standard_normal((npos, rope)).astype(np.float32))
+    ql = (rng.standard_normal(r) * 0.3).astype(np.float32)
+    qr = rng.standard_normal(rope).astype(np.float32)
+    # one position: that position's latent; zero queries: equal scores, the mean latent
+    assert np.array_equal(oracle.mla_attn(ql, qr, lat, kr, 0, 0.1), lat[0])
+    o = oracle.mla_attn(np.zeros(r, np.float32), np.zeros(rope, np.float32), lat, kr, npos - 1, 0.1)
+    assert np.array_equal(o, packs.round_bf16(lat.astype(np.float64).mean(0).astype(np.float32)))
+    # the general case against numpy in float64 (tests/test_mova_kernels.c:1006-1024)
+    s = (lat[:6].astype(np.float64) @ ql + kr[:6].astype(np.float64) @ qr) * 0.125
+    p = np.exp(s - s.max())
+    want = packs.round_bf16(((p[:, None] * lat[:6]).sum(0) / p.sum()).astype(np.float32))
+    assert np.array_equal(oracle.mla_attn(ql, qr, lat, kr, 5, 0.125), want)
+    # rope: a rotation (norm kept), angle (float) pos * inv
+    y0, y1 = oracle.rope_pair(0.3, -0.7, 11, 0.01)
+    th = float(np.float32(np.float32(11) * np.float32(0.01)))
+    assert abs(y0 - (0.3 * np.cos(th) + 0.7 * np.sin(th))) < 1e-15 and abs(y1 - (-0.7 * np.cos(th) + 0.3 * np.sin(th))) < 1e-15
+    # per-head maps: bf16 of the double dot; with the gate, times bf16(softplus_ln2(g)), softplus_ln2(0) = 1
+    H, O, I, T = 2, 3, 16, 2
+    W = packs.round_bf16((rng.standard_normal((H * O, I)) * 0.1).astype(np.float32))
+    x = packs.round_bf16(rng.standard_normal((T, H * I)).astype(np.float32))
+    y = oracle.heads_map(W, x, H, O, I, H * I, I)
+    want = packs.round_bf16(np.einsum("hoi,thi->tho", W.reshape(H, O, I).astype(np.float64), x.reshape(T, H, I).astype(np.float64)).astype(np.float32))
+    assert np.array_equal(y, want)
+    assert np.array_equal(oracle.heads_map(W, x, H, O, I, H * I, I, g=np.zeros((T, H, O), np.float32)), want)
