@@ -215,6 +215,16 @@ void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvV
  * attention reads, for tests */
 void kc_kv_f32(kc_stream_t s, int fmt, const uint8_t* codes, const uint8_t* scales, int n, int rows, float* y);
 
+/* ---- additions for a host that runs a whole synthetic model (no counterpart in the reference's header) -------------------- */
+/* x = bf16(x + bf16(a + b)) (b may be NULL): the residual stream takes a block's branch outputs, BF16 at the boundary */
+void kc_residual_add(kc_stream_t s, float* x, const float* a, const float* b, size_t n);
+/* ri[t].pos += 1 for t < T: positions live on the device so that a captured decode step replays */
+void kc_rows_advance(kc_stream_t s, RowInfo* ri, int T);
+/* reproducible pseudo-random fills for synthetic packs: bytes (any bytes are valid seed records; nbytes rounded down to 8),
+ * and BF16 values uniform in [-scale, scale] */
+void kc_fill_random(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);
+void kc_fill_bf16(kc_stream_t s, uint16_t* p, size_t n, uint64_t seed, float scale);
+
 /* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
  * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same
  * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.

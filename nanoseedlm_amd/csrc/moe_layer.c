@@ -136,6 +136,13 @@ int nslm_moe_set_router(NslmMoe* m, int layer, const uint16_t* W, const uint16_t
     return e ? -1 : 0;
 }
 
+int nslm_moe_fill_random(NslmMoe* m, uint64_t seed, int eb, float router_scale) {
+    kc_fill_random(0, m->arena, m->unit_bytes * (uint64_t) m->units, seed);
+    kc_fill_bf16(0, m->rw, (size_t) m->c.n_layer * m->c.n_exp * m->c.d, seed ^ 0x5151, router_scale);
+    for (int i = 0; i < m->units * 3; ++i) m->eb[i] = eb;
+    return nh_device_sync() || kc_last_error() ? -1 : 0;
+}
+
 /* initial residency round-robin over the layers, expert-major, and the slice tables (engine/mova_cuda.c:372-392) */
 int nslm_moe_finalize(NslmMoe* m) {
     const int units = m->units, slots = m->pool.slots, E = m->c.n_exp, nl = m->c.n_layer;

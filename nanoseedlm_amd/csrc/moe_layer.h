@@ -37,6 +37,9 @@ int nslm_moe_set_expert(NslmMoe* m, int layer, int expert, int tensor, const uin
 /* router weight [n_exp][d] as BF16 bits; bias [n_exp] BF16 bits (sigmoid router only, else NULL) */
 int nslm_moe_set_router(NslmMoe* m, int layer, const uint16_t* W, const uint16_t* bias);
 int nslm_moe_finalize(NslmMoe* m);
+/* benchmarks: every expert's records filled on the device from a reproducible generator (any bytes are valid seed records),
+ * one exponent bias for all, router weights BF16 uniform in [-router_scale, router_scale].  Call before nslm_moe_finalize. */
+int nslm_moe_fill_random(NslmMoe* m, uint64_t seed, int eb, float router_scale);
 /* One MoE layer for T rows, asynchronous on stream s (launches only, capturable into a graph).
  * xn: the layer input [T][d] (device).  io [T][d] (device): softmax composition: receives sum_k wt_k y_k;
  * sigmoid composition: the residual stream, updated in place x = bf16(x + bf16(bf16(sum) + 0)). */

@@ -129,9 +129,59 @@ __global__ void __launch_bounds__(1024) k_argmax(const float* logits, int32_t* o
     }
 }
 
+// ---- what a host that runs a whole synthetic model needs beside the reference's kernels ---------------------------------
+// x = bf16(x + bf16(a + b)): the residual stream takes a block's two branch outputs, BF16 at the tensor boundary as the
+// MoVA engine keeps it (engine/kernels_moe.cu:780-788 does the same for its expert sum + shared expert)
+__global__ void __launch_bounds__(256) k_residual_add(float* x, const float* a, const float* b, size_t n) {
+    const size_t i = (size_t) blockIdx.x * 256 + threadIdx.x;
+    if (i < n) x[i] = bfr(x[i] + bfr(a[i] + (b ? b[i] : 0.0f)));
+}
+__global__ void k_rows_advance(RowInfo* ri, int T) {
+    const int t = (int) (blockIdx.x * blockDim.x + threadIdx.x);
+    if (t < T) ri[t].pos += 1;
+}
+// splitmix64 of the word index: reproducible pseudo-random bytes for synthetic packs (any bytes are valid seed records)
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__global__ void __launch_bounds__(256) k_fill_random(uint64_t* p, size_t nwords, uint64_t seed) {
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < nwords; i += (size_t) gridDim.x * 256) p[i] = mix64(seed ^ (i * 0xD1342543DE82EF95ull));
+}
+// BF16 values uniform in [-scale, scale]
+__global__ void __launch_bounds__(256) k_fill_bf16(uint16_t* p, size_t n, uint64_t seed, float scale) {
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) gridDim.x * 256) {
+        const uint32_t u = (uint32_t) (mix64(seed ^ (i * 0xD1342543DE82EF95ull)) >> 40);   // 24 bits
+        p[i] = (uint16_t) tobf(((float) u * (1.0f / 8388608.0f) - 1.0f) * scale);
+    }
+}
+
 }   // namespace
 
 extern "C" {
+
+void kc_residual_add(kc_stream_t s, float* x, const float* a, const float* b, size_t n) {
+    if (!n) return;
+    hipLaunchKernelGGL(k_residual_add, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, (hipStream_t) s, x, a, b, n);
+    host_note_launch();
+}
+void kc_rows_advance(kc_stream_t s, RowInfo* ri, int T) {
+    if (T < 1) return;
+    hipLaunchKernelGGL(k_rows_advance, dim3((unsigned) (T + 63) / 64), dim3(64), 0, (hipStream_t) s, ri, T);
+    host_note_launch();
+}
+void kc_fill_random(kc_stream_t s, void* p, size_t nbytes, uint64_t seed) {
+    if (nbytes < 8) return;
+    hipLaunchKernelGGL(k_fill_random, dim3(2048), dim3(256), 0, (hipStream_t) s, (uint64_t*) p, nbytes / 8, seed);
+    host_note_launch();
+}
+void kc_fill_bf16(kc_stream_t s, uint16_t* p, size_t n, uint64_t seed, float scale) {
+    if (!n) return;
+    hipLaunchKernelGGL(k_fill_bf16, dim3(2048), dim3(256), 0, (hipStream_t) s, p, n, seed, scale);
+    host_note_launch();
+}
 
 void kc_embed(kc_stream_t s, int fmt, WSlice w, int d, const int32_t* ids, float* x, int T) {
     if (T < 1 || d < 8) return;

@@ -45,6 +45,12 @@ def test_kt_backend_exports(libs):
     for n in set(re.findall(r"\b(kt_\w+)\s*\(", txt)):
         assert hasattr(K, n), n
     assert K.kt_name() == b"HIP gfx950" and K.kt_mm_tile() == 128
+    for h in ("moe_layer.h", "decode_model.h"):                        # the layer and whole-model hosts live in the same library
+        txt = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "nanoseedlm_amd", "csrc", h)).read(), flags=re.S)
+        names = set(re.findall(r"\b(nslm_\w+)\s*\(", txt))
+        assert len(names) > 8
+        for n in names:
+            assert hasattr(K, n), n
 
 
 def test_missing_library_fails_loudly(libs, monkeypatch):
