@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """bench.py - the SeedLM decode-in-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1|c3b16] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1|c3b16|c4b1|c4b16] [--no-cpu]
 
 A step is one pass of the workload over one batch of seeded synthetic input already resident in HBM:
   c2b1 (default; the configuration the metric is quoted on): one MoE decode layer step at batch 1 - 128 experts seeded
@@ -223,6 +223,77 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     return res
 
 
+def model_workload(name, steps, warmup, no_graph):
+    """Config 4: greedy decode of the whole synthetic model (24 layers of MLA attention over an FP8 latent cache + 128 seeded
+    experts top-8 + a shared expert, tied BF16 LM head over 151936 ids), the cache pre-filled so that the timed steps end at
+    the 4096th position.  A step = one token for each of the batch's sequences, all of its launches in one hipGraph."""
+    from nanoseedlm_amd import backend, model, moe
+    T = int(name[3:])
+    cfg = dict(n_layer=24, d=2048, n_head=16, head_dim=128, r=512, rope=64, n_exp=128, top_k=8, ff=768, ff_shared=768, vocab=151936,
+               max_ctx=4096, max_rows=T, kv_fmt=backend.KV_FP8, n_splits=32, eps=1e-6, rope_theta=10000.0)
+    if steps + warmup + 8 > cfg["max_ctx"]:
+        sys.exit("bench.py: c4 decodes towards position 4096; --steps + --warmup must stay below 4088")
+    m = model.DecodeModel(**cfg)
+    m.fill_random(seed=20261125, eb=-24)
+    start = cfg["max_ctx"] - steps - warmup - 4
+    rng = np.random.default_rng(4)
+    m.fill_cache(T, start, seed=5)
+    m.start(rng.integers(0, cfg["vocab"], T), np.full(T, start))
+    stream = moe.new_stream()
+    m.step(stream, T)                                                  # warm every kernel before capture
+    moe.device_sync()
+    g = None if no_graph else m.graph_of_step(stream, T)
+
+    def run():
+        if g:
+            m.launch(g, stream)
+        else:
+            m.step(stream, T)
+    seen = set()
+    for _ in range(warmup):
+        run()
+    moe.device_sync()
+    e0, e1 = moe.Event(), moe.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        run()
+    e1.record(stream)
+    e1.sync()
+    moe.device_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = e1.ms_since(e0) / steps
+    ids, logits = m.ids(T), m.logits(T)
+    if not np.isfinite(logits).all():
+        raise RuntimeError("the synthetic model's logits are not finite")
+    # bytes a step has to read: weight records (top-k experts per row; rows of a batch share some, counted once from the
+    # last layer's routing), the latent cache rows up to each sequence's position, the LM head
+    mh = C.c_void_p(m.L.nslm_model_moe(m.h))
+    ind = np.zeros((T, cfg["top_k"]), dtype=np.int32)
+    wt = np.zeros((T, cfg["top_k"]), dtype=np.float32)
+    backend.check(m.L.nslm_moe_last_routing(mh, T, ind.ctypes.data_as(C.c_void_p), wt.ctypes.data_as(C.c_void_p)), "nslm_moe_last_routing")
+    uniq = len(set(ind.reshape(-1).tolist()))
+    m.L.nslm_moe_expert_bytes.restype = C.c_uint64
+    eb = int(m.L.nslm_moe_expert_bytes(mh))
+    pos_mean = cfg["max_ctx"] - 4 - steps / 2.0
+    kv_bytes = T * cfg["n_layer"] * pos_mean * (cfg["r"] + cfg["rope"]) * (1 + 1 / 32.0)
+    bytes_step = m.step_bytes() - cfg["n_layer"] * cfg["top_k"] * eb + cfg["n_layer"] * uniq * eb + kv_bytes
+    flops = 2.0 * T * (m.step_bytes() - 2 * cfg["vocab"] * cfg["d"]) / 4.5 * 8 + 2.0 * T * cfg["vocab"] * cfg["d"]
+    res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
+    res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s", frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
+                           traffic=None, kernel="whole decode step (k_moe_decode x 24 is the largest share)" if T <= 8 else
+                           "whole decode step (grouped k_mm_stream launches are the largest share)",
+                           launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
+    res["config"] = {"workload": f"C4 full synthetic model greedy decode: 24 layers, hidden 2048, MLA 16 heads (latent 512 + rope 64, FP8 cache), "
+                                 f"128 seeded P=4 experts top-8 (intermediate 768) + shared expert, vocab 151936 BF16 LM head, batch {T}, "
+                                 f"positions {start + 1 + warmup}..{start + warmup + steps}",
+                     "launch": "stream" if no_graph else "hipGraph per step", "unique_experts_last_layer": uniq,
+                     "last_ids": [int(v) for v in ids[:4]]}
+    res["cpu_sample"] = dict(shapes=[(cfg["ff"], cfg["d"]), (cfg["ff"], cfg["d"]), (cfg["d"], cfg["ff"])], reps=cfg["top_k"], fmt=4)
+    m.close()
+    return res
+
+
 def dense_workload(name, steps, warmup):
     from nanoseedlm_amd import backend, moe, packs
     L = backend.hip()
@@ -369,6 +440,8 @@ def main():
         # (bucket + grouped GEMMs + glue, about ten launches) are captured into one graph per step.
         single = int(a.workload[3:]) <= 8 and a.workload[:2] == "c2"
         r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or (single and not a.graph))
+    elif a.workload[:2] == "c4":
+        r = model_workload(a.workload, a.steps, a.warmup, a.no_graph)
     else:
         r = dense_workload(a.workload, a.steps, a.warmup)
     gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6

@@ -224,6 +224,7 @@ void kc_rows_advance(kc_stream_t s, RowInfo* ri, int T);
  * and BF16 values uniform in [-scale, scale] */
 void kc_fill_random(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);
 void kc_fill_bf16(kc_stream_t s, uint16_t* p, size_t n, uint64_t seed, float scale);
+void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);   /* random E4M3 codes the cache's encoder can write (no 0x7F / 0xFF) */
 
 /* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
  * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same

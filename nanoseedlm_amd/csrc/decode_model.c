@@ -226,9 +226,9 @@ int nslm_model_fill_cache(NslmModel* m, int T, int upto, uint64_t seed) {
             if (c->kv_fmt == KV_BF16) {
                 kc_fill_bf16(0, (uint16_t*) m->kc + r0 * c->rope, (size_t) upto * c->rope, seed ^ (uint64_t) (l * 64 + t), 1.0f);
                 kc_fill_bf16(0, (uint16_t*) m->vc + r0 * c->r, (size_t) upto * c->r, seed ^ (uint64_t) (l * 64 + t + 4096), 1.0f);
-            } else {   /* every byte is a finite E4M3 code in this codec (no NaN patterns, nslm/kvq.h:19-23); scales 2^-6 */
-                kc_fill_random(0, m->kc + (r0 * c->rope) * e, (size_t) upto * c->rope, seed ^ (uint64_t) (l * 64 + t));
-                kc_fill_random(0, m->vc + (r0 * c->r) * e, (size_t) upto * c->r, seed ^ (uint64_t) (l * 64 + t + 4096));
+            } else {   /* codes as kc_mla_rope's encoder writes them (it saturates at 0x7E, nslm/kvq.h:19-23); scales 2^-6 */
+                kc_fill_fp8_codes(0, m->kc + (r0 * c->rope) * e, (size_t) upto * c->rope, seed ^ (uint64_t) (l * 64 + t));
+                kc_fill_fp8_codes(0, m->vc + (r0 * c->r) * e, (size_t) upto * c->r, seed ^ (uint64_t) (l * 64 + t + 4096));
                 nh_memset(m->ks + r0 * (c->rope / 32), 121, (size_t) upto * (c->rope / 32));
                 nh_memset(m->vs + r0 * (c->r / 32), 121, (size_t) upto * (c->r / 32));
             }

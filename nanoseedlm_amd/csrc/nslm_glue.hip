@@ -150,6 +150,14 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
 __global__ void __launch_bounds__(256) k_fill_random(uint64_t* p, size_t nwords, uint64_t seed) {
     for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < nwords; i += (size_t) gridDim.x * 256) p[i] = mix64(seed ^ (i * 0xD1342543DE82EF95ull));
 }
+// Random E4M3 codes as the cache's encoder can write them: it saturates at 0x7E, so the all-ones magnitude never occurs
+__global__ void __launch_bounds__(256) k_fill_fp8_codes(uint64_t* p, size_t nwords, uint64_t seed) {
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < nwords; i += (size_t) gridDim.x * 256) {
+        const uint64_t x = mix64(seed ^ (i * 0xD1342543DE82EF95ull));
+        const uint64_t ones = ((x & 0x7F7F7F7F7F7F7F7Full) + 0x0101010101010101ull) & 0x8080808080808080ull;
+        p[i] = x & ~(ones >> 7);
+    }
+}
 // BF16 values uniform in [-scale, scale]
 __global__ void __launch_bounds__(256) k_fill_bf16(uint16_t* p, size_t n, uint64_t seed, float scale) {
     for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) gridDim.x * 256) {
@@ -175,6 +183,11 @@ void kc_rows_advance(kc_stream_t s, RowInfo* ri, int T) {
 void kc_fill_random(kc_stream_t s, void* p, size_t nbytes, uint64_t seed) {
     if (nbytes < 8) return;
     hipLaunchKernelGGL(k_fill_random, dim3(2048), dim3(256), 0, (hipStream_t) s, (uint64_t*) p, nbytes / 8, seed);
+    host_note_launch();
+}
+void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed) {
+    if (nbytes < 8) return;
+    hipLaunchKernelGGL(k_fill_fp8_codes, dim3(2048), dim3(256), 0, (hipStream_t) s, (uint64_t*) p, nbytes / 8, seed);
     host_note_launch();
 }
 void kc_fill_bf16(kc_stream_t s, uint16_t* p, size_t n, uint64_t seed, float scale) {

@@ -254,23 +254,336 @@ __global__ void __launch_bounds__(64 * HG) k_mla_attn(MlaArgs a, int rope, const
             if (j < nl && lane + 64 * j < r) pp[2 + lane + 64 * j] = acc[j];
     }
 }
-// Reduce the splits: olat[t][h][d] = bf16(acc / l).  Workgroup (head, row); threads stride d.
-__global__ void __launch_bounds__(128) k_mla_reduce(MlaArgs a, const RowInfo* ri, const float* part, float* olat) {
-    const int h = (int) blockIdx.x, t = (int) blockIdx.y, r = a.r, w = r + 2, ns = mla_row_splits(a, ri[t].pos);
-    const float* pp = part + ((size_t) t * a.n_head + h) * a.n_splits * w;
-    float m = -INFINITY;
-    for (int s = 0; s < ns; ++s) m = fmaxf(m, pp[s * w]);
-    for (int d = (int) (blockIdx.z * blockDim.x + threadIdx.x); d < r; d += (int) (gridDim.z * blockDim.x)) {
-        float l = 0.0f, acc = 0.0f;
-        for (int s = 0; s < ns; ++s) {
-            const float ms = pp[s * w];
-            if (ms == -INFINITY) continue;
-            const float c = expf(ms - m);
-            l = fmaf(pp[s * w + 1], c, l);
-            acc = fmaf(pp[s * w + 2 + d], c, acc);
-        }
-        olat[((size_t) t * a.n_head + h) * r + d] = bfr(acc / l);
+
+// ---- latent attention on the matrix cores ---------------------------------------------------------------------------------
+// Absorbed MLA is multi-query attention over the latent: the 16 heads of a group read the same keys, so a tile of keys is
+// one MFMA operand for all of them (the reference's default path does the same on its tensor cores,
+// engine/kernels_moe.cu:1388-1397, with the same rounding points: queries are BF16 values, products exact, f32 sums,
+// f32 online softmax, P entering the second product as two BF16 terms hi + lo).
+// Workgroup (split, group of 16 heads, row) of 4 waves; tile = 32 keys.  Per tile:
+//   decode  the tile's cache rows -> BF16 in LDS twice: Ks[key][r + rope] (rows padded by 8) for the scores and
+//           Vt[latent dim][key] for P c (MFMA contracts over the index that is contiguous in a lane's fragment).  A thread
+//           owns 8 latent dims x 8 keys, so the transposition is 32 v_perm in registers.  FP8 -> BF16 is
+//           v_cvt_scalef32_pk_bf16_fp8 (E4M3 code x E8M0 scale, exact); the codes 0x7F / 0xFF (never written by the
+//           encoder; the reference's decoder reads them as +-480, the instruction as NaN) and scales outside 2^+-95
+//           take the arithmetic decoder, so every byte decodes as in nslm/kvq.h.
+//   scores  S^T[key][head] = Ks Q^T by v_mfma_f32_16x16x32_bf16, 18 k-slices x 2 key tiles; Q fragments stay in registers.
+//           Wave w sums half of the k-slices of key tile w & 1; the four partial tiles meet in LDS (a third barrier, but a
+//           quarter of the LDS reads of every wave computing all of S^T, which is what bounded the tile).
+//   softmax lane (head l % 16, keys {4g .. 4g + 3, 16 + 4g .. 16 + 4g + 3}, g = l / 16): two shuffles for the tile's max.
+//   P c     O^T[dim][head] += Vt P^T, wave w owns latent dims 128 w .. 128 w + 127 (8 accumulator tiles); the lane's P
+//           values are already the B fragment when Vt holds key (16 u + 4 g + i) at column 8 g + 4 u + i.
+// The next tile's cache bytes are loaded into registers before the current tile's MFMAs.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+#define MA_KB 32
+template <int R, int ROPE>
+constexpr int mla_mfma_lds() { return (MA_KB * (R + ROPE + 8) + R * MA_KB) * 2 + 4 * 64 * 16; }   // Vt (R x 32) also stages the 16 query rows
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf2(float lo, float hi) {   // v_cvt_pk_bf16_f32: both round to nearest even
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+template <int R, int ROPE, int FMT>
+__global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* out) {
+    static_assert(R == 512 && ROPE == 64, "the thread mapping of the decode covers 64 latent dim groups and 8 RoPE dim groups");
+    constexpr int KW = R + ROPE, KLD = KW + 8, NKS = KW / 32, MT = R / 64, NW = FMT == KV_FP8 ? 2 : 4;
+    extern __shared__ __attribute__((aligned(16))) uint8_t mla_lds[];
+    uint16_t* Ks = (uint16_t*) mla_lds;
+    uint16_t* Vt = Ks + MA_KB * KLD;
+    f32x4* Sx = (f32x4*) (Vt + R * MA_KB);   // [wave][lane]: the waves' partial score tiles
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int split = (int) blockIdx.x, t = (int) blockIdx.z, h = (int) blockIdx.y * 16 + c;
+    const int pos = ri[t].pos, kv0 = ri[t].kv0, ns = mla_row_splits(a, pos);
+    const int nsr = min(ns, (pos + a.chunk) / a.chunk);
+    const int chunk = (pos + nsr) / nsr;
+    const int p0 = split * chunk, p1 = split < nsr ? min(pos + 1, p0 + chunk) : p0;
+    const bool live = h < a.n_head;
+#ifdef NSLM_MLA_DEV   // development builds only: a.pad[1] switches parts of the tile loop off (1 loads, 2 decode, 4 scores, 8 P c)
+    const int abl = a.pad[1];
+#else
+    constexpr int abl = 0;
+#endif
+
+    // The group's queries, staged once for the four waves: thread e loads 4 consecutive values of head e / 128 (latent) or
+    // e / 16 (RoPE part); heads past n_head read head 0 and are zeroed.  The loads are issued here and converted after the
+    // first tile's loads are in flight.
+    constexpr int QV = 16 * KW / 4 / 256;   // float4 a thread
+    u32x4 qv[QV];
+#pragma unroll
+    for (int i = 0; i < QV; ++i) {
+        const int e = tid + 256 * i, hh = e < 16 * R / 4 ? e / (R / 4) : (e - 16 * R / 4) / (ROPE / 4);
+        const int hq = (int) blockIdx.y * 16 + hh;
+        const size_t th = (size_t) t * a.n_head + (hq < a.n_head ? hq : 0);
+        const NSLM_GLOBAL uint32_t* src = e < 16 * R / 4 ? gp<uint32_t>(ql) + th * R + 4 * (e % (R / 4)) : gp<uint32_t>(qr) + th * ROPE + 4 * ((e - 16 * R / 4) % (ROPE / 4));
+        qv[i] = *(const NSLM_GLOBAL u32x4*) src;
     }
+    // decode roles: latent dims 8 dg .. + 7 of keys {4 kap + j, 16 + 4 kap + j}; RoPE dims rd .. + 7 of key rkey
+    constexpr int ES = FMT == KV_FP8 ? 1 : 2;   // bytes a cached value
+    const int dgl = lane & 15, kap = lane >> 4, dg = 16 * w + dgl, par = dgl & 1, rkey = tid >> 3, rd = 8 * (tid & 7);
+    const uint32_t selA = par ? 0x07060302u : 0x05040100u, selB = par ? 0x05040100u : 0x07060302u;
+    uint32_t raw[8][NW] = {}, rraw[NW] = {}, rsc[8] = {127u, 127u, 127u, 127u, 127u, 127u, 127u, 127u}, rrsc = 127u;
+    auto fetch = [&](const void* codes, const void* scales, int row, int n, int d, uint32_t (&x)[NW], uint32_t& sc) {
+        if (FMT == KV_FP8) {
+            const uint2 q = ldg8(gp<uint8_t>(codes) + (size_t) row * n + d);
+            x[0] = q.x; x[1] = q.y;
+            sc = gp<uint8_t>(scales)[(size_t) row * (n / 32) + d / 32];
+        } else {
+            const uint4 q = ldg16(gp<uint16_t>(codes) + (size_t) row * n + d);
+            x[0] = q.x; x[1] = q.y; x[NW - 2] = q.z; x[NW - 1] = q.w;
+        }
+    };
+    // Keys past the split's end read its last key (finite values; their scores are masked), so no load is conditional.
+    auto load_tile = [&](int p) {
+        if (abl & 1) return;
+        const int rb = kv0 + p, last = p1 - 1 - p;
+        if (rb + MA_KB <= kv.nv || rb >= kv.nv) {   // the tile lies in one segment of the view (uniform): 32-bit offsets from its first row
+            const bool first = rb < kv.nv;
+            const KvSeg sg = first ? kv.a : kv.b;
+            const size_t r0 = (size_t) (first ? rb : rb - kv.nv);
+            const NSLM_GLOBAL uint8_t* vb = gp<uint8_t>(sg.v) + r0 * (R * ES);
+            const NSLM_GLOBAL uint8_t* kb = gp<uint8_t>(sg.k) + r0 * (ROPE * ES);
+            const NSLM_GLOBAL uint8_t* vsb = gp<uint8_t>(sg.vs) + r0 * (R / 32);
+            const NSLM_GLOBAL uint8_t* ksb = gp<uint8_t>(sg.ks) + r0 * (ROPE / 32);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t kj = (uint32_t) min(j < 4 ? 4 * kap + j : 12 + 4 * kap + j, last);
+                if (FMT == KV_FP8) {
+                    const uint2 q = ldg8(vb + (kj * (uint32_t) R + 8u * (uint32_t) dg));
+                    raw[j][0] = q.x; raw[j][1] = q.y;
+                    rsc[j] = vsb[kj * (uint32_t) (R / 32) + (uint32_t) (dg >> 2)];
+                } else {
+                    const uint4 q = ldg16(vb + (kj * (uint32_t) (2 * R) + 16u * (uint32_t) dg));
+                    raw[j][0] = q.x; raw[j][1] = q.y; raw[j][NW - 2] = q.z; raw[j][NW - 1] = q.w;
+                }
+            }
+            const uint32_t kr = (uint32_t) min(rkey, last);
+            if (FMT == KV_FP8) {
+                const uint2 q = ldg8(kb + (kr * (uint32_t) ROPE + (uint32_t) rd));
+                rraw[0] = q.x; rraw[1] = q.y;
+                rrsc = ksb[kr * (uint32_t) (ROPE / 32) + (uint32_t) (rd >> 5)];
+            } else {
+                const uint4 q = ldg16(kb + (kr * (uint32_t) (2 * ROPE) + 2u * (uint32_t) rd));
+                rraw[0] = q.x; rraw[1] = q.y; rraw[NW - 2] = q.z; rraw[NW - 1] = q.w;
+            }
+        } else {   // the tile straddles the view's two segments: each key finds its own
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int row;
+                const KvSeg sg = kv_seg(kv, rb + min(j < 4 ? 4 * kap + j : 12 + 4 * kap + j, last), &row);
+                fetch(sg.v, sg.vs, row, R, 8 * dg, raw[j], rsc[j]);
+            }
+            int row;
+            const KvSeg sg = kv_seg(kv, rb + min(rkey, last), &row);
+            fetch(sg.k, sg.ks, row, ROPE, rd, rraw, rrsc);
+        }
+    };
+    // FP8 words that v_cvt_scalef32_pk_bf16_fp8 reads as the codec does: no all-ones magnitude (bit 7 of a byte of the
+    // result set otherwise); a scale byte in [32, 222] keeps code x scale a normal BF16 value
+    auto odd_codes = [](uint32_t x0, uint32_t x1) { return ((x0 & 0x7F7F7F7Fu) + 0x01010101u) | ((x1 & 0x7F7F7F7Fu) + 0x01010101u); };
+    auto decode8 = [&](const uint32_t (&x)[NW], uint32_t sc, bool exact, uint32_t (&d)[4]) {
+        if (FMT != KV_FP8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) d[i] = x[i * NW / 4];
+        } else if (!exact) {
+            const float f = __uint_as_float(sc << 23);
+            d[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[0], f, false));
+            d[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[0], f, true));
+            d[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[1], f, false));
+            d[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[1], f, true));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t wd = x[i >> 1] >> (16 * (i & 1));
+                d[i] = (__float_as_uint(fp8_value(wd & 255u, sc)) >> 16) | (__float_as_uint(fp8_value((wd >> 8) & 255u, sc)) & 0xFFFF0000u);
+            }
+        }
+    };
+    auto store_tile = [&]() {
+        if (abl & 2) return;
+        uint32_t D[8][4], dr[4];
+        bool exact = false;
+        if (FMT == KV_FP8) {
+            uint32_t odd = odd_codes(rraw[0], rraw[1]), far = rrsc - 32u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                odd |= odd_codes(raw[j][0], raw[j][1]);
+                far = max(far, rsc[j] - 32u);
+            }
+            exact = (odd & 0x80808080u) != 0u || far > 190u;
+        }
+        if (!exact) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) decode8(raw[j], rsc[j], false, D[j]);
+            decode8(rraw, rrsc, false, dr);
+        } else {   // the arithmetic decoder for this lane's whole share
+#pragma unroll 1
+            for (int rep = 0; rep < 1; ++rep) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) decode8(raw[j], rsc[j], true, D[j]);
+                decode8(rraw, rrsc, true, dr);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int key = j < 4 ? 4 * kap + j : 12 + 4 * kap + j;
+            *(u32x4*) &Ks[key * KLD + 8 * dg] = u32x4{D[j][0], D[j][1], D[j][2], D[j][3]};
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {   // latent dims 8 dg + 2 q (+ 1): 8 keys each = one 16-byte block of a Vt row
+            u32x4 oa, ob;
+#pragma unroll
+            for (int jp = 0; jp < 4; ++jp) {
+                oa[jp] = __builtin_amdgcn_perm(D[2 * jp + 1][q], D[2 * jp][q], selA);
+                ob[jp] = __builtin_amdgcn_perm(D[2 * jp + 1][q], D[2 * jp][q], selB);
+            }
+            const int blk = kap ^ (q & 3) ^ ((dg >> 1) & 3), row = 8 * dg + 2 * q;
+            *(u32x4*) &Vt[(row + par) * MA_KB + 8 * blk] = oa;
+            *(u32x4*) &Vt[(row + 1 - par) * MA_KB + 8 * blk] = ob;
+        }
+        *(u32x4*) &Ks[rkey * KLD + R + rd] = u32x4{dr[0], dr[1], dr[2], dr[3]};
+    };
+
+    // Online softmax against a reference score m per head that is raised only when a tile's maximum exceeds it by more than
+    // MLA_LAZY (so P <= e^MLA_LAZY and the accumulators are rescaled on few tiles); l and acc are in the scale e^-m.
+    constexpr float MLA_LAZY = 8.0f;
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = -INFINITY, l = 0.0f;
+    if (p0 < p1) load_tile(p0);
+    // scores: wave w sums k-slices [9 (w >> 1), + 9) of key tile w & 1
+    constexpr int KH = NKS / 2;
+    const int su = w & 1, sk = (w >> 1) * KH;
+    bf16x8 qf[KH];
+    {   // queries -> BF16 rows in LDS (over Vt, which the first tile fills after the barrier below) -> the wave's B fragments
+        uint16_t* Qs = Vt;
+#pragma unroll
+        for (int i = 0; i < QV; ++i) {
+            const int e = tid + 256 * i, hh = e < 16 * R / 4 ? e / (R / 4) : (e - 16 * R / 4) / (ROPE / 4);
+            const int d = e < 16 * R / 4 ? 4 * (e % (R / 4)) : R + 4 * ((e - 16 * R / 4) % (ROPE / 4));
+            const uint32_t keep = (int) blockIdx.y * 16 + hh < a.n_head ? 0xFFFFFFFFu : 0u;
+            *(u32x2*) &Qs[hh * KLD + d] = u32x2{bf2(__uint_as_float(qv[i][0]), __uint_as_float(qv[i][1])) & keep,
+                                                bf2(__uint_as_float(qv[i][2]), __uint_as_float(qv[i][3])) & keep};
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < KH; ++ks) qf[ks] = *(const bf16x8*) &Qs[c * KLD + 32 * (sk + ks) + 8 * g];
+        __syncthreads();
+    }
+    for (int p = p0; p < p1; p += MA_KB) {
+        store_tile();
+        __syncthreads();
+        if (p + MA_KB < p1) load_tile(p + MA_KB);
+        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;   // two chains over the wave's 9 k-slices
+#pragma unroll
+        for (int ks = 0; ks < KH; ++ks) {
+            if (abl & 4) break;
+            const bf16x8 a0 = *(const bf16x8*) &Ks[(16 * su + c) * KLD + 32 * (sk + ks) + 8 * g];
+            if (ks & 1) s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s1, 0, 0, 0);
+            else s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
+        }
+        Sx[tid] = s0 + s1;
+        __syncthreads();
+        s0 = Sx[lane] + Sx[128 + lane];        // key tile 0: waves 0 and 2
+        s1 = Sx[64 + lane] + Sx[192 + lane];   // key tile 1: waves 1 and 3
+        float sv[8], mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int key = j < 4 ? 4 * g + j : 12 + 4 * g + j;
+            sv[j] = p + key < p1 ? (j < 4 ? s0[j] : s1[j - 4]) * a.scale : -INFINITY;
+            mx = fmaxf(mx, sv[j]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const bool up = mx > m + MLA_LAZY;   // true on the first tile (m = -inf; every tile has a key, so mx is finite)
+        if (__any(up)) {
+            const float cor = up ? __expf(m - mx) : 1.0f;
+            m = up ? mx : m;
+            l *= cor;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[mt] *= cor;
+        }
+        u32x4 bh, bl;
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+            const float e0 = __expf(sv[j] - m), e1 = __expf(sv[j + 1] - m);   // masked keys: exp(-inf) = 0
+            l += e0 + e1;
+            bh[j >> 1] = bf2(e0, e1);
+            bl[j >> 1] = bf2(e0 - __uint_as_float(bh[j >> 1] << 16), e1 - __uint_as_float(bh[j >> 1] & 0xFFFF0000u));
+        }
+        const bf16x8 ph = __builtin_bit_cast(bf16x8, bh), pl = __builtin_bit_cast(bf16x8, bl);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (abl & 8) break;
+            const int tile = w * MT + mt;
+            const bf16x8 vt = *(const bf16x8*) &Vt[(16 * tile + c) * MA_KB + 8 * (g ^ ((c >> 1) & 3) ^ (tile & 3))];
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, ph, acc[mt], 0, 0, 0);
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, pl, acc[mt], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    if (!live) return;
+    if (a.n_splits == 1) {
+        float* o = out + ((size_t) t * a.n_head + h) * R;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[16 * (w * MT + mt) + 4 * g + i] = bfr(acc[mt][i] / l);
+    } else {
+        float* pp = out + (((size_t) t * a.n_head + h) * a.n_splits + split) * (R + 2);
+        if (w == 0 && g == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pp[2 + 16 * (w * MT + mt) + 4 * g + i] = acc[mt][i];
+    }
+}
+
+// Reduce the splits: olat[t][h][d] = bf16(acc / l).  Workgroup (head, row, 128 latent dims): the splits' maxima and
+// weights exp(m_s - m) once per workgroup (threads stride the splits, so their loads are in flight together), then each
+// thread sums its dim over the splits.
+#define MLA_RED_MAXS 256
+__global__ void __launch_bounds__(128) k_mla_reduce(MlaArgs a, const RowInfo* ri, const float* part, float* olat) {
+    __shared__ float wts[MLA_RED_MAXS], red[4];
+    const int h = (int) blockIdx.x, t = (int) blockIdx.y, r = a.r, w = r + 2, ns = mla_row_splits(a, ri[t].pos), tid = threadIdx.x;
+    const NSLM_GLOBAL float* pp = gp<float>(part) + ((size_t) t * a.n_head + h) * a.n_splits * w;
+    float ms[MLA_RED_MAXS / 128], m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < MLA_RED_MAXS / 128; ++i) {
+        const int s = tid + 128 * i;
+        ms[i] = s < ns ? pp[(size_t) s * w] : -INFINITY;
+        m = fmaxf(m, ms[i]);
+    }
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(red[0], red[1]);
+    float l = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MLA_RED_MAXS / 128; ++i) {
+        const int s = tid + 128 * i;
+        if (s < ns) {
+            const float c = ms[i] == -INFINITY ? 0.0f : expf(ms[i] - m);
+            wts[s] = c;
+            l = fmaf(pp[(size_t) s * w + 1], c, l);
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    if ((tid & 63) == 0) red[2 + (tid >> 6)] = l;
+    __syncthreads();
+    l = red[2] + red[3];
+    const int d = (int) blockIdx.z * 128 + tid;
+    if (d >= r) return;
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int s = 0; s < ns; ++s) acc = fmaf(pp[(size_t) s * w + 2 + d], wts[s], acc);
+    olat[((size_t) t * a.n_head + h) * r + d] = bfr(acc / l);
 }
 
 // y = `rows` FP8 cache rows of n values, decoded (8 values a thread; for tests)
@@ -315,7 +628,17 @@ void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvV
         return;
     }
     float* o = a.n_splits > 1 ? part : olat;
-    if (a.n_head > 8)
+    if (a.n_splits > MLA_RED_MAXS) { host_note_unsupported(); return; }
+    if (a.r == 512 && rope == 64 && (((uintptr_t) ql | (uintptr_t) qr) & 15u) == 0) {   // the matrix-core kernel: 16 heads a workgroup
+        constexpr int lds = mla_mfma_lds<512, 64>();
+        static const hipError_t once[2] = {
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_FP8>, hipFuncAttributeMaxDynamicSharedMemorySize, lds)};
+        (void) once;
+        const dim3 grid((unsigned) a.n_splits, (unsigned) (a.n_head + 15) / 16, (unsigned) T);
+        if (kv.fmt == KV_FP8) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_FP8>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+        else hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_BF16>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+    } else if (a.n_head > 8)
         hipLaunchKernelGGL(k_mla_attn<16>, dim3((unsigned) a.n_splits, (unsigned) (a.n_head + 15) / 16, (unsigned) T), dim3(1024), 0, (hipStream_t) s,
                            a, rope, ql, qr, kv, ri, o);
     else

@@ -89,7 +89,8 @@ def test_kv_f32_decodes_the_codec(be, oracle):
 
 
 CASES = [(32, 768, 128, 3, 1, 0), (32, 768, 128, 3, 5, 0), (20, 64, 128, 3, 3, 0), (8, 96, 128, 45, 1, 0), (32, 768, 128, 3, 40, 150),
-         (20, 64, 128, 3, 40, 150), (16, 512, 64, 3, 8, 0)]
+         (20, 64, 128, 3, 40, 150), (16, 512, 64, 3, 8, 0), (16, 512, 64, 3, 1, 0), (20, 512, 64, 3, 5, 0), (5, 512, 64, 45, 3, 0),
+         (40, 512, 64, 3, 40, 150)]
 
 
 @pytest.mark.parametrize("nh,r,rope,T,ns,lp", CASES)
@@ -116,6 +117,33 @@ def test_latent_attention(be, oracle, nh, r, rope, T, ns, lp):
     dec = dict(k=packs.f32_to_bf16_bits(oracle.fp8_decode(kc, ksc)), v=packs.f32_to_bf16_bits(oracle.fp8_decode(vc, vsc)))
     od = be.kt_mla_attn(nh, r, rope, be.KV_BF16, ql, qr, dec, pos, kv0, scale, (301 + ns - 1) // ns, ns, long_from=lp)
     assert np.array_equal(o8.view(np.uint32), od.view(np.uint32))
+
+
+def test_latent_attention_over_any_cache_bytes(be, oracle):
+    """Every byte is a code of this codec: a cache of random bytes (0x7F / 0xFF, which the encoder never writes, and scale
+    bytes far from 127 included) reads as the decoded cache does."""
+    rng = np.random.default_rng(77)
+    nh, r, rope, NP, T = 16, 512, 64, 200, 2
+    vc, kc = rng.integers(0, 256, (NP, r)).astype(np.uint8), rng.integers(0, 256, (NP, rope)).astype(np.uint8)
+    vsc = rng.integers(118, 124, (NP, r // 32)).astype(np.uint8)
+    ksc = rng.integers(118, 124, (NP, rope // 32)).astype(np.uint8)
+    vsc[rng.random(vsc.shape) < 0.1] = 20                             # outside the range the conversion instruction takes
+    vc[::7, 5], vc[3::11, 130], kc[::5, 9] = 0x7F, 0xFF, 0x7F
+    ql = packs.round_bf16((rng.standard_normal((T, nh, r)) * 0.05).astype(np.float32))
+    qr = packs.round_bf16((rng.standard_normal((T, nh, rope)) * 0.05).astype(np.float32))
+    scale = float(1 / np.sqrt(192.0))
+    ld, kd = oracle.fp8_decode(vc, vsc), oracle.fp8_decode(kc, ksc)
+    assert np.isfinite(ld).all() and np.abs(ld).max() == 480 * 2.0 ** -4
+    for ns in (1, 4):
+        o8 = be.kt_mla_attn(nh, r, rope, be.KV_FP8, ql, qr, dict(k=kc, v=vc, ks=ksc, vs=vsc), [199, 70], [0, 0], scale, 64, ns)
+        od = be.kt_mla_attn(nh, r, rope, be.KV_BF16, ql, qr, dict(k=packs.f32_to_bf16_bits(kd), v=packs.f32_to_bf16_bits(ld)), [199, 70], [0, 0],
+                            scale, 64, ns)
+        assert np.array_equal(o8.view(np.uint32), od.view(np.uint32))
+        for t, p in ((0, 199), (1, 70)):
+            for h in (0, 9):
+                want = oracle.mla_attn(ql[t, h], qr[t, h], ld, kd, p, scale)
+                # P enters the second product as BF16 hi + lo terms (16 bits of P): an absolute slack of 2^-16 of the largest value
+                assert np.all(close_bf(o8[t, h], want.astype(np.float64), 30.0 * 2.0 ** -16)), (ns, t, h)
 
 
 def test_latent_attention_long_context_fp8(be, oracle):
