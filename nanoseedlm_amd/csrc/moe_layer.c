@@ -1,5 +1,6 @@
 /* moe_layer.c - see moe_layer.h.  Plain C99 over the kc_ / kq4_ / nh_ entry points. */
 #include "moe_layer.h"
+#include "model_folder.h"
 
 #include <stdio.h>
 #include <stdlib.h>
@@ -134,6 +135,37 @@ int nslm_moe_set_router(NslmMoe* m, int layer, const uint16_t* W, const uint16_t
     int e = nh_memcpy_h2d(m->rw + (size_t) layer * m->c.n_exp * m->c.d, W, 2 * (size_t) m->c.n_exp * m->c.d);
     if (bias) e |= nh_memcpy_h2d(m->rb + (size_t) layer * m->c.n_exp, bias, 2 * (size_t) m->c.n_exp);
     return e ? -1 : 0;
+}
+
+/* A model folder's stacked expert tensor [experts][rows][cols / 8] into the arena: expert e's share of each stream is
+ * contiguous in the file, its exponent bias is entry e of the exp_bias stream. */
+int nslm_moe_load_experts(NslmMoe* m, int layer, int which, const NsfTensor* t) {
+    const int rows = which == 2 ? m->c.d : m->c.ff, cols = which == 2 ? m->c.ff : m->c.d;
+    if (!t || layer < 0 || layer >= m->c.n_layer || which < 0 || which > 2 || t->enc != m->c.fmt || t->slices != m->c.n_exp || t->rows != rows ||
+        t->cols != cols)
+        return -1;
+    int bad = 0;
+    for (int e = 0; e < m->c.n_exp && !bad; ++e) {
+        const int u = layer * m->c.n_exp + e;
+        uint8_t* base = m->arena + (uint64_t) u * m->unit_bytes;
+        for (int s = 0; s < 4; ++s) {
+            if (s == 2 || !m->stream_len[which][s]) continue;
+            const uint64_t n = m->stream_len[which][s];
+            if (t->s[s].len != n * (uint64_t) m->c.n_exp) return -1;
+            bad |= nsf_upload(base + m->pool.off[which][s], &t->s[s], (uint64_t) e * n, n);
+        }
+        int32_t eb;
+        memcpy(&eb, t->s[2].p + 4 * (size_t) e, 4);
+        m->eb[u * 3 + which] = eb;
+    }
+    return bad ? -1 : 0;
+}
+int nslm_moe_load_router(NslmMoe* m, int layer, const NsfTensor* w, const NsfTensor* bias) {
+    if (!w || layer < 0 || layer >= m->c.n_layer || w->enc != NSF_BF16 || w->slices != 1 || w->rows != m->c.n_exp || w->cols != m->c.d) return -1;
+    if (bias && (bias->enc != NSF_BF16 || bias->s[0].len != 2 * (uint64_t) m->c.n_exp)) return -1;
+    int bad = nsf_upload(m->rw + (size_t) layer * m->c.n_exp * m->c.d, &w->s[0], 0, w->s[0].len);
+    if (bias) bad |= nsf_upload(m->rb + (size_t) layer * m->c.n_exp, &bias->s[0], 0, bias->s[0].len);
+    return bad ? -1 : 0;
 }
 
 int nslm_moe_fill_random(NslmMoe* m, uint64_t seed, int eb, float router_scale) {

@@ -51,6 +51,11 @@ def test_kt_backend_exports(libs):
         assert len(names) > 8
         for n in names:
             assert hasattr(K, n), n
+    txt = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "model_folder.h")).read(), flags=re.S)
+    names = set(re.findall(r"\b((?:nsf|nslm_moe)_\w+)\s*\(", txt))                # the model-folder reader and its loaders
+    assert len(names) >= 11
+    for n in names:
+        assert hasattr(K, n), n
 
 
 def test_missing_library_fails_loudly(libs, monkeypatch):
