@@ -223,7 +223,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     return res
 
 
-def model_workload(name, steps, warmup, no_graph):
+def model_workload(name, steps, warmup, no_graph, branches=False):
     """Config 4: greedy decode of the whole synthetic model (24 layers of MLA attention over an FP8 latent cache + 128 seeded
     experts top-8 + a shared expert, tied BF16 LM head over 151936 ids), the cache pre-filled so that the timed steps end at
     the 4096th position.  A step = one token for each of the batch's sequences, all of its launches in one hipGraph."""
@@ -235,6 +235,7 @@ def model_workload(name, steps, warmup, no_graph):
         sys.exit("bench.py: c4 decodes towards position 4096; --steps + --warmup must stay below 4088")
     m = model.DecodeModel(**cfg)
     m.fill_random(seed=20261125, eb=-24)
+    m.set_branches(branches)
     start = cfg["max_ctx"] - steps - warmup - 4
     rng = np.random.default_rng(4)
     m.fill_cache(T, start, seed=5)
@@ -287,7 +288,7 @@ def model_workload(name, steps, warmup, no_graph):
     res["config"] = {"workload": f"C4 full synthetic model greedy decode: 24 layers, hidden 2048, MLA 16 heads (latent 512 + rope 64, FP8 cache), "
                                  f"128 seeded P=4 experts top-8 (intermediate 768) + shared expert, vocab 151936 BF16 LM head, batch {T}, "
                                  f"positions {start + 1 + warmup}..{start + warmup + steps}",
-                     "launch": "stream" if no_graph else "hipGraph per step", "unique_experts_last_layer": uniq,
+                     "launch": ("stream" if no_graph else "hipGraph per step") + (", side-stream branches" if branches else ""), "unique_experts_last_layer": uniq,
                      "last_ids": [int(v) for v in ids[:4]]}
     res["cpu_sample"] = dict(shapes=[(cfg["ff"], cfg["d"]), (cfg["ff"], cfg["d"]), (cfg["d"], cfg["ff"])], reps=cfg["top_k"], fmt=4)
     m.close()
@@ -427,6 +428,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="plain stream launches even for multi-launch steps")
     ap.add_argument("--graph", action="store_true", help="one hipGraph per step even when the step is a single launch")
+    ap.add_argument("--branches", action="store_true", help="c4: independent launches of a layer on side streams (parallel graph branches; measured slower)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="after the workload, run 20 device-to-device copies of this size: a copy kernel of known traffic "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -441,7 +443,7 @@ def main():
         single = int(a.workload[3:]) <= 8 and a.workload[:2] == "c2"
         r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or (single and not a.graph))
     elif a.workload[:2] == "c4":
-        r = model_workload(a.workload, a.steps, a.warmup, a.no_graph)
+        r = model_workload(a.workload, a.steps, a.warmup, a.no_graph, a.branches)
     else:
         r = dense_workload(a.workload, a.steps, a.warmup)
     gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6

@@ -30,7 +30,29 @@ struct NslmModel {
     float *x, *xn, *q, *cl, *kr, *qr, *ql, *olat, *o, *part, *mo, *as, *gs, *us, *sh, *logits;
     uint16_t *px, *pa;                 /* BF16 views of activations for the GEMM path */
     int final;
+    int branches;                      /* independent launches of a layer on side streams (parallel graph branches) */
+    nh_stream_t side[2];
+    nh_event_t ev[4];
 };
+
+/* side stream i starts after everything queued on s so far / s continues after everything queued on side stream i */
+static void fork_to(NslmModel* m, kc_stream_t s, int i) {
+    nh_event_record(m->ev[0], (nh_stream_t) s);
+    nh_stream_wait_event(m->side[i], m->ev[0]);
+}
+static void join_from(NslmModel* m, kc_stream_t s, int i) {
+    nh_event_record(m->ev[1 + i], m->side[i]);
+    nh_stream_wait_event((nh_stream_t) s, m->ev[1 + i]);
+}
+int nslm_model_set_branches(NslmModel* m, int on) {
+    if (on && !m->side[0]) {
+        int bad = nh_stream_create(&m->side[0]) | nh_stream_create(&m->side[1]);
+        for (int i = 0; i < 4; ++i) bad |= nh_event_create(&m->ev[i]);
+        if (bad) return -1;
+    }
+    m->branches = on != 0;
+    return 0;
+}
 
 static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
 static int qd(const NslmModelCfg* c) { return c->n_head * c->head_dim; }
@@ -146,6 +168,10 @@ void nslm_model_close(NslmModel* m) {
                  m->sh, m->logits, m->px, m->pa};
     for (size_t i = 0; i < sizeof d / sizeof d[0]; ++i)
         if (d[i]) nh_free(d[i]);
+    for (int i = 0; i < 2; ++i)
+        if (m->side[i]) nh_stream_destroy(m->side[i]);
+    for (int i = 0; i < 4; ++i)
+        if (m->ev[i]) nh_event_destroy(m->ev[i]);
     free(m->dense);
     free(m);
 }
@@ -264,16 +290,32 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         /* ---- attention: x += W_o v_up(attn(q_lat(q), q_rope_mix(q); c, k_rope)) ---- */
         kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l) * d, c->eps, m->xn, T);
         if (big) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
-        dense(m, s, &dn[NSLM_W_Q], m->xn, m->px, d, m->q, T, 0);
-        dense(m, s, &dn[NSLM_W_KVA], m->xn, m->px, d, m->cl, T, 0);
-        dense(m, s, &dn[NSLM_W_KR], m->xn, m->px, d, m->kr, T, 0);
         WSlice hw;
         memset(&hw, 0, sizeof hw);
         HmvArgs hq = {H, rope, hd, QD, hd, 0, {0, 0}}, hl = {H, r, hd, QD, hd, 0, {0, 0}}, hv = {H, hd, r, H * r, r, 0, {0, 0}};
+        const int par = m->branches && !big;
+        /* three projections of xn and two maps of q: with branches, [Q -> q RoPE mix] | [KV down, then q -> latent] | [K rope] */
+        kc_stream_t s1 = par ? (kc_stream_t) m->side[0] : s, s2 = par ? (kc_stream_t) m->side[1] : s;
+        if (par) { fork_to(m, s, 0); fork_to(m, s, 1); }
+        int one = 0;   /* the three projections of xn as one launch (steps of up to 8 rows on one stream) */
+        if (!big && !par) {
+            const WSlice w3[3] = {dn[NSLM_W_Q].w, dn[NSLM_W_KVA].w, dn[NSLM_W_KR].w};
+            const int R3[3] = {QD, r, rope}, a3[3] = {0, 0, 0};
+            float* const y3[3] = {m->q, m->cl, m->kr};
+            one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->xn, d, T);
+        }
+        if (!one) {
+            dense(m, s, &dn[NSLM_W_Q], m->xn, m->px, d, m->q, T, 0);
+            if (par) nh_event_record(m->ev[3], (nh_stream_t) s);
+            dense(m, s1, &dn[NSLM_W_KVA], m->xn, m->px, d, m->cl, T, 0);
+            dense(m, s2, &dn[NSLM_W_KR], m->xn, m->px, d, m->kr, T, 0);
+        }
         hw.p[0] = m->heads[NSLM_H_QRMIX] + (size_t) l * H * rope * hd;
         kc_heads_mv(s, hq, MF_BF16, hw, NULL, m->q, NULL, m->qr, T);
+        if (par) nh_stream_wait_event(m->side[0], m->ev[3]);
         hw.p[0] = m->heads[NSLM_H_QLAT] + (size_t) l * H * r * hd;
-        kc_heads_mv(s, hl, MF_BF16, hw, NULL, m->q, NULL, m->ql, T);
+        kc_heads_mv(s1, hl, MF_BF16, hw, NULL, m->q, NULL, m->ql, T);
+        if (par) { join_from(m, s, 0); join_from(m, s, 1); }
         KvView kv;
         memset(&kv, 0, sizeof kv);
         kv.a.k = m->kc + (size_t) l * rows * rope * e;
@@ -290,12 +332,22 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         dense(m, s, &dn[NSLM_W_O], m->o, m->pa, QD, m->x, T, 1);   /* x = bf16(x + bf16(W_o o)) */
         /* ---- experts: x = bf16(x + bf16(sum_k wt_k y_k + shared(xn))) ---- */
         kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l + 1) * d, c->eps, m->xn, T);
-        if (nslm_moe_step(m->moe, s, l, m->xn, T, m->mo)) return -1;
         const WSlice* st = m->shared_tab + (size_t) l * 3;
-        if (!big) {   /* the shared expert through the gather entry points with every pair on slice 0 (engine/qwen4_cuda.c:1029) */
-            kc_mv_gu(s, MF_SEED4P4, st, st + 1, d, ffs, m->xn, d, m->as, ffs, m->sel0, T, 1, NULL);
-            kc_mv(s, MF_SEED4P4, dn[NSLM_W_SD].w, ffs, d, m->as, ffs, m->sh, d, T, 0, NULL);
+        if (!big) {   /* the shared expert through the gather entry points with every pair on slice 0 (engine/qwen4_cuda.c:1029),
+                         beside the routed experts when branches are on (as the reference runs it on its second stream, :1026-1032) */
+            if (!par && ffs == c->ff) {   /* the whole expert block (routed + shared + residual) in the one persistent launch */
+                const WSlice sh3[3] = {dn[NSLM_W_SG].w, dn[NSLM_W_SU].w, dn[NSLM_W_SD].w};
+                const int rc = nslm_moe_step_layer(m->moe, s, l, m->xn, T, sh3, m->x, m->x);
+                if (rc < 0) return -1;
+                if (rc == 0) continue;
+            }
+            if (par) fork_to(m, s, 0);
+            kc_mv_gu(s1, MF_SEED4P4, st, st + 1, d, ffs, m->xn, d, m->as, ffs, m->sel0, T, 1, NULL);
+            kc_mv(s1, MF_SEED4P4, dn[NSLM_W_SD].w, ffs, d, m->as, ffs, m->sh, d, T, 0, NULL);
+            if (nslm_moe_step(m->moe, s, l, m->xn, T, m->mo)) return -1;
+            if (par) join_from(m, s, 0);
         } else {
+            if (nslm_moe_step(m->moe, s, l, m->xn, T, m->mo)) return -1;
             kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
             dense(m, s, &dn[NSLM_W_SG], m->xn, m->px, d, m->gs, T, 0);
             dense(m, s, &dn[NSLM_W_SU], m->xn, m->px, d, m->us, T, 0);

@@ -55,6 +55,10 @@ int nslm_model_start(NslmModel* m, int T, const int32_t* ids, const int32_t* pos
 int nslm_model_fill_cache(NslmModel* m, int T, int upto, uint64_t seed);
 /* one greedy decode step for the T sequences, asynchronous on s: reads the ids, appends to the caches at the positions,
  * leaves the arg-max tokens as the next ids and advances the positions.  Launches only. */
+/* on: a layer's independent launches (the three projections of the normed input, the two maps of the query, the shared
+ * expert beside the routed ones - the reference runs that one on a second stream, engine/qwen4_cuda.c:1026-1032) go to
+ * two side streams joined by events, which a captured step turns into parallel graph branches.  Steps of up to 8 rows. */
+int nslm_model_set_branches(NslmModel* m, int on);
 int nslm_model_step(NslmModel* m, kc_stream_t s, int T);
 /* synchronising reads for tests: the current ids, the last step's logits [T][vocab], the last step's final hidden rows */
 int nslm_model_ids(NslmModel* m, int T, int32_t* ids);

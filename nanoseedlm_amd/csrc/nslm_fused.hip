@@ -33,6 +33,10 @@ struct FusedArgs {
     int32_t* ind;                       // [T][k]
     uint32_t* sync;                     // [FUSED_SYNC_WORDS + T * ntile_d], see below
     int E, k, d, ff, T, xs, os;
+    int kk;                             // pairs a token: k routed experts + ns always-on (shared) experts
+    int ns;
+    WSlice sh[3];                       // ns = 1: the shared expert's gate / up / down slices (pair k of every token, weight 1)
+    const float* res;                   // non-null: out = bf16(res + bf16(sum)) (the residual stream; may alias out)
     int Lg, rpig, rows_g, ntile_g;      // gate+up pass: chunks per row, virtual rows per iteration / per item, items per pair
     int Ld, rpid, rows_d, ntile_d;      // down pass
     int grid;
@@ -164,13 +168,13 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[2][256];
     __shared__ __attribute__((aligned(16))) float rv[1024];   // route: the token's logits
-    __shared__ float rw_s[32];      // route: weight by rank
-    __shared__ int ri_s[32];        // route: expert by rank
-    __shared__ WSlice sl_s[3][32];  // route: the chosen experts' gate / up / down slices
+    __shared__ float rw_s[33];      // route: weight by rank (+ the shared expert's 1)
+    __shared__ int ri_s[33];        // route: expert by rank
+    __shared__ WSlice sl_s[3][33];  // route: the chosen experts' gate / up / down slices (+ the shared expert's)
     __shared__ int s_flag;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t G = (uint32_t) a.grid;
-    const int P_ = a.T * a.k;
+    const int P_ = a.T * a.kk;
     // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
     unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
 #ifdef NSLM_FUSED_STAMPS   // development builds: every workgroup's timeline
@@ -208,7 +212,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     }
     // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
     if ((int) blockIdx.x < items_g) {
-        staged = ((int) blockIdx.x / a.ntile_g) / a.k;
+        staged = ((int) blockIdx.x / a.ntile_g) / a.kk;
         stage_row(a.x + (size_t) staged * a.xs, a.d, xl, false);
     }
     STAMP(1);
@@ -243,6 +247,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
             const int which = tid / a.k, j = tid - which * a.k;
             sl_s[which][j] = (which == 0 ? a.gate : which == 1 ? a.up : a.down)[ri_s[j]];
         }
+        if (a.ns && tid >= 253) sl_s[tid - 253][a.k] = a.sh[tid - 253];
         if (tid < a.k) rw_s[tid] = expf(rv[ri_s[tid]] - rv[ri_s[0]]);
         __syncthreads();
         if (tid < a.k) {
@@ -250,6 +255,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
             for (int r = 0; r < a.k; ++r) top += rw_s[r];
             rw_s[tid] = rw_s[tid] / top;   // every lane has read all k values before any lane writes: one wave, in order
         }
+        if (a.ns && tid == 255) rw_s[a.k] = 1.0f;
         __syncthreads();
         if (blockIdx.x == (unsigned) t % G && tid < a.k) {   // one writer per token publishes the routing
             a.ind[(size_t) t * a.k + tid] = ri_s[tid];
@@ -259,7 +265,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
 
     // ---- phase 2: gate + up + SwiGLU, items (pair, row tile) -------------------------------------------------------------
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
-        const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.k, j = p - t * a.k;
+        const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
         const int v0 = tile * a.rows_g, v1 = min(v0 + a.rows_g, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
@@ -282,14 +288,14 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
     Chunk d0;
     if ((int) blockIdx.x < items_d) {
-        const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.k, j = p - t * a.k;
+        const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
         d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.rows_d, min(tile * a.rows_d + a.rows_d, a.d));
     }
     grid_barrier(a.sync, G);
     STAMP(4);
     for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
-        const int p = item / a.ntile_d, tile = item - p * a.ntile_d, t = p / a.k, j = p - t * a.k;
+        const int p = item / a.ntile_d, tile = item - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
         const int v0 = tile * a.rows_d, v1 = min(v0 + a.rows_d, a.d);
         if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
@@ -302,14 +308,14 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
                                     [&](int r, float s, float) { st_agent(Dp + r, bfr(s)); });
         wg_release();
         __syncthreads();
-        if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.k - 1);
+        if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.kk - 1);
         __syncthreads();
         if (s_flag) {   // all k experts' rows of this tile are written: out = 0.5 * 0 + sum_j wt_j D_j, in j order
             wg_acquire();
             for (int r = v0 + tid; r < v1; r += 256) {
                 float acc = 0.0f;
-                for (int jj = 0; jj < a.k; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.k + jj) * a.d + r), acc);
-                a.out[(size_t) t * a.os + r] = acc;
+                for (int jj = 0; jj < a.kk; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.kk + jj) * a.d + r), acc);
+                a.out[(size_t) t * a.os + r] = a.res ? bfr(a.res[(size_t) t * a.os + r] + bfr(acc)) : acc;
             }
             if (tid == 0) st_agent(&tick[t * a.ntile_d + tile], 0u);
         }
@@ -353,7 +359,7 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     }
     // the grid must be resident at once: all the device holds, but no more than the work can use
     int grid = (per_cu < 3 ? per_cu : 3) * cu_count();
-    const int items = a.T * a.k * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
+    const int items = a.T * a.kk * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     // A phase with a few items more than workgroups would leave stragglers a whole second item long (C2 at one token:
     // 784 down-row items on 768 workgroups); when the device can hold them, a few extra workgroups cost less.
     if (items > grid && items <= grid + grid / 8 && items <= per_cu * cu_count()) grid = items;
@@ -375,6 +381,12 @@ int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                   int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                   int32_t* ind, float* wt, float* A, float* D, uint32_t* sync) {
+    return kc_moe_decode_layer(s, fmt, router_w, gate, up, down, n_exp, top_k, d, ff, x, xs, T, out, os, logits, ind, wt, A, D, sync, NULL, NULL);
+}
+
+int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
+                        int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
+                        int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res) {
     if (T < 1 || T > MV_MAXT || top_k < 1 || top_k > 32 || n_exp > 1024 || n_exp < top_k) return -1;
     if (fmt != MF_SEED4P4 && fmt != MF_SEED4) return -1;
     if (host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u)) return -1;
@@ -383,10 +395,12 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
     if (!shape_of(d, true, &a.Lg, &a.rpig, &sg) || !shape_of(ff, false, &a.Ld, &a.rpid, &sd)) return -1;
     a.rw = router_w; a.gate = gate; a.up = up; a.down = down; a.x = x; a.out = out; a.logits = logits; a.wt = wt; a.A = A;
     a.D = D; a.ind = ind; a.sync = sync; a.E = n_exp; a.k = top_k; a.d = d; a.ff = ff; a.T = T; a.xs = xs; a.os = os;
+    a.ns = shared ? 1 : 0; a.kk = top_k + a.ns; a.res = res;
+    for (int i = 0; i < 3 && shared; ++i) a.sh[i] = shared[i];
     // Iterations per item (an item = one pair's row tile): the count that gives the busiest workgroup of a full grid the
     // fewest iterations, an item's set-up priced at a third of an iteration; a few items over the grid count as one round
     // (the launch adds workgroups for them).
-    const int full = 3 * cu_count(), P_ = T * top_k;
+    const int full = 3 * cu_count(), P_ = T * a.kk;
     const int it_g = (2 * ff + a.rpig - 1) / a.rpig, it_d = (d + a.rpid - 1) / a.rpid;
     auto pick = [&](int iters) {
         int best = 1;

@@ -34,9 +34,14 @@ struct MvArgs {
     const int32_t* sel;
     int K, R, xdiv, xs, ys, add, nt, f32out;
     int L, rpi, rows_per_wg;   // fast path: chunks per row, rows per iteration, virtual rows per workgroup
+    // MULTI: up to MV_MAXJ dense matrices over the same x in one launch; job j owns workgroups [wg0[j], wg0[j + 1])
+    WSlice wj[4];
+    float* yj[4];
+    int Rj[4], ysj[4], addj[4], wg0[5], nj;
 };
+#define MV_MAXJ 4
 
-enum { DENSE = 0, GATHER = 1, GATEUP = 2 };
+enum { DENSE = 0, GATHER = 1, GATEUP = 2, MULTI = 3 };
 
 // SHFL: L is a power of two <= 64 (<= 32 for GATEUP): row sums by wave shuffles, no barrier.  Otherwise through LDS.
 template <int P, int MODE, int NT, bool SHFL>
@@ -47,16 +52,24 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     const int tid = threadIdx.x, L = a.L, rpi = a.rpi;
     const int lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
-    const int pair = MODE == DENSE ? 0 : (int) blockIdx.y;
-    const int V = MODE == GATEUP ? 2 * a.R : a.R;   // virtual rows: gate row r = 2r, up row r = 2r + 1
-    const int v0 = (int) blockIdx.x * a.rows_per_wg, v1 = min(v0 + a.rows_per_wg, V);
-    WSlice wA = a.wd, wB = a.wd;
-    if (MODE != DENSE) {
+    constexpr bool DN = MODE == DENSE || MODE == MULTI;   // all tokens against one matrix
+    const int pair = DN ? 0 : (int) blockIdx.y;
+    int job = 0, wg = (int) blockIdx.x;
+    if (MODE == MULTI) {
+        while (job + 1 < a.nj && wg >= a.wg0[job + 1]) ++job;
+        wg -= a.wg0[job];
+    }
+    const int R = MODE == MULTI ? a.Rj[job] : a.R, ys = MODE == MULTI ? a.ysj[job] : a.ys, add = MODE == MULTI ? a.addj[job] : a.add;
+    float* const yb = MODE == MULTI ? a.yj[job] : a.y;
+    const int V = MODE == GATEUP ? 2 * R : R;   // virtual rows: gate row r = 2r, up row r = 2r + 1
+    const int v0 = wg * a.rows_per_wg, v1 = min(v0 + a.rows_per_wg, V);
+    WSlice wA = MODE == MULTI ? a.wj[job] : a.wd, wB = wA;
+    if (!DN) {
         const int sl = a.sel[pair];
         wA = a.ws[sl];
         if (MODE == GATEUP) wB = a.wu[sl];
     }
-    const float* xrow = a.x + (size_t) (MODE == DENSE ? 0 : pair / a.xdiv) * a.xs;
+    const float* xrow = a.x + (size_t) (DN ? 0 : pair / a.xdiv) * a.xs;
 
     const bool al = streams_aligned(P, wA) && (MODE != GATEUP || streams_aligned(P, wB));
 
@@ -113,11 +126,11 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                     const float other = __shfl_xor(s, L);   // rows 2r and 2r+1 sit side by side in the wave
                     if (active && ch == 0 && !(v & 1) && v < v1) {
                         const float gs = s * NSLM_R32, us = other * NSLM_R32;
-                        float* yo = a.y + (size_t) pair * a.ys + (v >> 1);
+                        float* yo = yb + (size_t) pair * ys + (v >> 1);
                         *yo = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                     }
                 } else if (active && ch == 0 && v < v1) {
-                    store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + v, s * NSLM_R32, a.add, a.f32out);
+                    store_y(yb + (size_t) (DN ? t : pair) * ys + v, s * NSLM_R32, add, a.f32out);
                 }
             }
         } else {
@@ -132,14 +145,14 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                     for (int j = 0; j < L; ++j) us += part[par][0][(2 * tid + 1) * L + j];
                     gs *= NSLM_R32;
                     us *= NSLM_R32;
-                    float* yo = a.y + (size_t) pair * a.ys + ((vb >> 1) + tid);
+                    float* yo = yb + (size_t) pair * ys + ((vb >> 1) + tid);
                     *yo = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                 }
             } else if (tid < nrow * (NT > 1 ? a.nt : 1)) {
                 const int t = tid / nrow, r = tid - t * nrow;
                 float s = 0.0f;
                 for (int j = 0; j < L; ++j) s += part[par][t][r * L + j];
-                store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + (vb + r), s * NSLM_R32, a.add, a.f32out);
+                store_y(yb + (size_t) (DN ? t : pair) * ys + (vb + r), s * NSLM_R32, add, a.f32out);
             }
         }
         cur = nxt;
@@ -482,6 +495,35 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
     if (T <= MV_MAXT && wide_ok(fmt, K, x, xs, T)) launch_wide<DENSE>(st, fmt, a, 1);
     else hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, a);
     note_launch();
+}
+
+int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,
+                const float* x, int xs, int T) {
+    int L, rpi;
+    bool shfl;
+    if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;
+    MvArgs a = {};
+    a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n;
+    int total = 0;
+    for (int j = 0; j < n; ++j) total += R[j];
+    a.rows_per_wg = pick_rows_per_wg(total, rpi, 1);
+    for (int j = 0; j < n; ++j) {
+        if (R[j] < 1) return -1;
+        a.wj[j] = w[j]; a.Rj[j] = R[j]; a.ysj[j] = ys[j]; a.addj[j] = add[j];
+        a.wg0[j + 1] = a.wg0[j] + (R[j] + a.rows_per_wg - 1) / a.rows_per_wg;
+    }
+    const dim3 grid((unsigned) a.wg0[n], 1);
+    hipStream_t st = (hipStream_t) s;
+    for (int t0 = 0; t0 < T; t0 += T > 1 ? MV_TG : 1) {   // passes of tokens as kc_mv's: a token's arithmetic is the same in either
+        MvArgs b = a;
+        b.x = x + (size_t) t0 * xs;
+        for (int j = 0; j < n; ++j) b.yj[j] = y[j] + (size_t) t0 * ys[j];
+        b.nt = T > 1 ? (T - t0 < MV_TG ? T - t0 : MV_TG) : 1;
+        if (T > 1) launch_seed_fmt<MULTI, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
+        else launch_seed_fmt<MULTI, 1>(st, fmt, b, shfl, grid, 0);
+    }
+    note_launch();
+    return 0;
 }
 
 void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,

@@ -77,6 +77,9 @@ class DecodeModel:
     def fill_cache(self, T, upto, seed=3):
         backend.check(self.L.nslm_model_fill_cache(self.h, T, upto, C.c_uint64(seed)), "nslm_model_fill_cache")
 
+    def set_branches(self, on=True):
+        backend.check(self.L.nslm_model_set_branches(self.h, int(on)), "nslm_model_set_branches")
+
     def step(self, stream, T):
         backend.check(self.L.nslm_model_step(self.h, stream, T), "nslm_model_step")
 

@@ -380,3 +380,41 @@ def test_cache_copy_moves_units(be):
     for u in (3, 7, 11):
         assert unit_slot[u] >= 0 and np.array_equal(pool[unit_slot[u]], arena[u])
     assert np.count_nonzero(unit_slot >= 0) == 3
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("T", [1, 3, 8])
+def test_mv_multi_equals_separate_matvecs(fmt, T):
+    """kc_mv_multi: several dense seed matrices over the same x in one launch, bit-equal to one kc_mv each (ragged row
+    counts, one job accumulating into y)."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(31 + T)
+    K, Rs, adds = 512, [200, 72, 1000, 8], [0, 1, 0, 0]
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    x = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, K)).astype(np.float32)))
+    keep, ws = [], (backend.WSlice * 4)()
+    for j, R in enumerate(Rs):
+        p = mk(rng, 1, R, K, eb=-20 - j)
+        words = p["coefs"] if fmt == packs.MF_SEED4P4 else p["nibs"]
+        bufs = [moe.DevBuf.from_array(p["seeds"][0]), moe.DevBuf.from_array(words[0])]
+        ws[j].p[0], ws[j].p[1], ws[j].eb = bufs[0].ptr.value, bufs[1].ptr.value, int(p["eb"][0])
+        if fmt == packs.MF_SEED4P4:
+            bufs.append(moe.DevBuf.from_array(p["codes"][0]))
+            ws[j].p[3] = bufs[2].ptr.value
+        keep += bufs
+    y0 = [packs.round_bf16(rng.standard_normal((T, R)).astype(np.float32)) for R in Rs]
+    ya, yb = [moe.DevBuf.from_array(v) for v in y0], [moe.DevBuf.from_array(v) for v in y0]
+    for j, R in enumerate(Rs):
+        L.kc_mv(None, fmt, ws[j], K, R, x.ptr, K, ya[j].ptr, R, T, adds[j], None)
+    Ra, ysa, ada = (C.c_int * 4)(*Rs), (C.c_int * 4)(*Rs), (C.c_int * 4)(*adds)
+    yp = (C.c_void_p * 4)(*[b.ptr.value for b in yb])
+    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, K, x.ptr, K, T) == 0
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    for j, R in enumerate(Rs):
+        a, b = ya[j].to_array(np.float32, (T, R)), yb[j].to_array(np.float32, (T, R))
+        assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32)), j
+    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, 520, x.ptr, 520, T) == -1      # K % 64: not launched

@@ -29,9 +29,9 @@ def norm_ref(x, w, eps):
     return (x / np.sqrt(np.mean(x * x) + eps) * (1.0 + f64(w))).astype(np.float32)
 
 
-@pytest.mark.parametrize("T", [2, 12])
+@pytest.mark.parametrize("T,branches", [(2, False), (2, True), (12, False)])
 @pytest.mark.parametrize("kv", ["bf16", "fp8"])
-def test_tiny_model_decode(oracle, kv, T):
+def test_tiny_model_decode(oracle, kv, T, branches):
     from nanoseedlm_amd import backend, model, moe
     backend.require_gpu()
     rng = np.random.default_rng(2024 + T)
@@ -39,6 +39,7 @@ def test_tiny_model_decode(oracle, kv, T):
     cfg = dict(n_layer=2, d=128, n_head=2, head_dim=64, r=64, rope=64, n_exp=8, top_k=2, ff=64, ff_shared=64, vocab=96, max_ctx=16,
                max_rows=T, kv_fmt=backend.KV_FP8 if kv == "fp8" else backend.KV_BF16, n_splits=2, eps=1e-6, rope_theta=10000.0)
     m = model.DecodeModel(**cfg)
+    m.set_branches(branches)                                           # independent launches of a layer on side streams
     L, d, H, hd, r, rope, E, k = cfg["n_layer"], cfg["d"], cfg["n_head"], cfg["head_dim"], cfg["r"], cfg["rope"], cfg["n_exp"], cfg["top_k"]
     QD, ffs, V = H * hd, cfg["ff_shared"], cfg["vocab"]
     shapes = {model.W_Q: (QD, d), model.W_KVA: (r, d), model.W_KR: (rope, d), model.W_O: (d, QD), model.W_SG: (ffs, d), model.W_SU: (ffs, d),
