@@ -214,8 +214,17 @@ void kc_mla_rope(kc_stream_t s, MlaArgs a, float* qr, const float* kr, const flo
 /* engine/kernels_cuda.h:157-161, engine/kernels_moe.cu:1217-1323,2459-2489.  olat[t][h] = bf16(sum_p softmax_p(scale (ql_th .
  * c_p + qr_th . k_p)) c_p) over p <= pos_t; n_splits > 1 splits the keys (partials in part: T x n_head x n_splits x (r + 2)
  * floats) and reduces.  r % 8 == 0, r <= 1024. */
+/* No counterpart in the reference (three launches there): kc_heads_mv(hq: query -> RoPE mix, O = rope) + kc_heads_mv(hl: query
+ * -> latent, O = r) + kc_mla_rope in ONE launch, the same bits.  Both maps in fmt over the same query rows (equal I, xs, hs, no
+ * gate).  0, or -1 when the shapes are outside it (r % 64, I / 8 not a power of two <= 64 ...): nothing is launched. */
+int kc_mla_qmaps_rope(kc_stream_t s, MlaArgs a, HmvArgs hq, HmvArgs hl, int fmt, WSlice Wq, WSlice Wl, const float* q, float* qr, float* ql,
+                      const float* kr, const float* c, KvView kv, const RowInfo* ri, const float* inv, int T);
 void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part,
                  float* olat, int T);
+/* No counterpart in the reference: kc_mla_attn (n_splits >= 2) followed by kc_heads_mv(hv: latent -> value, I = r) with the
+ * splits' reduce and the map in one launch; y[t][h][o] gets the same bits as the two calls write.  0, or -1 (nothing launched). */
+int kc_mla_attn_vup(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part, HmvArgs hv, int fmt,
+                    WSlice W, float* y, int T);
 /* engine/kernels_cuda.h:173-176.  y[i] = value i of `rows` cache rows of n values in fmt (KV_BF16 / KV_FP8): the decode the
  * attention reads, for tests */
 void kc_kv_f32(kc_stream_t s, int fmt, const uint8_t* codes, const uint8_t* scales, int n, int rows, float* y);

@@ -30,6 +30,18 @@ class MlaArgs(C.Structure):
 KV_BF16, KV_FP8 = 0, 2
 
 
+class HmvArgs(C.Structure):
+    _fields_ = [("H", C.c_int), ("O", C.c_int), ("I", C.c_int), ("xs", C.c_int), ("hs", C.c_int), ("gate", C.c_int), ("pad", C.c_int * 2)]
+
+
+class KvSeg(C.Structure):
+    _fields_ = [("k", C.c_void_p), ("v", C.c_void_p), ("ks", C.c_void_p), ("vs", C.c_void_p)]
+
+
+class KvView(C.Structure):
+    _fields_ = [("a", KvSeg), ("b", KvSeg), ("nv", C.c_int32), ("fmt", C.c_int32)]
+
+
 class RouterArgs(C.Structure):
     _fields_ = [("d", C.c_int), ("n", C.c_int), ("top_k", C.c_int), ("hw", C.c_int), ("scale", C.c_float)]
 

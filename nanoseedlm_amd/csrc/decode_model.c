@@ -310,12 +310,10 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
             dense(m, s1, &dn[NSLM_W_KVA], m->xn, m->px, d, m->cl, T, 0);
             dense(m, s2, &dn[NSLM_W_KR], m->xn, m->px, d, m->kr, T, 0);
         }
-        hw.p[0] = m->heads[NSLM_H_QRMIX] + (size_t) l * H * rope * hd;
-        kc_heads_mv(s, hq, MF_BF16, hw, NULL, m->q, NULL, m->qr, T);
-        if (par) nh_stream_wait_event(m->side[0], m->ev[3]);
-        hw.p[0] = m->heads[NSLM_H_QLAT] + (size_t) l * H * r * hd;
-        kc_heads_mv(s1, hl, MF_BF16, hw, NULL, m->q, NULL, m->ql, T);
-        if (par) { join_from(m, s, 0); join_from(m, s, 1); }
+        WSlice hwq = hw, hwl = hw, hwv = hw;
+        hwq.p[0] = m->heads[NSLM_H_QRMIX] + (size_t) l * H * rope * hd;
+        hwl.p[0] = m->heads[NSLM_H_QLAT] + (size_t) l * H * r * hd;
+        hwv.p[0] = m->heads[NSLM_H_VUP] + (size_t) l * H * hd * r;
         KvView kv;
         memset(&kv, 0, sizeof kv);
         kv.a.k = m->kc + (size_t) l * rows * rope * e;
@@ -324,10 +322,21 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         kv.a.vs = (float*) (m->vs + (size_t) l * rows * (r / 32));
         kv.nv = (int32_t) rows;
         kv.fmt = c->kv_fmt;
-        kc_mla_rope(s, ma, m->qr, m->kr, m->cl, kv, m->ri, m->inv, T);
-        kc_mla_attn(s, ma, m->ql, m->qr, kv, m->ri, m->part, m->olat, T);
-        hw.p[0] = m->heads[NSLM_H_VUP] + (size_t) l * H * hd * r;
-        kc_heads_mv(s, hv, MF_BF16, hw, NULL, m->olat, NULL, m->o, T);
+        /* the query's two maps + RoPE + cache write as one launch, and the splits' reduce + value-up map as one, where the
+           shapes allow (single stream); else the reference's sequence of five launches */
+        int fusedq = 0;
+        if (!par) fusedq = !kc_mla_qmaps_rope(s, ma, hq, hl, MF_BF16, hwq, hwl, m->q, m->qr, m->ql, m->kr, m->cl, kv, m->ri, m->inv, T);
+        if (!fusedq) {
+            kc_heads_mv(s, hq, MF_BF16, hwq, NULL, m->q, NULL, m->qr, T);
+            if (par) nh_stream_wait_event(m->side[0], m->ev[3]);
+            kc_heads_mv(s1, hl, MF_BF16, hwl, NULL, m->q, NULL, m->ql, T);
+            if (par) { join_from(m, s, 0); join_from(m, s, 1); }
+            kc_mla_rope(s, ma, m->qr, m->kr, m->cl, kv, m->ri, m->inv, T);
+        }
+        if (kc_mla_attn_vup(s, ma, m->ql, m->qr, kv, m->ri, m->part, hv, MF_BF16, hwv, m->o, T)) {
+            kc_mla_attn(s, ma, m->ql, m->qr, kv, m->ri, m->part, m->olat, T);
+            kc_heads_mv(s, hv, MF_BF16, hwv, NULL, m->olat, NULL, m->o, T);
+        }
         if (big) kc_pack_input_bf16(s, m->o, m->pa, (size_t) T * QD);
         dense(m, s, &dn[NSLM_W_O], m->o, m->pa, QD, m->x, T, 1);   /* x = bf16(x + bf16(W_o o)) */
         /* ---- experts: x = bf16(x + bf16(sum_k wt_k y_k + shared(xn))) ---- */

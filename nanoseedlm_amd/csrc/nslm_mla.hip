@@ -6,9 +6,9 @@
 //
 // Per cached position the kernel reads r + rope values once for ALL heads of a workgroup (multi-query over the shared
 // latent): 660 bytes at r = 512, rope 128, FP8 - so the attention of a 4096-token context moves 2.7 MB per row, and what
-// it costs is the 2 x (r + rope) multiply-adds per (key, head).  Those stay in f32 on the vector ALUs: the reference's
-// tests hold the output to one BF16 ulp + 2e-6 of a double-precision softmax, which BF16 matrix products of the scores
-// would not meet.
+// it costs is the 2 x (r + rope) multiply-adds per (key, head).  Latent 512 + RoPE 64 runs them on the matrix cores
+// (k_mla_attn_mfma: exact BF16 products, f32 sums, P as BF16 hi + lo, which holds the reference tests' bound of one BF16
+// ulp + 2e-6 of a double-precision softmax); other shapes stay in f32 on the vector ALUs (k_mla_attn).
 #include "nslm_mv_dev.h"
 
 using namespace nslm;
@@ -123,15 +123,17 @@ __global__ void __launch_bounds__(256) k_heads_mv(HmvArgs a, int fmt, WSlice W, 
 
 // ---- RoPE of the query RoPE parts (in place) and of the RoPE key into the cache; the latent into the cache -------------
 // Thread i: latent dim i (i < r) and the pair (i % half, + half) of head i / half (head n_head: the key), half = rope / 2.
-__global__ void __launch_bounds__(64) k_mla_rope(MlaArgs a, int rope, float* qr, const float* kr, const float* c, KvView kv,
-                                                 const RowInfo* ri, const float* inv) {
-    const int i = (int) blockIdx.x * 64 + threadIdx.x, t = (int) blockIdx.y, pos = ri[t].pos, half = rope / 2;
+// One wave's share (i = 64 consecutive values of one row t); QPART false leaves the query heads to the caller.
+template <bool QPART>
+__device__ __forceinline__ void rope_cache_wave(const MlaArgs& a, int rope, float* qr, const float* kr, const float* c, const KvView& kv,
+                                                const RowInfo* ri, const float* inv, int i, int t) {
+    const int pos = ri[t].pos, half = rope / 2;
     int row;
     const KvSeg sg = kv_seg(kv, ri[t].kv0 + pos, &row);
     const int head = i / half, p = i % half;
     const bool lat = i < a.r, key = head == a.n_head;
     float y0 = 0.0f, y1 = 0.0f;
-    if (head <= a.n_head) {
+    if (QPART ? head <= a.n_head : key) {
         float sn, cs;
         sincosf((float) pos * inv[p], &sn, &cs);
         float* qh = qr + ((size_t) t * a.n_head + (key ? 0 : head)) * rope;
@@ -154,6 +156,71 @@ __global__ void __launch_bounds__(64) k_mla_rope(MlaArgs a, int rope, float* qr,
     fp8_put(lat, lat ? bfr(c[(size_t) t * a.r + i]) : 0.0f, (uint8_t*) sg.v, (uint8_t*) sg.vs, (size_t) row, a.r, lat ? i : 0);
     fp8_put(key, bfr(y0), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, p);
     fp8_put(key, bfr(y1), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, p + half);
+}
+__global__ void __launch_bounds__(64) k_mla_rope(MlaArgs a, int rope, float* qr, const float* kr, const float* c, KvView kv,
+                                                 const RowInfo* ri, const float* inv) {
+    rope_cache_wave<true>(a, rope, qr, kr, c, kv, ri, inv, (int) blockIdx.x * 64 + threadIdx.x, (int) blockIdx.y);
+}
+
+// ---- the two maps of the query, its RoPE, and the cache write as ONE launch -----------------------------------------------
+// Grid (1 + r / 64 | cache blocks, n_head + 1, rows).  Head h < n_head: block 0 computes the `rope` rows of the RoPE mix
+// (k_heads_mv's arithmetic), rotates them (k_mla_rope's) and stores them; block b > 0 computes latent-query rows
+// [64 (b - 1), 64 b).  "Head" n_head: the blocks write the rotated key and the latent into the cache (rope_cache_wave).
+// The same bits as kc_heads_mv x 2 + kc_mla_rope.
+__global__ void __launch_bounds__(256) k_qmaps_rope(MlaArgs a, int rope, HmvArgs hq, HmvArgs hl, int fmt, WSlice Wq, WSlice Wl, const float* q,
+                                                   float* qr, float* ql, const float* kr, const float* c, KvView kv, const RowInfo* ri,
+                                                   const float* inv, int lpr) {
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    __shared__ float qs[ATT_HD];
+    const int tid = threadIdx.x, h = (int) blockIdx.y, t = (int) blockIdx.z, b = (int) blockIdx.x;
+    if (h == a.n_head) {   // uniform over the block
+        const int nx = (a.n_head + 1) * (rope / 2) > a.r ? (a.n_head + 1) * (rope / 2) : a.r;
+        const int i0 = (b * 4 + (tid >> 6)) * 64;
+        if (i0 < nx) rope_cache_wave<false>(a, rope, qr, kr, c, kv, ri, inv, i0 + (tid & 63), t);
+        return;
+    }
+    if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
+        load_tables(tab);
+        __syncthreads();
+    }
+    const bool mix = b == 0;
+    const HmvArgs& hm = mix ? hq : hl;
+    const int O = hm.O, o0 = mix ? 0 : 64 * (b - 1), o1 = mix ? O : min(o0 + 64, O);
+    const int rpw = 64 / lpr, sub = (tid & 63) / lpr, ln = tid & (lpr - 1);
+    const float* xv = q + (size_t) t * hm.xs + (size_t) h * hm.hs;
+    WSlice ws = mix ? Wq : Wl;
+    if (fmt == MF_SEED4P4) ws.eb = gp<int32_t>(ws.p[2])[h];
+    for (int ob = o0; ob < o1; ob += 4 * rpw) {
+        const int o = ob + (tid >> 6) * rpw + sub;
+        const bool live = o < o1;
+        float acc = 0.0f;
+        if (live)
+            for (int j = ln; j < hm.I / 8; j += lpr) {
+                float w[8], sc;
+                block_weights(fmt, ws, tab, h * O + o, hm.I, j, w, &sc);
+                const float* xb = xv + (size_t) j * 8;
+                float d = w[0] * xb[0];
+#pragma unroll
+                for (int cc = 1; cc < 8; ++cc) d = fmaf(w[cc], xb[cc], d);
+                acc = fmaf(d, sc, acc);
+            }
+        for (int sft = lpr >> 1; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft);
+        if (live && ln == 0) {
+            if (mix) qs[o] = bfr(acc);
+            else ql[((size_t) t * hl.H + h) * O + o] = bfr(acc);
+        }
+    }
+    if (!mix) return;
+    __syncthreads();
+    const int half = rope / 2;
+    if (tid < half) {
+        float sn, cs;
+        sincosf((float) ri[t].pos * inv[tid], &sn, &cs);
+        const float x0 = qs[tid], x1 = qs[tid + half];
+        float* qh = qr + ((size_t) t * a.n_head + h) * rope;
+        qh[tid] = bfr(x0 * cs - x1 * sn);
+        qh[tid + half] = bfr(x1 * cs + x0 * sn);
+    }
 }
 
 // ---- latent attention -----------------------------------------------------------------------------------------------------
@@ -586,6 +653,131 @@ __global__ void __launch_bounds__(128) k_mla_reduce(MlaArgs a, const RowInfo* ri
     olat[((size_t) t * a.n_head + h) * r + d] = bfr(acc / l);
 }
 
+// The splits' reduce and the value-up map of a head in ONE launch: workgroup (row group, head, row) reduces the head's
+// latent output into LDS (k_mla_reduce's arithmetic, all r dims: the map needs them all) and computes rows
+// [RG g, RG (g + 1)) of y[t][h] = bf16(W_h . olat[t][h]) (k_heads_mv's arithmetic).  The same bits as the two kernels.
+#define MLA_RV_GROUPS 16
+__global__ void __launch_bounds__(256) k_mla_reduce_vup(MlaArgs a, const RowInfo* ri, const float* part, HmvArgs hv, int fmt, WSlice W, float* y,
+                                                       int lpr) {
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    __shared__ float wts[MLA_RED_MAXS], red[4];
+    __shared__ __attribute__((aligned(16))) float ol[64 * MLA_MAXL];
+    constexpr int PF = 32, NP = 2;   // splits / map passes whose loads are issued before anything waits
+    const int g = (int) blockIdx.x, h = (int) blockIdx.y, t = (int) blockIdx.z, r = a.r, w = r + 2, ns = mla_row_splits(a, ri[t].pos), tid = threadIdx.x;
+    const NSLM_GLOBAL float* pp = gp<float>(part) + ((size_t) t * a.n_head + h) * a.n_splits * w;
+    const int rg = (hv.O + MLA_RV_GROUPS - 1) / MLA_RV_GROUPS, o0 = g * rg, o1 = min(o0 + rg, hv.O);
+    const int rpw = 64 / lpr, sub = (tid & 63) / lpr, ln = tid & (lpr - 1);
+    // Every load whose address is known now is in flight before the first wait: the splits' (m, l), this thread's two
+    // output dims of the first PF splits, and (BF16 maps, one block a lane) the map rows of the first NP passes.
+    // (loads are unconditional on clamped indices: a conditional load waits for the ones before it)
+    float msv[MLA_RED_MAXS / 128], lsv[MLA_RED_MAXS / 128], pv[2][PF];
+#pragma unroll
+    for (int i = 0; i < MLA_RED_MAXS / 128; ++i) {
+        const int s = tid + 128 * i, sc = min(s, ns - 1);
+        const bool ok = tid < 128 && s < ns;
+        const float mv = pp[(size_t) sc * w], lv = pp[(size_t) sc * w + 1];
+        msv[i] = ok ? mv : -INFINITY;
+        lsv[i] = ok ? lv : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int s = 0; s < PF; ++s) pv[k][s] = pp[(size_t) min(s, ns - 1) * w + 2 + min(tid + 256 * k, r - 1)];
+    const bool pre = fmt == MF_BF16 && hv.I / 8 == lpr && (((uintptr_t) W.p[0] | (uintptr_t) (2 * hv.I)) & 15u) == 0;
+    uint4 wq[NP];
+    if (pre) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int o = min(o0 + i * 4 * rpw + (tid >> 6) * rpw + sub, hv.O - 1);
+            wq[i] = ldg16(gp<uint16_t>(W.p[0]) + ((size_t) h * hv.O + o) * hv.I + (size_t) ln * 8);
+        }
+    }
+    if (fmt == MF_SEED4P4 || fmt == MF_SEED4) load_tables(tab);
+    // the splits' maximum and the sum of l exactly as k_mla_reduce forms them: its two waves, splits tid and tid + 128
+    float m = -INFINITY, l = 0.0f;
+    if (tid < 128) {
+#pragma unroll
+        for (int i = 0; i < MLA_RED_MAXS / 128; ++i) m = fmaxf(m, msv[i]);
+        for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        if ((tid & 63) == 0) red[tid >> 6] = m;
+    }
+    __syncthreads();
+    m = fmaxf(red[0], red[1]);
+    if (tid < 128) {
+#pragma unroll
+        for (int i = 0; i < MLA_RED_MAXS / 128; ++i) {
+            const int s = tid + 128 * i;
+            if (s < ns) {
+                const float c = msv[i] == -INFINITY ? 0.0f : expf(msv[i] - m);
+                wts[s] = c;
+                l = fmaf(lsv[i], c, l);
+            } else if (s < PF) wts[s] = 0.0f;   // the prefetched terms past the last split add x * 0
+        }
+        for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+        if ((tid & 63) == 0) red[2 + (tid >> 6)] = l;
+    }
+    __syncthreads();
+    l = red[2] + red[3];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int d = tid + 256 * k;
+        if (d >= r) break;
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < PF; ++s) acc = fmaf(pv[k][s], wts[s], acc);
+        for (int s = PF; s < ns; ++s) acc = fmaf(pp[(size_t) s * w + 2 + d], wts[s], acc);
+        ol[d] = bfr(acc / l);
+    }
+    for (int d = tid + 512; d < r; d += 256) {   // latent widths above 512
+        float acc = 0.0f;
+        for (int s = 0; s < ns; ++s) acc = fmaf(pp[(size_t) s * w + 2 + d], wts[s], acc);
+        ol[d] = bfr(acc / l);
+    }
+    __syncthreads();
+    WSlice ws = W;
+    if (fmt == MF_SEED4P4) ws.eb = gp<int32_t>(W.p[2])[h];
+    auto finish = [&](int o, bool live, float acc) {
+        for (int sft = lpr >> 1; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft);
+        if (live && ln == 0) y[((size_t) t * hv.H + h) * hv.O + o] = bfr(acc);
+    };
+    int ob = o0;
+    if (pre) {   // one block a lane from the prefetched rows: the same products and sums as the loop below
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            if (ob >= o1) break;
+            const int o = ob + (tid >> 6) * rpw + sub;
+            const uint4 q = wq[i];
+            const float* xb = ol + (size_t) ln * 8;
+            float d = bf(q.x & 0xFFFFu) * xb[0];
+            d = fmaf(bf(q.x >> 16), xb[1], d);
+            d = fmaf(bf(q.y & 0xFFFFu), xb[2], d);
+            d = fmaf(bf(q.y >> 16), xb[3], d);
+            d = fmaf(bf(q.z & 0xFFFFu), xb[4], d);
+            d = fmaf(bf(q.z >> 16), xb[5], d);
+            d = fmaf(bf(q.w & 0xFFFFu), xb[6], d);
+            d = fmaf(bf(q.w >> 16), xb[7], d);
+            finish(o, o < o1, fmaf(d, 1.0f, 0.0f));
+            ob += 4 * rpw;
+        }
+    }
+    for (; ob < o1; ob += 4 * rpw) {
+        const int o = ob + (tid >> 6) * rpw + sub;
+        const bool live = o < o1;
+        float acc = 0.0f;
+        if (live)
+            for (int j = ln; j < hv.I / 8; j += lpr) {
+                float wv[8], sc;
+                block_weights(fmt, ws, tab, h * hv.O + o, hv.I, j, wv, &sc);
+                const float* xb = ol + (size_t) j * 8;
+                float d = wv[0] * xb[0];
+#pragma unroll
+                for (int cc = 1; cc < 8; ++cc) d = fmaf(wv[cc], xb[cc], d);
+                acc = fmaf(d, sc, acc);
+            }
+        finish(o, live, acc);
+    }
+}
+
 // y = `rows` FP8 cache rows of n values, decoded (8 values a thread; for tests)
 __global__ void k_kv_f32(int fmt, const uint8_t* C, const uint8_t* S, int n, int rows, float* y) {
     const int i = ((int) blockIdx.x * (int) blockDim.x + threadIdx.x) * 8;
@@ -620,15 +812,31 @@ void kc_mla_rope(kc_stream_t s, MlaArgs a, float* qr, const float* kr, const flo
     hipLaunchKernelGGL(k_mla_rope, dim3((unsigned) (nx + 63) / 64, (unsigned) T), dim3(64), 0, (hipStream_t) s, a, rope, qr, kr, c, kv, ri, inv);
     host_note_launch();
 }
-void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part, float* olat,
-                 int T) {
+int kc_mla_qmaps_rope(kc_stream_t s, MlaArgs a, HmvArgs hq, HmvArgs hl, int fmt, WSlice Wq, WSlice Wl, const float* q, float* qr, float* ql,
+                      const float* kr, const float* c, KvView kv, const RowInfo* ri, const float* inv, int T) {
+    const int rope = rope_of(a);
+    int lpr = 1;
+    while (lpr < 64 && lpr < hq.I / 8) lpr <<= 1;
+    if (T < 1 || (kv.fmt != KV_BF16 && kv.fmt != KV_FP8) || (rope != 64 && rope != 128) || a.r % 64 || hq.O != rope || hl.O != a.r || hq.I != hl.I ||
+        hq.I % 8 || hq.I / 8 > 64 || lpr != hq.I / 8 || hq.H != a.n_head || hl.H != a.n_head || hq.gate || hl.gate || hq.xs != hl.xs || hq.hs != hl.hs)
+        return -1;
+    const int nx = (a.n_head + 1) * (rope / 2) > a.r ? (a.n_head + 1) * (rope / 2) : a.r;
+    const int bx = 1 + a.r / 64 > (nx + 255) / 256 ? 1 + a.r / 64 : (nx + 255) / 256;
+    hipLaunchKernelGGL(k_qmaps_rope, dim3((unsigned) bx, (unsigned) a.n_head + 1, (unsigned) T), dim3(256), 0, (hipStream_t) s, a, rope, hq, hl, fmt,
+                       Wq, Wl, q, qr, ql, kr, c, kv, ri, inv, lpr);
+    host_note_launch();
+    return 0;
+}
+// attention into the partials (n_splits > 1) or olat; the reduce when `reduce`.  false: unsupported, nothing launched
+static bool mla_attn_launch(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part, float* olat,
+                            int T, bool reduce) {
     const int rope = rope_of(a);
     if (T < 1 || (kv.fmt != KV_BF16 && kv.fmt != KV_FP8) || (rope != 64 && rope != 128) || a.r % 8 || a.r > 64 * MLA_MAXL || a.n_splits < 1) {
         host_note_unsupported();
-        return;
+        return false;
     }
     float* o = a.n_splits > 1 ? part : olat;
-    if (a.n_splits > MLA_RED_MAXS) { host_note_unsupported(); return; }
+    if (a.n_splits > MLA_RED_MAXS) { host_note_unsupported(); return false; }
     if (a.r == 512 && rope == 64 && (((uintptr_t) ql | (uintptr_t) qr) & 15u) == 0) {   // the matrix-core kernel: 16 heads a workgroup
         constexpr int lds = mla_mfma_lds<512, 64>();
         static const hipError_t once[2] = {
@@ -643,10 +851,28 @@ void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvV
                            a, rope, ql, qr, kv, ri, o);
     else
         hipLaunchKernelGGL(k_mla_attn<8>, dim3((unsigned) a.n_splits, 1, (unsigned) T), dim3(512), 0, (hipStream_t) s, a, rope, ql, qr, kv, ri, o);
-    if (a.n_splits > 1)
+    if (a.n_splits > 1 && reduce)
         hipLaunchKernelGGL(k_mla_reduce, dim3((unsigned) a.n_head, (unsigned) T, (unsigned) (a.r + 127) / 128), dim3(128), 0, (hipStream_t) s, a, ri,
                            part, olat);
     host_note_launch();
+    return true;
+}
+void kc_mla_attn(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part, float* olat,
+                 int T) {
+    (void) mla_attn_launch(s, a, ql, qr, kv, ri, part, olat, T, true);
+}
+int kc_mla_attn_vup(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* part, HmvArgs hv, int fmt,
+                    WSlice W, float* y, int T) {
+    int lpr = 1;
+    while (lpr < 64 && lpr < hv.I / 8) lpr <<= 1;
+    if (a.n_splits < 2 || a.n_splits > MLA_RED_MAXS || hv.I != a.r || a.r % 8 || a.r > 64 * MLA_MAXL || hv.H != a.n_head || hv.gate ||
+        (lpr != hv.I / 8 && hv.I / 8 <= 64) || hv.O < 1)
+        return -1;
+    if (!mla_attn_launch(s, a, ql, qr, kv, ri, part, NULL, T, false)) return -1;
+    hipLaunchKernelGGL(k_mla_reduce_vup, dim3(MLA_RV_GROUPS, (unsigned) a.n_head, (unsigned) T), dim3(256), 0, (hipStream_t) s, a, ri, part, hv, fmt, W,
+                       y, lpr);
+    host_note_launch();
+    return 0;
 }
 void kc_kv_f32(kc_stream_t s, int fmt, const uint8_t* codes, const uint8_t* scales, int n, int rows, float* y) {
     if (rows < 1 || n < 8 || (fmt != KV_BF16 && fmt != KV_FP8)) { host_note_unsupported(); return; }

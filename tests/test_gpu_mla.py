@@ -163,3 +163,103 @@ def test_latent_attention_long_context_fp8(be, oracle):
         for h in (0, 7, 15):
             want = oracle.mla_attn(ql[t, h], qr[t, h], ld, kd, p, scale)
             assert np.all(close_bf(o[t, h], want.astype(np.float64), 2e-6)), (t, h)
+
+
+@pytest.mark.parametrize("kvf", ["bf16", "fp8"])
+@pytest.mark.parametrize("H,hd,r,rope,T", [(16, 128, 512, 64, 3), (5, 64, 128, 128, 2)])
+def test_query_maps_rope_and_cache_write_in_one_launch(be, kvf, H, hd, r, rope, T):
+    """kc_mla_qmaps_rope == kc_heads_mv (RoPE mix) + kc_heads_mv (latent query) + kc_mla_rope: the same bits in qr, ql and
+    the cache rows."""
+    import ctypes as C
+    from nanoseedlm_amd import moe
+    L = be.hip()
+    rng = np.random.default_rng(H * r + T)
+    fmt = be.KV_FP8 if kvf == "fp8" else be.KV_BF16
+    es, NP = (1 if fmt == be.KV_FP8 else 2), 40
+    q = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, H * hd)).astype(np.float32)))
+    kr = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, rope)).astype(np.float32)))
+    c = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, r)).astype(np.float32)))
+    wq = moe.DevBuf.from_array(packs.f32_to_bf16_bits((rng.standard_normal((H, rope, hd)) / np.sqrt(hd)).astype(np.float32)))
+    wl = moe.DevBuf.from_array(packs.f32_to_bf16_bits((rng.standard_normal((H, r, hd)) / np.sqrt(hd)).astype(np.float32)))
+    inv = moe.DevBuf.from_array(np.array([10000.0 ** (-2.0 * p / rope) for p in range(rope // 2)], dtype=np.float32))
+    ri = (be.RowInfo * T)()
+    for t in range(T):
+        ri[t].pos, ri[t].kv0 = 3 + 5 * t, 10 * t
+    rib = moe.DevBuf(C.sizeof(ri))
+    be.check(L.nh_memcpy_h2d(rib.ptr, ri, C.c_size_t(C.sizeof(ri))), "h2d")
+    Wq, Wl = be.WSlice(), be.WSlice()
+    Wq.p[0], Wl.p[0] = wq.ptr.value, wl.ptr.value
+    a = be.MlaArgs(H, r, 128, 1, 0.1)
+    a.pad[0] = rope
+    hq, hl = be.HmvArgs(H, rope, hd, H * hd, hd, 0), be.HmvArgs(H, r, hd, H * hd, hd, 0)
+    L.kc_heads_mv.argtypes = [C.c_void_p, be.HmvArgs, C.c_int, be.WSlice, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.kc_mla_rope.argtypes = [C.c_void_p, be.MlaArgs, C.c_void_p, C.c_void_p, C.c_void_p, be.KvView, C.c_void_p, C.c_void_p, C.c_int]
+    L.kc_mla_qmaps_rope.argtypes = [C.c_void_p, be.MlaArgs, be.HmvArgs, be.HmvArgs, C.c_int, be.WSlice, be.WSlice, C.c_void_p, C.c_void_p, C.c_void_p,
+                                    C.c_void_p, C.c_void_p, be.KvView, C.c_void_p, C.c_void_p, C.c_int]
+    outs = []
+    for fused in (False, True):
+        kc, vc = moe.DevBuf(NP * rope * es), moe.DevBuf(NP * r * es)
+        ks, vs = moe.DevBuf(NP * rope // 32 + 16), moe.DevBuf(NP * r // 32 + 16)
+        for b in (kc, vc, ks, vs):
+            be.check(L.nh_memset(b.ptr, 0, C.c_size_t(b.nbytes)), "memset")
+        kv = be.KvView(be.KvSeg(kc.ptr, vc.ptr, ks.ptr, vs.ptr), be.KvSeg(None, None, None, None), NP, fmt)
+        qr, ql = moe.DevBuf(4 * T * H * rope), moe.DevBuf(4 * T * H * r)
+        if fused:
+            assert L.kc_mla_qmaps_rope(None, a, hq, hl, packs.MF_BF16, Wq, Wl, q.ptr, qr.ptr, ql.ptr, kr.ptr, c.ptr, kv, rib.ptr, inv.ptr, T) == 0
+        else:
+            L.kc_heads_mv(None, hq, packs.MF_BF16, Wq, None, q.ptr, None, qr.ptr, T)
+            L.kc_heads_mv(None, hl, packs.MF_BF16, Wl, None, q.ptr, None, ql.ptr, T)
+            L.kc_mla_rope(None, a, qr.ptr, kr.ptr, c.ptr, kv, rib.ptr, inv.ptr, T)
+        moe.device_sync()
+        assert L.kc_last_error() == 0
+        outs.append([qr.to_array(np.uint32, (T, H, rope)), ql.to_array(np.uint32, (T, H, r)), kc.to_array(np.uint8, (NP * rope * es,)),
+                     vc.to_array(np.uint8, (NP * r * es,)), ks.to_array(np.uint8, (NP * rope // 32,)), vs.to_array(np.uint8, (NP * r // 32,))])
+    assert outs[0][0].any() and outs[0][1].any() and outs[0][2].any() and outs[0][3].any()
+    for x, y in zip(*outs):
+        assert np.array_equal(x, y)
+
+
+@pytest.mark.parametrize("kvf,H,hd,r,rope,ns", [("fp8", 16, 128, 512, 64, 32), ("bf16", 16, 128, 512, 64, 5), ("bf16", 6, 64, 128, 128, 3)])
+def test_attention_with_reduce_and_value_map_in_one_launch(be, oracle, kvf, H, hd, r, rope, ns):
+    """kc_mla_attn_vup == kc_mla_attn + kc_heads_mv (latent -> value): the same bits."""
+    import ctypes as C
+    from nanoseedlm_amd import moe
+    L = be.hip()
+    rng = np.random.default_rng(H + r + ns)
+    T, NP = 3, 700
+    fmt = be.KV_FP8 if kvf == "fp8" else be.KV_BF16
+    lat = packs.round_bf16(rng.standard_normal((NP, r)).astype(np.float32))
+    krr = packs.round_bf16(rng.standard_normal((NP, rope)).astype(np.float32))
+    if fmt == be.KV_FP8:
+        kc, ksc = oracle.fp8_row(krr)
+        vc, vsc = oracle.fp8_row(lat)
+        bufs = [moe.DevBuf.from_array(x) for x in (kc, vc, ksc, vsc)]
+    else:
+        bufs = [moe.DevBuf.from_array(packs.f32_to_bf16_bits(krr)), moe.DevBuf.from_array(packs.f32_to_bf16_bits(lat)), moe.DevBuf(16), moe.DevBuf(16)]
+    kv = be.KvView(be.KvSeg(*[b.ptr for b in bufs]), be.KvSeg(None, None, None, None), NP, fmt)
+    ql = moe.DevBuf.from_array(packs.round_bf16((rng.standard_normal((T, H, r)) * 0.3).astype(np.float32)))
+    qr = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, H, rope)).astype(np.float32)))
+    wv = moe.DevBuf.from_array(packs.f32_to_bf16_bits((rng.standard_normal((H, hd, r)) / np.sqrt(r)).astype(np.float32)))
+    ri = (be.RowInfo * T)()
+    for t, (p, k0) in enumerate(((650, 0), (37, 20), (300, 310))):
+        ri[t].pos, ri[t].kv0 = p, k0
+    rib = moe.DevBuf(C.sizeof(ri))
+    be.check(L.nh_memcpy_h2d(rib.ptr, ri, C.c_size_t(C.sizeof(ri))), "h2d")
+    a = be.MlaArgs(H, r, 128, ns, float(1 / np.sqrt(hd + rope)))
+    a.pad[0] = rope
+    W = be.WSlice()
+    W.p[0] = wv.ptr.value
+    hv = be.HmvArgs(H, hd, r, H * r, r, 0)
+    part, olat = moe.DevBuf(4 * T * H * ns * (r + 2)), moe.DevBuf(4 * T * H * r)
+    ya, yb = moe.DevBuf(4 * T * H * hd), moe.DevBuf(4 * T * H * hd)
+    L.kc_mla_attn.argtypes = [C.c_void_p, be.MlaArgs, C.c_void_p, C.c_void_p, be.KvView, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.kc_heads_mv.argtypes = [C.c_void_p, be.HmvArgs, C.c_int, be.WSlice, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.kc_mla_attn_vup.argtypes = [C.c_void_p, be.MlaArgs, C.c_void_p, C.c_void_p, be.KvView, C.c_void_p, C.c_void_p, be.HmvArgs, C.c_int, be.WSlice,
+                                  C.c_void_p, C.c_int]
+    L.kc_mla_attn(None, a, ql.ptr, qr.ptr, kv, rib.ptr, part.ptr, olat.ptr, T)
+    L.kc_heads_mv(None, hv, packs.MF_BF16, W, None, olat.ptr, None, ya.ptr, T)
+    assert L.kc_mla_attn_vup(None, a, ql.ptr, qr.ptr, kv, rib.ptr, part.ptr, hv, packs.MF_BF16, W, yb.ptr, T) == 0
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    A, B = ya.to_array(np.uint32, (T, H, hd)), yb.to_array(np.uint32, (T, H, hd))
+    assert A.any() and np.array_equal(A, B)
