@@ -75,9 +75,11 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
  * uses slice sel[p] and input row p / xdiv. */
 /* No counterpart in the reference (its hosts launch kc_mv once per matrix): n <= 4 dense seed matrices w[j] ([R[j]][K]) against
  * the same T <= MV_MAXT rows of x in ONE launch, y[j][t * ys[j] + r] (+)= as kc_mv writes it, bit for bit.  0, or -1 when the
- * shapes are outside the seed fast path (K % 64, K > 6144, unaligned x): nothing is launched, call kc_mv per matrix. */
+ * shapes are outside the seed fast path (K % 64, K > 6144, unaligned x): nothing is launched, call kc_mv per matrix.
+ * norm_w (f32 [K], K <= 4096) or NULL: the rows of x are normalised first, exactly as kq4_norm1p(x, K, K, norm_w, norm_eps) would
+ * have stored them (each workgroup recomputes the row's scale; the launch of the norm is saved). */
 int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,
-                const float* x, int xs, int T);
+                const float* x, int xs, int T, const float* norm_w, float norm_eps);
 void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
                const int32_t* sel, int P, int xdiv, const uint32_t* G);
 /* engine/kernels_cuda.h:84-85, engine/kernels_moe.cu:2324-2328.  Routed experts' gate + up + SwiGLU in one pass:
@@ -258,10 +260,13 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
  * expert as kc_mv_gu + kc_mv on a second stream and adds the residual in its combine, engine/qwen4_cuda.c:1026-1083).
  * shared (host pointer to 3 slices: gate [ff][d], up [ff][d], down [d][ff]) or NULL: an always-on expert of the routed experts'
  * shape, pair top_k of every token with weight 1.  res or NULL: out = bf16(res + bf16(sum)), res may be out.  A and D then
- * hold T * (top_k + 1) rows.  Same results as the separate launches: sum = f32 sum_j wt_j bf16(y_j) + bf16(y_shared). */
+ * hold T * (top_k + 1) rows.  norm_w (f32 [d], d <= 4096) or NULL: x is normalised first, as kq4_norm1p(x, d, d, norm_w, norm_eps)
+ * would have stored it (res stays the raw stream).  Same results as the separate launches: sum = f32 sum_j wt_j bf16(y_j) +
+ * bf16(y_shared). */
 int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
-                        int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res);
+                        int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res, const float* norm_w,
+                        float norm_eps);
 /* last launch-configuration error of this library on the calling thread's device: 0 none, else a hipError_t value */
 int kc_last_error(void);
 

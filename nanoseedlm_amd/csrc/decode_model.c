@@ -288,23 +288,23 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
     for (int l = 0; l < c->n_layer; ++l) {
         const Dense* dn = m->dense + (size_t) l * NSLM_W_COUNT;
         /* ---- attention: x += W_o v_up(attn(q_lat(q), q_rope_mix(q); c, k_rope)) ---- */
-        kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l) * d, c->eps, m->xn, T);
-        if (big) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
         WSlice hw;
         memset(&hw, 0, sizeof hw);
         HmvArgs hq = {H, rope, hd, QD, hd, 0, {0, 0}}, hl = {H, r, hd, QD, hd, 0, {0, 0}}, hv = {H, hd, r, H * r, r, 0, {0, 0}};
         const int par = m->branches && !big;
-        /* three projections of xn and two maps of q: with branches, [Q -> q RoPE mix] | [KV down, then q -> latent] | [K rope] */
         kc_stream_t s1 = par ? (kc_stream_t) m->side[0] : s, s2 = par ? (kc_stream_t) m->side[1] : s;
-        if (par) { fork_to(m, s, 0); fork_to(m, s, 1); }
-        int one = 0;   /* the three projections of xn as one launch (steps of up to 8 rows on one stream) */
+        int one = 0;   /* steps of up to 8 rows on one stream: the norm and the three projections of its output as one launch */
         if (!big && !par) {
             const WSlice w3[3] = {dn[NSLM_W_Q].w, dn[NSLM_W_KVA].w, dn[NSLM_W_KR].w};
             const int R3[3] = {QD, r, rope}, a3[3] = {0, 0, 0};
             float* const y3[3] = {m->q, m->cl, m->kr};
-            one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->xn, d, T);
+            one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->x, d, T, m->norm + (size_t) (2 * l) * d, c->eps);
         }
         if (!one) {
+            kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l) * d, c->eps, m->xn, T);
+            if (big) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
+            /* with branches: [Q -> q RoPE mix] | [KV down, then q -> latent] | [K rope] */
+            if (par) { fork_to(m, s, 0); fork_to(m, s, 1); }
             dense(m, s, &dn[NSLM_W_Q], m->xn, m->px, d, m->q, T, 0);
             if (par) nh_event_record(m->ev[3], (nh_stream_t) s);
             dense(m, s1, &dn[NSLM_W_KVA], m->xn, m->px, d, m->cl, T, 0);
@@ -340,16 +340,17 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         if (big) kc_pack_input_bf16(s, m->o, m->pa, (size_t) T * QD);
         dense(m, s, &dn[NSLM_W_O], m->o, m->pa, QD, m->x, T, 1);   /* x = bf16(x + bf16(W_o o)) */
         /* ---- experts: x = bf16(x + bf16(sum_k wt_k y_k + shared(xn))) ---- */
-        kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l + 1) * d, c->eps, m->xn, T);
         const WSlice* st = m->shared_tab + (size_t) l * 3;
+        const float* nw2 = m->norm + (size_t) (2 * l + 1) * d;
+        if (!big && !par && ffs == c->ff) {   /* norm + routed + shared + residual: the whole expert block in the one persistent launch */
+            const WSlice sh3[3] = {dn[NSLM_W_SG].w, dn[NSLM_W_SU].w, dn[NSLM_W_SD].w};
+            const int rc = nslm_moe_step_layer(m->moe, s, l, m->x, T, sh3, m->x, m->x, nw2, c->eps);
+            if (rc < 0) return -1;
+            if (rc == 0) continue;
+        }
+        kq4_norm1p(s, m->x, d, d, nw2, c->eps, m->xn, T);
         if (!big) {   /* the shared expert through the gather entry points with every pair on slice 0 (engine/qwen4_cuda.c:1029),
                          beside the routed experts when branches are on (as the reference runs it on its second stream, :1026-1032) */
-            if (!par && ffs == c->ff) {   /* the whole expert block (routed + shared + residual) in the one persistent launch */
-                const WSlice sh3[3] = {dn[NSLM_W_SG].w, dn[NSLM_W_SU].w, dn[NSLM_W_SD].w};
-                const int rc = nslm_moe_step_layer(m->moe, s, l, m->xn, T, sh3, m->x, m->x);
-                if (rc < 0) return -1;
-                if (rc == 0) continue;
-            }
             if (par) fork_to(m, s, 0);
             kc_mv_gu(s1, MF_SEED4P4, st, st + 1, d, ffs, m->xn, d, m->as, ffs, m->sel0, T, 1, NULL);
             kc_mv(s1, MF_SEED4P4, dn[NSLM_W_SD].w, ffs, d, m->as, ffs, m->sh, d, T, 0, NULL);

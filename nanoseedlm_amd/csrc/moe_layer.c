@@ -221,14 +221,15 @@ int nslm_moe_finalize(NslmMoe* m) {
 /* The layer's whole expert block in the one persistent launch: routed experts + a shared expert of their shape + the
  * residual (out = bf16(res + bf16(sum)), res may be out).  0 done, 1 not available for this stack / shape (nothing
  * launched: compose nslm_moe_step with kc_mv_gu / kc_mv / kc_residual_add), -1 error. */
-int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out) {
+int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out,
+                        const float* norm_w, float norm_eps) {
     const NslmMoeCfg* c = &m->c;
     if (!m->final || T < 1 || T > c->max_rows || layer < 0 || layer >= c->n_layer) return -1;
     const int E = c->n_exp;
     const WSlice* tab = m->pool.tab + (size_t) layer * 3 * E;
     if (!(m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= MV_MAXT)) return 1;
     if (kc_moe_decode_layer(s, c->fmt, m->rw + (size_t) layer * E * c->d, tab, tab + E, tab + 2 * E, E, c->top_k, c->d, c->ff, xn, c->d, T, out,
-                            c->d, m->logit, m->ind, m->wt, m->A, m->D, m->sync, shared, res))
+                            c->d, m->logit, m->ind, m->wt, m->A, m->D, m->sync, shared, res, norm_w, norm_eps))
         return 1;
     return kc_last_error() ? -1 : 0;
 }

@@ -46,7 +46,8 @@ int nslm_moe_fill_random(NslmMoe* m, uint64_t seed, int eb, float router_scale);
 int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, float* io);
 /* routed experts + a shared expert (3 host slices: gate, up, down of the routed experts' shape) + residual in the one persistent launch:
  * out = bf16(res + bf16(sum_j wt_j y_j + y_shared)).  0 done, 1 not available (nothing launched), -1 error. */
-int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out);
+int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out,
+                        const float* norm_w, float norm_eps);   /* norm_w: xn is the raw stream, normalised inside (kq4_norm1p's values) */
 /* 1 (default): decode steps of the softmax composition with every expert resident run as one persistent kernel
  * (kc_moe_decode); 0: always the separate launchers.  The results are the same bits either way. */
 void nslm_moe_set_fused(NslmMoe* m, int on);

@@ -254,4 +254,27 @@ int host_store_f32();
 void host_note_launch();
 void host_note_unsupported();   // a launcher refused its arguments: kc_last_error() reports an invalid value
 
+// the sum of v over the workgroup's 256 threads, the same value in every thread (every thread must call)
+__device__ __forceinline__ float wg_sum(float v, float* red) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads();   // red may still be read from a previous call
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+// rsqrt(mean(x^2) + eps) of a row of g <= 256 NSLM_NORM_NR values, bit for bit as the RMSNorm kernel forms it (thread tid
+// sums k = tid, tid + 256, .. in order, then the workgroup tree), so a consumer that normalises its own input,
+// xn_k = x_k * r * (1 + w_k), computes what the separate kernel would have stored.  256 threads, every thread calls.
+#define NSLM_NORM_NR 16
+__device__ __forceinline__ float row_rnorm(const float* xi, int g, float eps, float* red) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NSLM_NORM_NR; ++j) {
+        const int k = (int) threadIdx.x + j * 256;
+        const float v = k < g ? xi[k] : 0.0f;
+        ss = fmaf(v, v, ss);
+    }
+    return rsqrtf(wg_sum(ss, red) / (float) g + eps);
+}
+
 }   // namespace nslm

@@ -37,6 +37,8 @@ struct FusedArgs {
     int ns;
     WSlice sh[3];                       // ns = 1: the shared expert's gate / up / down slices (pair k of every token, weight 1)
     const float* res;                   // non-null: out = bf16(res + bf16(sum)) (the residual stream; may alias out)
+    const float* nw;                    // non-null: x is normalised first, xn_k = x_k r (1 + nw_k), r = rsqrt(mean(x^2) + neps)
+    float neps;
     int Lg, rpig, rows_g, ntile_g;      // gate+up pass: chunks per row, virtual rows per iteration / per item, items per pair
     int Ld, rpid, rows_d, ntile_d;      // down pass
     int grid;
@@ -158,6 +160,11 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
 __device__ __forceinline__ void stage_row(const float* src, int n, float* xl, bool coherent) {
     for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = coherent ? ld_agent(src + i) : src[i];
 }
+// an input row, normalised on the way when nw is given: the values kq4_norm1p would have stored
+__device__ __forceinline__ void stage_input(const float* src, int n, float* xl, const float* nw, float rn) {
+    if (!nw) { stage_row(src, n, xl, false); return; }
+    for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = src[i] * rn * (1.0f + nw[i]);
+}
 
 #ifdef NSLM_FUSED_STAMPS
 __device__ unsigned long long g_fstamp[1024 * 8];
@@ -172,6 +179,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     __shared__ int ri_s[33];        // route: expert by rank
     __shared__ WSlice sl_s[3][33];  // route: the chosen experts' gate / up / down slices (+ the shared expert's)
     __shared__ int s_flag;
+    __shared__ float rn_s[MV_MAXT], nred[4];   // the rows' RMSNorm scales when the kernel normalises its input
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t G = (uint32_t) a.grid;
     const int P_ = a.T * a.kk;
@@ -187,6 +195,13 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     load_tables(tab);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
+    if (a.nw) {   // uniform: every workgroup forms every row's scale (T rows of d values from L2)
+        for (int t = 0; t < a.T; ++t) {
+            const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
+            if (tid == 0) rn_s[t] = r;
+        }
+        __syncthreads();
+    }
 
     // ---- phase 1: router logits, one wave per (token, expert): k_mv_any's BF16 row dot and BF16 store ----------------
     for (int item = (int) blockIdx.x * 4 + wv; item < a.T * a.E; item += (int) G * 4) {
@@ -196,7 +211,13 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         float acc = 0.0f;
         for (int j = lane; j < a.d / 8; j += 64) {
             const uint4 q = *(const uint4*) (wr + (size_t) j * 8);
-            const float4 x0 = *(const float4*) (xr + (size_t) j * 8), x1 = *(const float4*) (xr + (size_t) j * 8 + 4);
+            float4 x0 = *(const float4*) (xr + (size_t) j * 8), x1 = *(const float4*) (xr + (size_t) j * 8 + 4);
+            if (a.nw) {
+                const float4 w0 = *(const float4*) (a.nw + (size_t) j * 8), w1 = *(const float4*) (a.nw + (size_t) j * 8 + 4);
+                const float rn = rn_s[t];
+                x0.x = x0.x * rn * (1.0f + w0.x); x0.y = x0.y * rn * (1.0f + w0.y); x0.z = x0.z * rn * (1.0f + w0.z); x0.w = x0.w * rn * (1.0f + w0.w);
+                x1.x = x1.x * rn * (1.0f + w1.x); x1.y = x1.y * rn * (1.0f + w1.y); x1.z = x1.z * rn * (1.0f + w1.z); x1.w = x1.w * rn * (1.0f + w1.w);
+            }
             float dd = bf(q.x & 0xFFFFu) * x0.x;
             dd = fmaf(bf(q.x >> 16), x0.y, dd);
             dd = fmaf(bf(q.y & 0xFFFFu), x0.z, dd);
@@ -213,7 +234,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
     if ((int) blockIdx.x < items_g) {
         staged = ((int) blockIdx.x / a.ntile_g) / a.kk;
-        stage_row(a.x + (size_t) staged * a.xs, a.d, xl, false);
+        stage_input(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
     }
     STAMP(1);
     grid_barrier(a.sync, G);
@@ -271,7 +292,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
         if (staged != t) {
             __syncthreads();
-            stage_row(a.x + (size_t) t * a.xs, a.d, xl, false);
+            stage_input(a.x + (size_t) t * a.xs, a.d, xl, a.nw, a.nw ? rn_s[t] : 1.0f);
             staged = t;
             __syncthreads();
         }
@@ -381,12 +402,13 @@ int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                   int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                   int32_t* ind, float* wt, float* A, float* D, uint32_t* sync) {
-    return kc_moe_decode_layer(s, fmt, router_w, gate, up, down, n_exp, top_k, d, ff, x, xs, T, out, os, logits, ind, wt, A, D, sync, NULL, NULL);
+    return kc_moe_decode_layer(s, fmt, router_w, gate, up, down, n_exp, top_k, d, ff, x, xs, T, out, os, logits, ind, wt, A, D, sync, NULL, NULL, NULL, 0.0f);
 }
 
 int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
-                        int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res) {
+                        int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res, const float* norm_w,
+                        float norm_eps) {
     if (T < 1 || T > MV_MAXT || top_k < 1 || top_k > 32 || n_exp > 1024 || n_exp < top_k) return -1;
     if (fmt != MF_SEED4P4 && fmt != MF_SEED4) return -1;
     if (host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u)) return -1;
@@ -395,7 +417,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     if (!shape_of(d, true, &a.Lg, &a.rpig, &sg) || !shape_of(ff, false, &a.Ld, &a.rpid, &sd)) return -1;
     a.rw = router_w; a.gate = gate; a.up = up; a.down = down; a.x = x; a.out = out; a.logits = logits; a.wt = wt; a.A = A;
     a.D = D; a.ind = ind; a.sync = sync; a.E = n_exp; a.k = top_k; a.d = d; a.ff = ff; a.T = T; a.xs = xs; a.os = os;
-    a.ns = shared ? 1 : 0; a.kk = top_k + a.ns; a.res = res;
+    a.ns = shared ? 1 : 0; a.kk = top_k + a.ns; a.res = res; a.nw = norm_w; a.neps = norm_eps;
+    if (norm_w && (d > 256 * 16 || ((uintptr_t) norm_w & 15u))) return -1;
     for (int i = 0; i < 3 && shared; ++i) a.sh[i] = shared[i];
     // Iterations per item (an item = one pair's row tile): the count that gives the busiest workgroup of a full grid the
     // fewest iterations, an item's set-up priced at a third of an iteration; a few items over the grid count as one round

@@ -37,19 +37,11 @@ __global__ void __launch_bounds__(256) k_embed(int fmt, WSlice w, int d, const i
     for (int c = 0; c < 8; ++c) xo[c] = seedf ? bfr(o[c] * sc) : o[c];
 }
 
-// the sum of v over the workgroup's 256 threads, the same value in every thread
-__device__ __forceinline__ float wg_sum(float v, float* red) {
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    __syncthreads();   // red may still be read from a previous call
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return (red[0] + red[1]) + (red[2] + red[3]);
-}
 
 // One workgroup per (token, group): y = f(x * rsqrt(mean_group(x^2) + eps), w).  The group's values stay in registers
 // between the sum and the scaling when the group is at most 256 * NR long; longer groups read x twice.
 // MODE 0: the MoVA grouped norm, BF16 weights, y = bf16(w * (x * r));  MODE 1: the Qwen form, f32 weights, y = x r (1 + w).
-#define NR 16
+#define NR NSLM_NORM_NR
 template <int MODE>
 __global__ void __launch_bounds__(256) k_rmsnorm(const float* x, int len, int g, const void* wv, float eps, float* y) {
     __shared__ float red[4];
@@ -60,7 +52,7 @@ __global__ void __launch_bounds__(256) k_rmsnorm(const float* x, int len, int g,
         if (MODE == 0) yi[k] = bfr(bf(((const uint16_t*) wv)[a + k]) * (v * r));
         else yi[k] = v * r * (1.0f + ((const float*) wv)[a + k]);
     };
-    if (g <= 256 * NR) {
+    if (g <= 256 * NSLM_NORM_NR) {
         float v[NR], ss = 0.0f;
 #pragma unroll
         for (int j = 0; j < NR; ++j) {

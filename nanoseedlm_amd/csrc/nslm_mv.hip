@@ -38,6 +38,8 @@ struct MvArgs {
     WSlice wj[4];
     float* yj[4];
     int Rj[4], ysj[4], addj[4], wg0[5], nj;
+    const float* nw;      // non-null (dense modes): x is normalised first, xn_k = x_k r (1 + nw_k), r = rsqrt(mean(x^2) + neps)
+    float neps;
 };
 #define MV_MAXJ 4
 
@@ -49,6 +51,7 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     extern __shared__ float xl[];                  // NT > 1: activations [token][chunk][XPAD]
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[SHFL ? 1 : 2][SHFL ? 1 : NT][SHFL ? 1 : 256];
+    __shared__ float nred[4];
     const int tid = threadIdx.x, L = a.L, rpi = a.rpi;
     const int lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
@@ -84,8 +87,10 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     Chunk cur = fetch(v);
 
     load_tables(tab);
+    const bool prenorm = DN && a.nw != nullptr;   // uniform
     float xreg[NT == 1 ? 64 : 1];
     if (NT == 1) {
+        const float rn = prenorm ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
         if (active) {
             const float4* xp = (const float4*) (xrow + (size_t) ch * 64);
 #pragma unroll
@@ -93,13 +98,30 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                 const float4 q = xp[i];
                 xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
             }
+            if (prenorm) {
+                const float4* wp = (const float4*) (a.nw + (size_t) ch * 64);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float4 w4 = wp[i];
+                    xreg[4 * i] = xreg[4 * i] * rn * (1.0f + w4.x);
+                    xreg[4 * i + 1] = xreg[4 * i + 1] * rn * (1.0f + w4.y);
+                    xreg[4 * i + 2] = xreg[4 * i + 2] * rn * (1.0f + w4.z);
+                    xreg[4 * i + 3] = xreg[4 * i + 3] * rn * (1.0f + w4.w);
+                }
+            }
         }
     } else {
-        for (int t = 0; t < a.nt; ++t)
+        for (int t = 0; t < a.nt; ++t) {
+            const float rn = prenorm ? row_rnorm(a.x + (size_t) t * a.xs, a.K, a.neps, nred) : 1.0f;
             for (int i = tid; i < a.K / 4; i += 256) {
-                const float4 q = ((const float4*) (a.x + (size_t) t * a.xs))[i];
+                float4 q = ((const float4*) (a.x + (size_t) t * a.xs))[i];
+                if (prenorm) {
+                    const float4 w4 = ((const float4*) a.nw)[i];
+                    q.x = q.x * rn * (1.0f + w4.x); q.y = q.y * rn * (1.0f + w4.y); q.z = q.z * rn * (1.0f + w4.z); q.w = q.w * rn * (1.0f + w4.w);
+                }
                 *(float4*) &xl[(t * L + (i >> 4)) * XPAD + (i & 15) * 4] = q;
             }
+        }
     }
     __syncthreads();
 
@@ -498,12 +520,13 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
 }
 
 int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,
-                const float* x, int xs, int T) {
+                const float* x, int xs, int T, const float* norm_w, float norm_eps) {
     int L, rpi;
     bool shfl;
     if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;
+    if (norm_w && (K > 256 * 16 || !aligned16(norm_w))) return -1;
     MvArgs a = {};
-    a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n;
+    a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n; a.nw = norm_w; a.neps = norm_eps;
     int total = 0;
     for (int j = 0; j < n; ++j) total += R[j];
     a.rows_per_wg = pick_rows_per_wg(total, rpi, 1);

@@ -411,10 +411,26 @@ def test_mv_multi_equals_separate_matvecs(fmt, T):
         L.kc_mv(None, fmt, ws[j], K, R, x.ptr, K, ya[j].ptr, R, T, adds[j], None)
     Ra, ysa, ada = (C.c_int * 4)(*Rs), (C.c_int * 4)(*Rs), (C.c_int * 4)(*adds)
     yp = (C.c_void_p * 4)(*[b.ptr.value for b in yb])
-    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, K, x.ptr, K, T) == 0
+    L.kc_mv_multi.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(backend.WSlice), C.POINTER(C.c_int), C.POINTER(C.c_void_p), C.POINTER(C.c_int),
+                              C.POINTER(C.c_int), C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_float]
+    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, K, x.ptr, K, T, None, 0.0) == 0
     moe.device_sync()
     assert L.kc_last_error() == 0
     for j, R in enumerate(Rs):
         a, b = ya[j].to_array(np.float32, (T, R)), yb[j].to_array(np.float32, (T, R))
         assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32)), j
-    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, 520, x.ptr, 520, T) == -1      # K % 64: not launched
+    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yp, ysa, ada, 520, x.ptr, 520, T, None, 0.0) == -1      # K % 64: not launched
+    # with the input's RMSNorm inside the launch: the same bits as kq4_norm1p followed by one kc_mv each
+    nw = moe.DevBuf.from_array((0.2 * rng.standard_normal(K)).astype(np.float32))
+    xn = moe.DevBuf(4 * T * K)
+    L.kq4_norm1p.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_void_p, C.c_int]
+    L.kq4_norm1p(None, x.ptr, K, K, nw.ptr, 1e-6, xn.ptr, T)
+    yc, yd = [moe.DevBuf.from_array(v) for v in y0], [moe.DevBuf.from_array(v) for v in y0]
+    for j, R in enumerate(Rs):
+        L.kc_mv(None, fmt, ws[j], K, R, xn.ptr, K, yc[j].ptr, R, T, adds[j], None)
+    yq = (C.c_void_p * 4)(*[b.ptr.value for b in yd])
+    assert L.kc_mv_multi(None, fmt, 4, ws, Ra, yq, ysa, ada, K, x.ptr, K, T, nw.ptr, 1e-6) == 0
+    moe.device_sync()
+    for j, R in enumerate(Rs):
+        a, b = yc[j].to_array(np.float32, (T, R)), yd[j].to_array(np.float32, (T, R))
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)) and not np.array_equal(a, ya[j].to_array(np.float32, (T, R))), j

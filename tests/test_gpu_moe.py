@@ -107,3 +107,47 @@ def test_moe_step(oracle, router, T, slots):
     else:
         assert hits + misses > 0 and misses > 0  # a pool of 20 slots over 32 experts must evict
     st.close()
+
+
+@pytest.mark.parametrize("T", [1, 3, 8])
+def test_whole_expert_block_in_one_launch(T):
+    """nslm_moe_step_layer (input RMSNorm + routed experts + shared expert + residual inside the persistent kernel) writes the
+    same bits as kq4_norm1p + nslm_moe_step + kc_mv_gu / kc_mv (shared expert) + kc_residual_add."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L, K = backend.hip(), backend.kt()
+    rng = np.random.default_rng(77 + T)
+    E, k, d, ff = 16, 4, 256, 128
+    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=8)
+    gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-12), packs.seed4p4(rng, E, ff, d, eb=-12), packs.seed4p4(rng, E, d, ff, eb=-12)
+    st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.3).astype(np.float32)))
+    st.finalize()
+    keep, sh = [], (backend.WSlice * 3)()
+    for i, (R, Kk) in enumerate(((ff, d), (ff, d), (d, ff))):
+        p = packs.seed4p4(rng, 1, R, Kk, eb=-12)
+        bufs = [moe.DevBuf.from_array(p["seeds"][0]), moe.DevBuf.from_array(p["coefs"][0]), moe.DevBuf.from_array(p["codes"][0])]
+        sh[i].p[0], sh[i].p[1], sh[i].p[3], sh[i].eb = bufs[0].ptr.value, bufs[1].ptr.value, bufs[2].ptr.value, int(p["eb"][0])
+        keep += bufs
+    shd = moe.DevBuf(C.sizeof(sh))
+    backend.check(L.nh_memcpy_h2d(shd.ptr, sh, C.c_size_t(C.sizeof(sh))), "h2d")
+    x0 = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
+    nw = moe.DevBuf.from_array((0.2 * rng.standard_normal(d)).astype(np.float32))
+    # separate launches
+    xa, xn, mo, a_, shv = moe.DevBuf.from_array(x0), moe.DevBuf(4 * T * d), moe.DevBuf(4 * T * d), moe.DevBuf(4 * T * ff), moe.DevBuf(4 * T * d)
+    sel0 = moe.DevBuf.from_array(np.zeros(T, dtype=np.int32))
+    L.kq4_norm1p.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_void_p, C.c_int]
+    L.kq4_norm1p(None, xa.ptr, d, d, nw.ptr, 1e-6, xn.ptr, T)
+    st.step(None, 0, xn.ptr, T, mo.ptr)
+    ws = backend.WSlice
+    L.kc_mv_gu(None, packs.MF_SEED4P4, shd.ptr, shd.at(C.sizeof(ws)), d, ff, xn.ptr, d, a_.ptr, ff, sel0.ptr, T, 1, None)
+    L.kc_mv(None, packs.MF_SEED4P4, sh[2], ff, d, a_.ptr, ff, shv.ptr, d, T, 0, None)
+    L.kc_residual_add(None, xa.ptr, mo.ptr, shv.ptr, C.c_size_t(T * d))
+    # the one launch
+    xb = moe.DevBuf.from_array(x0)
+    K.nslm_moe_step_layer.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.POINTER(ws), C.c_void_p, C.c_void_p, C.c_void_p, C.c_float]
+    assert K.nslm_moe_step_layer(st.h, None, 0, xb.ptr, T, sh, xb.ptr, xb.ptr, nw.ptr, 1e-6) == 0
+    moe.device_sync()
+    A, B = xa.to_array(np.float32, (T, d)), xb.to_array(np.float32, (T, d))
+    assert not np.array_equal(A, x0) and np.array_equal(A.view(np.uint32), B.view(np.uint32))
+    st.close()
