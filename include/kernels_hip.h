@@ -74,7 +74,7 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
 /* engine/kernels_cuda.h:81-82, engine/kernels_moe.cu:2317-2323.  Gather matvec over P (token, expert) pairs: pair p
  * uses slice sel[p] and input row p / xdiv. */
 /* No counterpart in the reference (its hosts launch kc_mv once per matrix): n <= 4 dense seed matrices w[j] ([R[j]][K]) against
- * the same T <= MV_MAXT rows of x in ONE launch, y[j][t * ys[j] + r] (+)= as kc_mv writes it, bit for bit.  0, or -1 when the
+ * the same T <= 64 rows of x in ONE launch per 8 rows, y[j][t * ys[j] + r] (+)= as kc_mv writes it, bit for bit.  0, or -1 when the
  * shapes are outside the seed fast path (K % 64, K > 6144, unaligned x): nothing is launched, call kc_mv per matrix.
  * norm_w (f32 [K], K <= 4096) or NULL: the rows of x are normalised first, exactly as kq4_norm1p(x, K, K, norm_w, norm_eps) would
  * have stored them (each workgroup recomputes the row's scale; the launch of the norm is saved). */

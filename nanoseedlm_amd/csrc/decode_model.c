@@ -262,10 +262,14 @@ int nslm_model_fill_cache(NslmModel* m, int T, int upto, uint64_t seed) {
     return nh_device_sync() || kc_last_error() ? -1 : 0;
 }
 
-/* y[T][R] (+)= W x: the matvec up to MV_MAXT rows, the packed MFMA GEMM above (engine/mova_cuda.c:1020-1028) */
+/* y[T][R] (+)= W x.  The reference takes the matvec up to MV_MAXT rows and the packed MFMA GEMM above
+ * (engine/mova_cuda.c:1020-1028).  Here the matvec (exact weights, f32 activations, passes of 8 rows) stays the choice up
+ * to DENSE_MV_ROWS rows: a 2048 x 2048 projection is a 32-workgroup grid for the GEMM's 64-row tiles (22 us at 16 rows),
+ * two matvec passes of 256 workgroups take about half of that. */
+#define DENSE_MV_ROWS 32
 static void dense(const NslmModel* m, kc_stream_t s, const Dense* dn, const float* x, const uint16_t* xp, int xs, float* y, int T, int add) {
     (void) m;
-    if (T <= MV_MAXT) kc_mv(s, MF_SEED4P4, dn->w, dn->K, dn->R, x, xs, y, dn->R, T, add, NULL);
+    if (T <= DENSE_MV_ROWS) kc_mv(s, MF_SEED4P4, dn->w, dn->K, dn->R, x, xs, y, dn->R, T, add, NULL);
     else kc_mm_packed(s, MF_SEED4P4, dn->w, dn->K, dn->R, xp, xs, y, dn->R, T, add, NULL);
 }
 
@@ -273,7 +277,7 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
     const NslmModelCfg* c = &m->c;
     if (!m->final || T < 1 || T > c->max_rows) return -1;
     const int d = c->d, H = c->n_head, hd = c->head_dim, r = c->r, rope = c->rope, QD = qd(c), ffs = c->ff_shared;
-    const int big = T > MV_MAXT;
+    const int big = T > MV_MAXT, bigd = T > DENSE_MV_ROWS;   /* rows above which the experts / the dense projections take the GEMMs */
     const size_t rows = cache_rows(c), e = kv_elem(c);
     MlaArgs ma;
     memset(&ma, 0, sizeof ma);
@@ -294,15 +298,18 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         const int par = m->branches && !big;
         kc_stream_t s1 = par ? (kc_stream_t) m->side[0] : s, s2 = par ? (kc_stream_t) m->side[1] : s;
         int one = 0;   /* steps of up to 8 rows on one stream: the norm and the three projections of its output as one launch */
-        if (!big && !par) {
-            const WSlice w3[3] = {dn[NSLM_W_Q].w, dn[NSLM_W_KVA].w, dn[NSLM_W_KR].w};
-            const int R3[3] = {QD, r, rope}, a3[3] = {0, 0, 0};
-            float* const y3[3] = {m->q, m->cl, m->kr};
-            one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->x, d, T, m->norm + (size_t) (2 * l) * d, c->eps);
-        }
+        const WSlice w3[3] = {dn[NSLM_W_Q].w, dn[NSLM_W_KVA].w, dn[NSLM_W_KR].w};
+        const int R3[3] = {QD, r, rope}, a3[3] = {0, 0, 0};
+        float* const y3[3] = {m->q, m->cl, m->kr};
+        if (!big && !par) one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->x, d, T, m->norm + (size_t) (2 * l) * d, c->eps);
         if (!one) {
             kq4_norm1p(s, m->x, d, d, m->norm + (size_t) (2 * l) * d, c->eps, m->xn, T);
-            if (big) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
+            /* more than 8 rows: the norm stays a launch (every workgroup of a pass would redo 8 rows' sums), the three
+               projections still go as one launch per 8 rows */
+            if (big && !bigd) one = !kc_mv_multi(s, MF_SEED4P4, 3, w3, R3, y3, R3, a3, d, m->xn, d, T, NULL, 0.0f);
+        }
+        if (!one) {
+            if (bigd) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
             /* with branches: [Q -> q RoPE mix] | [KV down, then q -> latent] | [K rope] */
             if (par) { fork_to(m, s, 0); fork_to(m, s, 1); }
             dense(m, s, &dn[NSLM_W_Q], m->xn, m->px, d, m->q, T, 0);
@@ -333,11 +340,12 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
             if (par) { join_from(m, s, 0); join_from(m, s, 1); }
             kc_mla_rope(s, ma, m->qr, m->kr, m->cl, kv, m->ri, m->inv, T);
         }
-        if (kc_mla_attn_vup(s, ma, m->ql, m->qr, kv, m->ri, m->part, hv, MF_BF16, hwv, m->o, T)) {
+        /* (above 8 rows the fused reduce re-reads the partials from too many workgroups: 19 us against 13 for the two kernels) */
+        if (big || kc_mla_attn_vup(s, ma, m->ql, m->qr, kv, m->ri, m->part, hv, MF_BF16, hwv, m->o, T)) {
             kc_mla_attn(s, ma, m->ql, m->qr, kv, m->ri, m->part, m->olat, T);
             kc_heads_mv(s, hv, MF_BF16, hwv, NULL, m->olat, NULL, m->o, T);
         }
-        if (big) kc_pack_input_bf16(s, m->o, m->pa, (size_t) T * QD);
+        if (bigd) kc_pack_input_bf16(s, m->o, m->pa, (size_t) T * QD);
         dense(m, s, &dn[NSLM_W_O], m->o, m->pa, QD, m->x, T, 1);   /* x = bf16(x + bf16(W_o o)) */
         /* ---- experts: x = bf16(x + bf16(sum_k wt_k y_k + shared(xn))) ---- */
         const WSlice* st = m->shared_tab + (size_t) l * 3;
@@ -358,11 +366,20 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
             if (par) join_from(m, s, 0);
         } else {
             if (nslm_moe_step(m->moe, s, l, m->xn, T, m->mo)) return -1;
-            kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
-            dense(m, s, &dn[NSLM_W_SG], m->xn, m->px, d, m->gs, T, 0);
-            dense(m, s, &dn[NSLM_W_SU], m->xn, m->px, d, m->us, T, 0);
+            int two = 0;   /* the shared expert's gate and up as one launch per 8 rows */
+            if (!bigd) {
+                const WSlice w2[2] = {dn[NSLM_W_SG].w, dn[NSLM_W_SU].w};
+                const int R2[2] = {ffs, ffs}, a2[2] = {0, 0};
+                float* const y2[2] = {m->gs, m->us};
+                two = !kc_mv_multi(s, MF_SEED4P4, 2, w2, R2, y2, R2, a2, d, m->xn, d, T, NULL, 0.0f);
+            }
+            if (!two) {
+                if (bigd) kc_pack_input_bf16(s, m->xn, m->px, (size_t) T * d);
+                dense(m, s, &dn[NSLM_W_SG], m->xn, m->px, d, m->gs, T, 0);
+                dense(m, s, &dn[NSLM_W_SU], m->xn, m->px, d, m->us, T, 0);
+            }
             kc_swiglu(s, m->gs, m->us, m->as, T * ffs);
-            kc_pack_input_bf16(s, m->as, m->pa, (size_t) T * ffs);
+            if (bigd) kc_pack_input_bf16(s, m->as, m->pa, (size_t) T * ffs);
             dense(m, s, &dn[NSLM_W_SD], m->as, m->pa, ffs, m->sh, T, 0);
         }
         kc_residual_add(s, m->x, m->mo, m->sh, (size_t) T * d);

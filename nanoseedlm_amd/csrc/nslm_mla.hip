@@ -656,7 +656,7 @@ __global__ void __launch_bounds__(128) k_mla_reduce(MlaArgs a, const RowInfo* ri
 // The splits' reduce and the value-up map of a head in ONE launch: workgroup (row group, head, row) reduces the head's
 // latent output into LDS (k_mla_reduce's arithmetic, all r dims: the map needs them all) and computes rows
 // [RG g, RG (g + 1)) of y[t][h] = bf16(W_h . olat[t][h]) (k_heads_mv's arithmetic).  The same bits as the two kernels.
-#define MLA_RV_GROUPS 16
+#define MLA_RV_GROUPS 16   // row groups a head at most: fewer when there are many (row, head) pairs, each group re-reads the partials
 __global__ void __launch_bounds__(256) k_mla_reduce_vup(MlaArgs a, const RowInfo* ri, const float* part, HmvArgs hv, int fmt, WSlice W, float* y,
                                                        int lpr) {
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
@@ -665,7 +665,7 @@ __global__ void __launch_bounds__(256) k_mla_reduce_vup(MlaArgs a, const RowInfo
     constexpr int PF = 32, NP = 2;   // splits / map passes whose loads are issued before anything waits
     const int g = (int) blockIdx.x, h = (int) blockIdx.y, t = (int) blockIdx.z, r = a.r, w = r + 2, ns = mla_row_splits(a, ri[t].pos), tid = threadIdx.x;
     const NSLM_GLOBAL float* pp = gp<float>(part) + ((size_t) t * a.n_head + h) * a.n_splits * w;
-    const int rg = (hv.O + MLA_RV_GROUPS - 1) / MLA_RV_GROUPS, o0 = g * rg, o1 = min(o0 + rg, hv.O);
+    const int rg = (hv.O + (int) gridDim.x - 1) / (int) gridDim.x, o0 = g * rg, o1 = min(o0 + rg, hv.O);
     const int rpw = 64 / lpr, sub = (tid & 63) / lpr, ln = tid & (lpr - 1);
     // Every load whose address is known now is in flight before the first wait: the splits' (m, l), this thread's two
     // output dims of the first PF splits, and (BF16 maps, one block a lane) the map rows of the first NP passes.
@@ -869,8 +869,10 @@ int kc_mla_attn_vup(kc_stream_t s, MlaArgs a, const float* ql, const float* qr, 
         (lpr != hv.I / 8 && hv.I / 8 <= 64) || hv.O < 1)
         return -1;
     if (!mla_attn_launch(s, a, ql, qr, kv, ri, part, NULL, T, false)) return -1;
-    hipLaunchKernelGGL(k_mla_reduce_vup, dim3(MLA_RV_GROUPS, (unsigned) a.n_head, (unsigned) T), dim3(256), 0, (hipStream_t) s, a, ri, part, hv, fmt, W,
-                       y, lpr);
+    int groups = 1024 / (a.n_head * T);   // about a thousand workgroups
+    groups = groups < 1 ? 1 : groups > MLA_RV_GROUPS ? MLA_RV_GROUPS : groups;
+    hipLaunchKernelGGL(k_mla_reduce_vup, dim3((unsigned) groups, (unsigned) a.n_head, (unsigned) T), dim3(256), 0, (hipStream_t) s, a, ri, part, hv, fmt,
+                       W, y, lpr);
     host_note_launch();
     return 0;
 }

@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     Chunk cur = fetch(v);
 
     load_tables(tab);
-    const bool prenorm = DN && a.nw != nullptr;   // uniform
+    const bool prenorm = MODE == MULTI && a.nw != nullptr;   // uniform; the other modes compile without it
     float xreg[NT == 1 ? 64 : 1];
     if (NT == 1) {
         const float rn = prenorm ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
@@ -111,15 +111,36 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
             }
         }
     } else {
-        for (int t = 0; t < a.nt; ++t) {
-            const float rn = prenorm ? row_rnorm(a.x + (size_t) t * a.xs, a.K, a.neps, nred) : 1.0f;
-            for (int i = tid; i < a.K / 4; i += 256) {
-                float4 q = ((const float4*) (a.x + (size_t) t * a.xs))[i];
+        // Stage nt rows of K floats: 8 loads in flight a thread before the first store (a loop of load-then-store over a
+        // run-time count waits for every load in turn).
+        __shared__ float rn_s[NT];
+        if (prenorm) {
+            for (int t = 0; t < a.nt; ++t) {
+                const float rn = row_rnorm(a.x + (size_t) t * a.xs, a.K, a.neps, nred);
+                if (tid == 0) rn_s[t] = rn;
+            }
+            __syncthreads();
+        }
+        const int K4 = a.K / 4, tot = a.nt * K4;
+        for (int base = tid; base < tot; base += 256 * 8) {
+            float4 q[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int idx = min(base + 256 * j, tot - 1), t = idx / K4, i = idx - t * K4;
+                q[j] = ((const float4*) (a.x + (size_t) t * a.xs))[i];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int idx = base + 256 * j;
+                if (idx >= tot) break;
+                const int t = idx / K4, i = idx - t * K4;
+                float4 v = q[j];
                 if (prenorm) {
                     const float4 w4 = ((const float4*) a.nw)[i];
-                    q.x = q.x * rn * (1.0f + w4.x); q.y = q.y * rn * (1.0f + w4.y); q.z = q.z * rn * (1.0f + w4.z); q.w = q.w * rn * (1.0f + w4.w);
+                    const float rn = rn_s[t];
+                    v.x = v.x * rn * (1.0f + w4.x); v.y = v.y * rn * (1.0f + w4.y); v.z = v.z * rn * (1.0f + w4.z); v.w = v.w * rn * (1.0f + w4.w);
                 }
-                *(float4*) &xl[(t * L + (i >> 4)) * XPAD + (i & 15) * 4] = q;
+                *(float4*) &xl[(t * L + (i >> 4)) * XPAD + (i & 15) * 4] = v;
             }
         }
     }
@@ -464,7 +485,10 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
 
 void note_launch() { nslm::host_note_launch(); }
 
-#define MV_TG 4   // tokens per pass of the multi-token fast path (activations staged in LDS)
+#define MV_TG 4   // tokens per pass of the multi-token fast path (activations staged in LDS); MV_TG2 when more than MV_TG remain
+#define MV_TG2 8
+#define MV_TG3 16   // one pass of 16 when the rows fit the LDS (K <= 2176): small matrices leave one workgroup a CU anyway
+#define MV_MULTI_MAXT 64
 
 }   // namespace
 
@@ -502,13 +526,19 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         // Tokens go in passes of at most MV_TG; a token's arithmetic is the same in every pass size.  Rows too long for
         // the LDS staging take one pass per token with the activations in registers.
         const bool stage = T > 1 && L <= 96;
-        for (int t0 = 0; t0 < T; t0 += stage ? MV_TG : 1) {
+        const bool wide8 = stage && (size_t) MV_TG2 * L * XPAD * sizeof(float) <= 72 * 1024;   // two workgroups a CU still fit
+        for (int t0 = 0; t0 < T;) {
             MvArgs b = a;
             b.x = x + (size_t) t0 * xs;
             b.y = y + (size_t) t0 * ys;
-            b.nt = stage ? (T - t0 < MV_TG ? T - t0 : MV_TG) : 1;
-            if (stage) launch_seed_fmt<DENSE, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
+            const bool wide16 = wide8 && (size_t) MV_TG3 * L * XPAD * sizeof(float) <= 150 * 1024;
+            const int tg = !stage ? 1 : (wide16 && T - t0 > MV_TG2) ? MV_TG3 : (wide8 && T - t0 > MV_TG) ? MV_TG2 : MV_TG;
+            b.nt = T - t0 < tg ? T - t0 : tg;
+            if (tg == MV_TG3) launch_seed_fmt<DENSE, MV_TG3>(st, fmt, b, shfl, grid, (size_t) MV_TG3 * L * XPAD * sizeof(float));
+            else if (tg == MV_TG2) launch_seed_fmt<DENSE, MV_TG2>(st, fmt, b, shfl, grid, (size_t) MV_TG2 * L * XPAD * sizeof(float));
+            else if (stage) launch_seed_fmt<DENSE, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
             else launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid, 0);
+            t0 += tg;
         }
         note_launch();
         return;
@@ -523,7 +553,7 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
                 const float* x, int xs, int T, const float* norm_w, float norm_eps) {
     int L, rpi;
     bool shfl;
-    if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;
+    if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MULTI_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;
     if (norm_w && (K > 256 * 16 || !aligned16(norm_w))) return -1;
     MvArgs a = {};
     a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n; a.nw = norm_w; a.neps = norm_eps;
@@ -537,13 +567,19 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     }
     const dim3 grid((unsigned) a.wg0[n], 1);
     hipStream_t st = (hipStream_t) s;
-    for (int t0 = 0; t0 < T; t0 += T > 1 ? MV_TG : 1) {   // passes of tokens as kc_mv's: a token's arithmetic is the same in either
+    const bool wide8 = (size_t) MV_TG2 * L * XPAD * sizeof(float) <= 72 * 1024;
+    for (int t0 = 0; t0 < T;) {   // passes of tokens as kc_mv's: a token's arithmetic is the same in every pass size
         MvArgs b = a;
         b.x = x + (size_t) t0 * xs;
         for (int j = 0; j < n; ++j) b.yj[j] = y[j] + (size_t) t0 * ys[j];
-        b.nt = T > 1 ? (T - t0 < MV_TG ? T - t0 : MV_TG) : 1;
-        if (T > 1) launch_seed_fmt<MULTI, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
+        const bool wide16 = wide8 && (size_t) MV_TG3 * L * XPAD * sizeof(float) <= 150 * 1024;
+        const int tg = T == 1 ? 1 : (wide16 && T - t0 > MV_TG2) ? MV_TG3 : (wide8 && T - t0 > MV_TG) ? MV_TG2 : MV_TG;
+        b.nt = T - t0 < tg ? T - t0 : tg;
+        if (tg == MV_TG3) launch_seed_fmt<MULTI, MV_TG3>(st, fmt, b, shfl, grid, (size_t) MV_TG3 * L * XPAD * sizeof(float));
+        else if (tg == MV_TG2) launch_seed_fmt<MULTI, MV_TG2>(st, fmt, b, shfl, grid, (size_t) MV_TG2 * L * XPAD * sizeof(float));
+        else if (tg == MV_TG) launch_seed_fmt<MULTI, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
         else launch_seed_fmt<MULTI, 1>(st, fmt, b, shfl, grid, 0);
+        t0 += tg;
     }
     note_launch();
     return 0;

@@ -66,14 +66,35 @@ __device__ __forceinline__ void chunk_dot(const Chunk& ck, int eb, const uint32_
         float w[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) w[c] = (float) is[c];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (NT > 1 && t >= nt) break;
-            const float* xb = xr + t * xstride + 8 * b;
+        if constexpr (NT == 1) {   // one token: its activations are in registers (or one LDS row)
+            const float* xb = xr + 8 * b;
             float d = w[0] * xb[0];
 #pragma unroll
             for (int c = 1; c < 8; ++c) d = fmaf(w[c], xb[c], d);
-            acc[t] = fmaf(d, e2, acc[t]);
+            acc[0] = fmaf(d, e2, acc[0]);
+        } else {
+            // Every token of the pass is computed (rows past nt hold whatever the LDS holds; their sums are never stored):
+            // an early exit on the run-time count would make each token's LDS reads wait for the one before.
+            (void) nt;
+            float4 xa[NT][2];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float* xb = xr + t * xstride + 8 * b;
+                xa[t][0] = *(const float4*) xb;
+                xa[t][1] = *(const float4*) (xb + 4);
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                float d = w[0] * xa[t][0].x;
+                d = fmaf(w[1], xa[t][0].y, d);
+                d = fmaf(w[2], xa[t][0].z, d);
+                d = fmaf(w[3], xa[t][0].w, d);
+                d = fmaf(w[4], xa[t][1].x, d);
+                d = fmaf(w[5], xa[t][1].y, d);
+                d = fmaf(w[6], xa[t][1].z, d);
+                d = fmaf(w[7], xa[t][1].w, d);
+                acc[t] = fmaf(d, e2, acc[t]);
+            }
         }
     }
 }

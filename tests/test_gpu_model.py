@@ -29,13 +29,14 @@ def norm_ref(x, w, eps):
     return (x / np.sqrt(np.mean(x * x) + eps) * (1.0 + f64(w))).astype(np.float32)
 
 
-@pytest.mark.parametrize("T,branches", [(2, False), (2, True), (12, False)])
+@pytest.mark.parametrize("T,branches", [(2, False), (2, True), (12, False), (40, False)])
 @pytest.mark.parametrize("kv", ["bf16", "fp8"])
 def test_tiny_model_decode(oracle, kv, T, branches):
     from nanoseedlm_amd import backend, model, moe
     backend.require_gpu()
     rng = np.random.default_rng(2024 + T)
-    gemm = T > 8                                                       # above 8 rows the step runs the packed GEMMs
+    gemm = T > 8                                                       # above 8 rows the experts, router and LM head run the packed GEMMs
+    dgemm = T > 32                                                     # the dense projections stay matvecs (exact weights) up to 32 rows
     cfg = dict(n_layer=2, d=128, n_head=2, head_dim=64, r=64, rope=64, n_exp=8, top_k=2, ff=64, ff_shared=64, vocab=96, max_ctx=16,
                max_rows=T, kv_fmt=backend.KV_FP8 if kv == "fp8" else backend.KV_BF16, n_splits=2, eps=1e-6, rope_theta=10000.0)
     m = model.DecodeModel(**cfg)
@@ -89,9 +90,9 @@ def test_tiny_model_decode(oracle, kv, T, branches):
             x = embf[ids[t]].copy()
             for l in range(L):
                 xn = norm_ref(x, Wn[l, 0], cfg["eps"])
-                q = dense_ref(oracle, Wd[l, model.W_Q], xn, gemm)
-                c = dense_ref(oracle, Wd[l, model.W_KVA], xn, gemm)
-                kr = dense_ref(oracle, Wd[l, model.W_KR], xn, gemm)
+                q = dense_ref(oracle, Wd[l, model.W_Q], xn, dgemm)
+                c = dense_ref(oracle, Wd[l, model.W_KVA], xn, dgemm)
+                kr = dense_ref(oracle, Wd[l, model.W_KR], xn, dgemm)
                 qr = oracle.heads_map(packs.bf16_bits_to_f32(Wh[l, model.H_QRMIX]).reshape(H * rope, hd), q[None], H, rope, hd, QD, hd)[0]
                 ql = oracle.heads_map(packs.bf16_bits_to_f32(Wh[l, model.H_QLAT]).reshape(H * r, hd), q[None], H, r, hd, QD, hd)[0]
                 half = rope // 2
@@ -106,7 +107,7 @@ def test_tiny_model_decode(oracle, kv, T, branches):
                 kr_c[l, t, pos[t]] = cache_value(krot)
                 olat = np.stack([oracle.mla_attn(ql[h], qrot[h], lat_c[l, t], kr_c[l, t], int(pos[t]), float(scale)) for h in range(H)])
                 o = oracle.heads_map(packs.bf16_bits_to_f32(Wh[l, model.H_VUP]).reshape(H * hd, r), olat.reshape(1, H * r), H, hd, r, H * r, r)[0]
-                x = r_(x + dense_ref(oracle, Wd[l, model.W_O], o.reshape(-1), gemm))
+                x = r_(x + dense_ref(oracle, Wd[l, model.W_O], o.reshape(-1), dgemm))
                 xn = norm_ref(x, Wn[l, 1], cfg["eps"])
                 gate, up, down, rw = Wx[l]
                 xe = r_(xn) if gemm else xn
@@ -114,11 +115,11 @@ def test_tiny_model_decode(oracle, kv, T, branches):
                 ind, wt = oracle.route_softmax(lg[None], k)
                 ys = np.stack([expert_ref(oracle, gate, up, down, int(ind[0, j]), xe, gemm=gemm) for j in range(k)])
                 mo = (f64(wt[0])[:, None] * ys).sum(0)
-                g = dense_ref(oracle, Wd[l, model.W_SG], xn, gemm)
-                u = dense_ref(oracle, Wd[l, model.W_SU], xn, gemm)
+                g = dense_ref(oracle, Wd[l, model.W_SG], xn, dgemm)
+                u = dense_ref(oracle, Wd[l, model.W_SU], xn, dgemm)
                 sg = r_((1 / (1 + np.exp(-f64(g)))).astype(np.float32))
                 a = r_(r_(g * sg) * u)
-                sh = dense_ref(oracle, Wd[l, model.W_SD], a, gemm)
+                sh = dense_ref(oracle, Wd[l, model.W_SD], a, dgemm)
                 x = r_(x + r_((mo + f64(sh)).astype(np.float32)))
             xn = norm_ref(x, Wn[L, 0], cfg["eps"])
             want = r_((f64(embf) @ f64(r_(xn) if gemm else xn)).astype(np.float32))
