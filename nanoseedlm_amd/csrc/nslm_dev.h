@@ -271,7 +271,8 @@ __device__ __forceinline__ float row_rnorm(const float* xi, int g, float eps, fl
 #pragma unroll
     for (int j = 0; j < NSLM_NORM_NR; ++j) {
         const int k = (int) threadIdx.x + j * 256;
-        const float v = k < g ? xi[k] : 0.0f;
+        const float xv = xi[min(k, g - 1)];   // unconditional (a conditional load waits for the loads before it)
+        const float v = k < g ? xv : 0.0f;
         ss = fmaf(v, v, ss);
     }
     return rsqrtf(wg_sum(ss, red) / (float) g + eps);

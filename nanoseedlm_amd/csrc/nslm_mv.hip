@@ -90,23 +90,29 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     const bool prenorm = MODE == MULTI && a.nw != nullptr;   // uniform; the other modes compile without it
     float xreg[NT == 1 ? 64 : 1];
     if (NT == 1) {
-        const float rn = prenorm ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
+        // The row's scale first, while few registers are live (its 16 loads then go out back to back; issued beside the
+        // 128 registers of row and weight data the allocator serialised them), then the row and the norm weights together.
+        const float rn = (MODE == MULTI && prenorm) ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
         if (active) {
             const float4* xp = (const float4*) (xrow + (size_t) ch * 64);
+            float4 wq[MODE == MULTI ? 16 : 1];
+            if (MODE == MULTI && prenorm) {
+                const float4* wp = (const float4*) (a.nw + (size_t) ch * 64);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) wq[i] = wp[i];
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const float4 q = xp[i];
                 xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
             }
-            if (prenorm) {
-                const float4* wp = (const float4*) (a.nw + (size_t) ch * 64);
+            if (MODE == MULTI && prenorm) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const float4 w4 = wp[i];
-                    xreg[4 * i] = xreg[4 * i] * rn * (1.0f + w4.x);
-                    xreg[4 * i + 1] = xreg[4 * i + 1] * rn * (1.0f + w4.y);
-                    xreg[4 * i + 2] = xreg[4 * i + 2] * rn * (1.0f + w4.z);
-                    xreg[4 * i + 3] = xreg[4 * i + 3] * rn * (1.0f + w4.w);
+                    xreg[4 * i] = xreg[4 * i] * rn * (1.0f + wq[i].x);
+                    xreg[4 * i + 1] = xreg[4 * i + 1] * rn * (1.0f + wq[i].y);
+                    xreg[4 * i + 2] = xreg[4 * i + 2] * rn * (1.0f + wq[i].z);
+                    xreg[4 * i + 3] = xreg[4 * i + 3] * rn * (1.0f + wq[i].w);
                 }
             }
         }
