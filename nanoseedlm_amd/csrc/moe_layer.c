@@ -325,3 +325,4 @@ uint64_t nslm_moe_expert_bytes(const NslmMoe* m) {
         for (int s = 0; s < 4; ++s) n += m->stream_len[i][s];
     return n;
 }
+

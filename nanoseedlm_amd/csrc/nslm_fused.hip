@@ -49,10 +49,13 @@ struct FusedArgs {
 //   [32 BAR_GROUPS]     groups that are complete
 //   [32 (BAR_GROUPS+1+g)] group g's sense word: flipped when the barrier opens
 //   [32 (2 BAR_GROUPS+1)] error word
-//   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile)
+//   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile); behind them (at T (d + 1)) three words per pair, each on
+//                        its own line: finished gate+up items (atomics only), the pair's ready flag (what waiters
+//                        poll: polling the counter's line would slow the arrivals), finished down items
 // Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
 // counters and only each group's last arrival touches the shared one; waiters poll their own group's sense word.  The
-// barrier is sense-reversing and resets its own counters, so the words need no clean-up between launches.
+// barrier is sense-reversing (each group's word flips from its own value, so launches with different numbers of groups
+// and any number of barriers a launch can follow each other) and resets its own counters: no clean-up between launches.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
 #define FUSED_SYNC_WORDS (32 * (2 * BAR_GROUPS + 2))
@@ -79,7 +82,15 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G) {
             if (atomicAdd(sync + 32 * BAR_GROUPS, 1u) == ng - 1) {
                 st_agent(sync + 32 * BAR_GROUPS, 0u);
                 wg_release();   // every counter is back at zero before anyone is let through
-                for (uint32_t i = 0; i < ng; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), s ^ 1u);
+                // Each group's word flips from ITS OWN value: launches of different grid sizes use different numbers of
+                // groups, so after an odd number of barriers the words need not agree with each other.
+                // (all the words are read before any is written: 32 independent loads, then 32 stores)
+                uint32_t cur[BAR_GROUPS];
+#pragma unroll
+                for (uint32_t i = 0; i < BAR_GROUPS; ++i) cur[i] = ld_agent(sync + 32 * (BAR_GROUPS + 1 + i));
+#pragma unroll
+                for (uint32_t i = 0; i < BAR_GROUPS; ++i)
+                    if (i < ng) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), cur[i] ^ 1u);
             }
         }
         uint32_t spins = 0;
@@ -195,6 +206,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     load_tables(tab);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
+    uint32_t* pairc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [pair][3][32]: arrivals, ready, done
     if (a.nw) {   // uniform: every workgroup forms every row's scale (T rows of d values from L2)
         for (int t = 0; t < a.T; ++t) {
             const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
@@ -299,6 +311,9 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         float* Ap = a.A + (size_t) p * a.ff;
         rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
                                    [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
+        wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
+        __syncthreads();
+        if (tid == 0 && atomicAdd(&pairc[p * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&pairc[p * 96 + 32], 1u);   // the pair's A is complete
     }
     // tokens whose routing nobody needed here still get published by their designated workgroup
     for (int t = (int) blockIdx.x; t < a.T; t += (int) G) route(t);
@@ -313,14 +328,26 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         route(t);
         d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.rows_d, min(tile * a.rows_d + a.rows_d, a.d));
     }
-    grid_barrier(a.sync, G);
-    STAMP(4);
+    // No grid barrier here: a down item needs its own pair's A only, so it waits for that pair's gate+up items (every
+    // workgroup finishes its gate+up items before it waits, and the whole grid is resident, so the wait ends; bounded anyway).
     for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
         const int p = item / a.ntile_d, tile = item - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
         const int v0 = tile * a.rows_d, v1 = min(v0 + a.rows_d, a.d);
         if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
+        if (tid == 0) {
+            uint32_t spins = 0;
+            while (ld_agent(&pairc[p * 96 + 32]) == 0u) {
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > SPIN_LIMIT) {
+                    atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                    break;
+                }
+            }
+        }
         __syncthreads();
+        wg_acquire();
+        if (item == (int) blockIdx.x) STAMP(4);   // the first down item's pair is ready
         stage_row(a.A + (size_t) p * a.ff, a.ff, xl, true);
         staged = -1;
         __syncthreads();
@@ -339,6 +366,12 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
                 a.out[(size_t) t * a.os + r] = a.res ? bfr(a.res[(size_t) t * a.os + r] + bfr(acc)) : acc;
             }
             if (tid == 0) st_agent(&tick[t * a.ntile_d + tile], 0u);
+        }
+        // the pair's last down item leaves its three words at zero for the next launch (everyone has read them by then)
+        if (tid == 0 && atomicAdd(&pairc[p * 96 + 64], 1u) == (uint32_t) (a.ntile_d - 1)) {
+            st_agent(&pairc[p * 96], 0u);
+            st_agent(&pairc[p * 96 + 32], 0u);
+            st_agent(&pairc[p * 96 + 64], 0u);
         }
     }
     STAMP(5);
@@ -396,7 +429,7 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
 
 extern "C" {
 
-size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1); }
+size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1) + (size_t) T * 33 * 96; }
 int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
 
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
