@@ -44,7 +44,7 @@ def traffic_of(workload):
 
 class Q4Projections:
     """Config 3's affine-int4 side of the layer: q / k / v / o and the shared expert's gate / up / down, each d x d, Q4
-    group 64 (BF16 scale ~U(0.005, 0.02), zero point uniform [0, 15] stored as bias = -z * scale).  BASELINE gives no
+    group 64 (BF16 scale ~U(0.005, 0.02), zero point uniform [0, 15] stored as bias = -z * scale).  The benchmark definition gives no
     shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs up to 8 tokens, the packed
     MFMA GEMM above (as the reference's enc_dense / enc_dense_packed choose, engine/mova_cuda.c:1020-1028)."""
 

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes, on the GPU.
+"""The benchmark configurations at their full sizes, on the GPU.
 
 Where the oracle finishes in seconds the whole result is compared (C0, and the C2 layer step on the experts the GPU chose);
 for the 60-GFLOP prefill GEMM a random sample of weight rows is checked against the oracle over every token, and the whole
