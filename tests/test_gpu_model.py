@@ -133,3 +133,39 @@ def test_tiny_model_decode(oracle, kv, T, branches):
     m.close()
     print("worst relative logit error", worst, "layers moved the stream by", moved, "tokens seen", sorted(seen))
     assert moved > 0.3, "the layers must matter to the logits for this comparison to test them"
+
+
+@pytest.mark.parametrize("T", [2, 12])
+def test_graph_replay_equals_eager_steps(T):
+    """The step captured once in a hipGraph and replayed (positions and ids live on the device) gives the bits of eager
+    launches at every step, with eager work and synchronisations of another model between the replays."""
+    from nanoseedlm_amd import backend, model, moe
+    backend.require_gpu()
+    cfg = dict(n_layer=2, d=128, n_head=2, head_dim=64, r=64, rope=64, n_exp=8, top_k=2, ff=64, ff_shared=64, vocab=96, max_ctx=24,
+               max_rows=T, kv_fmt=backend.KV_FP8, n_splits=2, eps=1e-6, rope_theta=10000.0)
+    rng = np.random.default_rng(5)
+    ids, pos = rng.integers(0, cfg["vocab"], T).astype(np.int32), rng.integers(0, 6, T).astype(np.int32)
+    ms = []
+    for _ in range(2):
+        m = model.DecodeModel(**cfg)
+        m.fill_random(seed=11, eb=-13)
+        m.start(ids, pos)
+        ms.append(m)
+    eager, replay = ms
+    stream = moe.new_stream()
+    replay.step(stream, T)                                           # warm every kernel, then rewind and capture
+    moe.device_sync()
+    replay.start(ids, pos)
+    g = replay.graph_of_step(stream, T)
+    seen = set()
+    for step in range(6):
+        eager.step(None, T)
+        a, ia = eager.logits(T), eager.ids(T)
+        replay.launch(g, stream)
+        moe.device_sync()
+        b, ib = replay.logits(T), replay.ids(T)
+        assert np.isfinite(a).all() and np.array_equal(a.view(np.uint32), b.view(np.uint32)) and np.array_equal(ia, ib), step
+        seen.add(a.tobytes())
+    assert len(seen) == 6                                            # the steps differ from one another (positions advance)
+    for m in ms:
+        m.close()
