@@ -136,7 +136,7 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
         const Chunk nxt = fetch(v + rpi);
         float acc[1] = {0.0f};
         const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
-        if (active && v < v1) chunk_dot<P, 1>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
+        if (active && v < v1) chunk_dot<P, 1, true>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
         if (SHFL) {
             float s = acc[0];
             for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
