@@ -72,3 +72,27 @@ def test_layer_step_from_a_folder(tmp_path, fmt, E, d, ff):
         st.close()
     mf.close()
     assert np.abs(outs[0]).max() > 0 and np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
+def test_upload_of_a_stream_longer_than_the_staging_buffers(tmp_path):
+    """nsf_upload stages through two 8 MiB pinned buffers: a 20 MB stream, from an odd offset, arrives byte for byte."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, folder, moe
+    backend.require_gpu()
+    rng = np.random.default_rng(9)
+    big = rng.integers(0, 65536, (2560, 4096), dtype=np.uint16)       # 20 MiB of BF16 bit patterns
+    write_folder(tmp_path, {"big": [(".weight", "BF16", big)]})
+    mf = folder.ModelFolder(tmp_path)
+    t = mf.find("big.weight")
+    assert t.s[0].len == big.nbytes
+    K = backend.kt()
+    K.nsf_upload.argtypes = [C.c_void_p, C.POINTER(folder.Stream), C.c_uint64, C.c_uint64]
+    raw = big.view(np.uint8).reshape(-1)
+    for skip, n in ((0, big.nbytes), (12345, 17 * 1024 * 1024 + 77), (big.nbytes - 5, 5)):
+        dst = moe.DevBuf(n)
+        assert K.nsf_upload(dst.ptr, C.byref(t.s[0]), skip, n) == 0
+        assert np.array_equal(dst.to_array(np.uint8, (n,)), raw[skip:skip + n])
+        dst.free()
+    dst = moe.DevBuf(16)
+    assert K.nsf_upload(dst.ptr, C.byref(t.s[0]), big.nbytes - 4, 8) == -1          # past the end of the stream
+    mf.close()
