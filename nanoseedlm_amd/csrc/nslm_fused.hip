@@ -39,8 +39,8 @@ struct FusedArgs {
     const float* res;                   // non-null: out = bf16(res + bf16(sum)) (the residual stream; may alias out)
     const float* nw;                    // non-null: x is normalised first, xn_k = x_k r (1 + nw_k), r = rsqrt(mean(x^2) + neps)
     float neps;
-    int Lg, rpig, rows_g, ntile_g;      // gate+up pass: chunks per row, virtual rows per iteration / per item, items per pair
-    int Ld, rpid, rows_d, ntile_d;      // down pass
+    int Lg, rpig, it_g, ntile_g;        // gate+up pass: chunks per row, virtual rows per iteration, iterations and items per pair
+    int Ld, rpid, it_d, ntile_d;        // down pass (item i of a pair owns iterations i it / ntile .. (i + 1) it / ntile)
     int grid;
 };
 
@@ -300,7 +300,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
-        const int v0 = tile * a.rows_g, v1 = min(v0 + a.rows_g, 2 * a.ff);
+        const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
         if (staged != t) {
             __syncthreads();
@@ -326,14 +326,14 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     if ((int) blockIdx.x < items_d) {
         const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
-        d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.rows_d, min(tile * a.rows_d + a.rows_d, a.d));
+        d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.it_d / a.ntile_d * a.rpid, min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d));
     }
     // No grid barrier here: a down item needs its own pair's A only, so it waits for that pair's gate+up items (every
     // workgroup finishes its gate+up items before it waits, and the whole grid is resident, so the wait ends; bounded anyway).
     for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
         const int p = item / a.ntile_d, tile = item - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
-        const int v0 = tile * a.rows_d, v1 = min(v0 + a.rows_d, a.d);
+        const int v0 = tile * a.it_d / a.ntile_d * a.rpid, v1 = min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d);
         if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
         if (tid == 0) {
             uint32_t spins = 0;
@@ -411,13 +411,28 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
         per_cu = 0;
         return -1;
     }
-    // the grid must be resident at once: all the device holds, but no more than the work can use
-    int grid = (per_cu < 3 ? per_cu : 3) * cu_count();
-    const int items = a.T * a.kk * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
-    // A phase with a few items more than workgroups would leave stragglers a whole second item long (C2 at one token:
-    // 784 down-row items on 768 workgroups); when the device can hold them, a few extra workgroups cost less.
-    if (items > grid && items <= grid + grid / 8 && items <= per_cu * cu_count()) grid = items;
-    if (grid > items) grid = items;
+    // The grid must be resident at once (the kernel has a grid barrier): at most what the device holds, and no more than
+    // five workgroups a CU (the most that was tried).  Items per pair (an item = a run of a pair's iterations, as
+    // equal as whole iterations allow): the count that gives the busiest workgroup the least to do, an item's set-up priced
+    // at a third of an iteration and unequal items at half an iteration (workgroups i, i + 256, ... share a CU, so the long
+    // items of a regular pattern meet on the same CUs).  Measured on C2: one token, 96 x 2 gate+up iterations and 98 x 1 down
+    // iterations a pair on 784 workgroups, 40.1 us (96 unequal down items on 768 workgroups: 42.9); 8 tokens, 20 items a
+    // pair on 1280 workgroups, 139.6 us (768 workgroups, 24 and 13 items of 8 iterations: 163.7).
+    const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
+    auto pick = [&](int iters) {
+        int best = 1;
+        long best_cost = -1;
+        for (int n = 1; n <= iters; ++n) {
+            const long rounds = ((long) P_ * n + gmax - 1) / gmax, per = (iters + n - 1) / n;
+            const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
+            if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }   // ties: more, shorter items
+        }
+        return best;
+    };
+    a.ntile_g = pick(a.it_g);
+    a.ntile_d = pick(a.it_d);
+    const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
+    int grid = items < gmax ? (int) items : gmax;
     if (grid < 1) grid = 1;
     a.grid = grid;
     hipLaunchKernelGGL(kern, dim3((unsigned) grid), dim3(256), lds, st, a);
@@ -453,27 +468,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     a.ns = shared ? 1 : 0; a.kk = top_k + a.ns; a.res = res; a.nw = norm_w; a.neps = norm_eps;
     if (norm_w && (d > 256 * 16 || ((uintptr_t) norm_w & 15u))) return -1;
     for (int i = 0; i < 3 && shared; ++i) a.sh[i] = shared[i];
-    // Iterations per item (an item = one pair's row tile): the count that gives the busiest workgroup of a full grid the
-    // fewest iterations, an item's set-up priced at a third of an iteration; a few items over the grid count as one round
-    // (the launch adds workgroups for them).
-    const int full = 3 * cu_count(), P_ = T * a.kk;
-    const int it_g = (2 * ff + a.rpig - 1) / a.rpig, it_d = (d + a.rpid - 1) / a.rpid;
-    auto pick = [&](int iters) {
-        int best = 1;
-        long best_cost = -1;
-        for (int per = 1; per <= 8; ++per) {
-            const long items = (long) P_ * ((iters + per - 1) / per);
-            const long rounds = items <= full + full / 8 ? 1 : (items + full - 1) / full;
-            const long cost = rounds * (3 * per + 1);
-            if (best_cost < 0 || cost < best_cost) { best = per; best_cost = cost; }
-        }
-        return best;
-    };
-    const int per_g = pick(it_g), per_d = pick(it_d);
-    a.rows_g = per_g * a.rpig;
-    a.ntile_g = (2 * ff + a.rows_g - 1) / a.rows_g;
-    a.rows_d = per_d * a.rpid;
-    a.ntile_d = (d + a.rows_d - 1) / a.rows_d;
+    a.it_g = (2 * ff + a.rpig - 1) / a.rpig;
+    a.it_d = (d + a.rpid - 1) / a.rpid;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
