@@ -178,10 +178,10 @@ __device__ __forceinline__ void stage_input(const float* src, int n, float* xl, 
 }
 
 #ifdef NSLM_FUSED_STAMPS
-__device__ unsigned long long g_fstamp[1024 * 8];
+__device__ unsigned long long g_fstamp[1024 * 16];
 #endif
 template <int P, bool SHFL_G, bool SHFL_D>
-__global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
+__global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five waves a SIMD: at most 96 registers
     extern __shared__ float xl[];   // activations of the current pair: max(d, ff) floats, chunk-padded
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[2][256];
@@ -197,8 +197,8 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
     unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
 #ifdef NSLM_FUSED_STAMPS   // development builds: every workgroup's timeline
-#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 8 + (i)] = wall_clock64(); } } while (0)
-    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 8 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } } while (0)
+    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 16 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
 #else
 #define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
 #endif
@@ -262,20 +262,57 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         const int E4 = (a.E + 3) & ~3;
         for (int e = tid; e < E4; e += 256) rv[e] = e < a.E ? ld_agent(a.logits + (size_t) t * a.E + e) : __uint_as_float(0xFF800000u);
         __syncthreads();
-        for (int e = tid; e < a.E; e += 256) {
-            const float v = rv[e];
-            int rank = 0;
-#pragma unroll 8
-            for (int o = 0; o < E4; o += 4) {
-                const float4 u = *(const float4*) &rv[o];
-                rank += (u.x > v || (u.x == v && o > e)) ? 1 : 0;
-                rank += (u.y > v || (u.y == v && o + 1 > e)) ? 1 : 0;
-                rank += (u.z > v || (u.z == v && o + 2 > e)) ? 1 : 0;
-                rank += (u.w > v || (u.w == v && o + 3 > e)) ? 1 : 0;
+        unsigned long long tq[4] = {0, 0, 0, 0};
+        (void) tq;
+#ifdef NSLM_FUSED_STAMPS
+        tq[0] = wall_clock64();
+#endif
+        // The logits are BF16 values (phase 1 rounds them), so the upper half of a float's order-preserving integer image
+        // holds all of a logit and the lower half is free for the expert's index: one 32-bit key whose integer order is the
+        // routing order, and no two keys are equal.  rank(e) = number of larger keys.  Up to 256 experts: thread (e, part)
+        // counts over its part of the experts (keys read four at a time as LDS broadcasts: two instructions a compare) and
+        // the parts' counts are added.  Every instruction counts here, scalar ones too: the workgroups of a CU rank at the
+        // same moment, and wave-wide compares with scalar population counts took 3 to 6 us of every workgroup's time.
+        auto key_of = [&](int o) {
+            const uint32_t b = __float_as_uint(rv[o] + 0.0f);   // -0 counts as +0, as in a float compare
+            return ((b ^ ((uint32_t) ((int32_t) b >> 31) | 0x80000000u)) & 0xFFFF0000u) | (uint32_t) o;
+        };
+        if (a.E <= 256) {
+            uint32_t* pk = (uint32_t*) &part[0][0];   // keys (0 = absent, below every real key)
+            int* gp = (int*) &part[1][0];             // the parts' counts, [part][expert]
+            pk[tid] = tid < a.E ? key_of(tid) : 0u;
+            __syncthreads();
+            const int epad = a.E <= 64 ? 64 : a.E <= 128 ? 128 : 256, len = epad * epad / 256;
+            const int e = tid & (epad - 1), o0 = tid / epad * len;
+            const uint32_t ke = pk[e];
+            int g = 0;
+#pragma unroll 4
+            for (int o = o0; o < o0 + len; o += 4) {
+                const uint4 q = *(const uint4*) &pk[o];
+                g += (q.x > ke ? 1 : 0) + (q.y > ke ? 1 : 0) + (q.z > ke ? 1 : 0) + (q.w > ke ? 1 : 0);
             }
-            if (rank < a.k) ri_s[rank] = e;
+            gp[tid] = g;
+            __syncthreads();
+            if (tid < a.E) {
+                int rank = 0;
+                for (int q = tid; q < 256; q += epad) rank += gp[q];
+                if (rank < a.k) ri_s[rank] = tid;
+            }
+        } else {   // a wave takes the experts one at a time
+            for (int e = wv; e < a.E; e += 4) {
+                const uint32_t ke = __builtin_amdgcn_readfirstlane(key_of(e));
+                int rank = 0;
+                for (int o = lane; o < E4 + 63; o += 64) rank += __popcll(__ballot(o < a.E && key_of(o < 1024 ? o : 1023) > ke));
+                if (rank < a.k && lane == 0) ri_s[rank] = e;
+            }
         }
+#ifdef NSLM_FUSED_STAMPS
+        tq[1] = wall_clock64();
+#endif
         __syncthreads();
+#ifdef NSLM_FUSED_STAMPS
+        tq[2] = wall_clock64();
+#endif
         if (tid < 3 * a.k) {   // the chosen experts' slices, fetched side by side
             const int which = tid / a.k, j = tid - which * a.k;
             sl_s[which][j] = (which == 0 ? a.gate : which == 1 ? a.up : a.down)[ri_s[j]];
@@ -283,6 +320,10 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
         if (a.ns && tid >= 253) sl_s[tid - 253][a.k] = a.sh[tid - 253];
         if (tid < a.k) rw_s[tid] = expf(rv[ri_s[tid]] - rv[ri_s[0]]);
         __syncthreads();
+#ifdef NSLM_FUSED_STAMPS
+        tq[3] = wall_clock64();
+        if (tid == 0 && blockIdx.x < 1024) for (int q = 0; q < 4; ++q) g_fstamp[blockIdx.x * 16 + 11 + q] = tq[q];
+#endif
         if (tid < a.k) {
             float top = 0.0f;
             for (int r = 0; r < a.k; ++r) top += rw_s[r];
@@ -300,6 +341,7 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
+        if (item == (int) blockIdx.x) STAMP(8);
         const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
         if (staged != t) {
@@ -308,9 +350,11 @@ __global__ void __launch_bounds__(256) k_moe_decode(FusedArgs a) {
             staged = t;
             __syncthreads();
         }
+        if (item == (int) blockIdx.x) STAMP(9);
         float* Ap = a.A + (size_t) p * a.ff;
         rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
                                    [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
+        if (item == (int) blockIdx.x) STAMP(10);
         wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
         __syncthreads();
         if (tid == 0 && atomicAdd(&pairc[p * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&pairc[p * 96 + 32], 1u);   // the pair's A is complete
@@ -479,6 +523,6 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
 
 #ifdef NSLM_FUSED_STAMPS
 extern "C" int kc_moe_decode_stamps(unsigned long long* host) {
-    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 8);
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 16);
 }
 #endif

@@ -152,3 +152,49 @@ def test_whole_expert_block_in_one_launch(T):
     bad = np.argwhere(A.view(np.uint32) != B.view(np.uint32))
     assert not np.array_equal(A, x0) and len(bad) == 0, (len(bad), bad[:8].tolist(), A[tuple(bad[0])], B[tuple(bad[0])], x0[tuple(bad[0])])
     st.close()
+
+
+@pytest.mark.parametrize("case", ["pairs", "all_equal"])
+def test_fused_step_equal_logits(oracle, case):
+    """Equal router logits (BF16 logits tie often): the persistent kernel orders them as the separate router does,
+    ties to the higher expert id (k_q4_route, engine/kernels_qwen4.cu:385-422)."""
+    from nanoseedlm_amd import moe
+    rng = np.random.default_rng(5)
+    E, k, d, ff, T = 16, 4, 256, 128, 3
+    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=8)
+    gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, d, ff, eb=-20)
+    W = (rng.standard_normal((E, d)) * 0.05).astype(np.float32)
+    for grp in ((3, 7, 12), (0, 15), (5, 6)):      # identical router rows -> identical logits for every input
+        W[list(grp)] = W[grp[0]]
+    rw = packs.f32_to_bf16_bits(W)
+    st.set_layer(0, gate, up, down, rw)
+    st.finalize()
+    xn = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
+    if case == "all_equal":
+        xn[:] = 0.0
+    outs = []
+    for fused in (1, 0):
+        st.set_fused(fused)
+        dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf.from_array(np.zeros((T, d), dtype=np.float32))
+        st.step(None, 0, dx.ptr, T, dio.ptr)
+        ind, wt = st.last_routing(T)
+        outs.append((ind.copy(), wt.copy(), dio.to_array(np.float32, (T, d)).copy()))
+        dx.free(); dio.free()
+    assert st.fused_error() == 0
+    assert np.array_equal(outs[0][0], outs[1][0]), (outs[0][0], outs[1][0])
+    assert np.array_equal(outs[0][1].view(np.uint32), outs[1][1].view(np.uint32))
+    assert np.array_equal(outs[0][2].view(np.uint32), outs[1][2].view(np.uint32))
+    Wd = packs.bf16_bits_to_f32(rw).astype(np.float64)
+    lg = packs.round_bf16((xn.astype(np.float64) @ Wd.T).astype(np.float32))
+    oi, _ = oracle.route_softmax(lg, k)
+    if case == "all_equal":
+        assert np.array_equal(outs[0][0], np.tile(np.arange(E - 1, E - 1 - k, -1, dtype=np.int32), (T, 1)))
+    # the groups really tie on the GPU: members of a group that are both chosen appear in descending id order
+    for t in range(T):
+        sel = outs[0][0][t].tolist()
+        for grp in ((3, 7, 12), (0, 15), (5, 6)):
+            pos = [sel.index(g) for g in grp if g in sel]
+            ids = [g for g in grp if g in sel]
+            assert pos == sorted(pos, reverse=True) or len(ids) < 2, (sel, grp)
+    assert np.mean([len(set(outs[0][0][t]) & set(oi[t])) / k for t in range(T)]) >= 0.75
+    st.close()
