@@ -255,6 +255,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
     // ---- route: every workgroup ranks the logits of the token it needs (cheap, and saves a grid barrier) ----------------
     // rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order
     int routed = -1;
+    bool weighted = true;
     auto route = [&](int t) {
         if (routed == t) return;
         routed = t;
@@ -318,22 +319,30 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
             sl_s[which][j] = (which == 0 ? a.gate : which == 1 ? a.up : a.down)[ri_s[j]];
         }
         if (a.ns && tid >= 253) sl_s[tid - 253][a.k] = a.sh[tid - 253];
-        if (tid < a.k) rw_s[tid] = expf(rv[ri_s[tid]] - rv[ri_s[0]]);
         __syncthreads();
 #ifdef NSLM_FUSED_STAMPS
         tq[3] = wall_clock64();
         if (tid == 0 && blockIdx.x < 1024) for (int q = 0; q < 4; ++q) g_fstamp[blockIdx.x * 16 + 11 + q] = tq[q];
 #endif
-        if (tid < a.k) {
+        weighted = false;
+    };
+    // The routing weights of the token last routed: softmax over the k chosen logits.  Only the combine needs them, so this
+    // runs after the item's first records are requested, on the first wave alone (a wave's LDS accesses stay in order, and a
+    // workgroup barrier separates this from every reader and from the next route()).
+    auto route_weights = [&](int t) {
+        if (weighted) return;
+        weighted = true;
+        if (wv != 0) return;
+        if (lane < a.k) rw_s[lane] = expf(rv[ri_s[lane]] - rv[ri_s[0]]);
+        if (lane < a.k) {
             float top = 0.0f;
             for (int r = 0; r < a.k; ++r) top += rw_s[r];
-            rw_s[tid] = rw_s[tid] / top;   // every lane has read all k values before any lane writes: one wave, in order
+            rw_s[lane] = rw_s[lane] / top;   // every lane has read all k values before any lane writes
         }
-        if (a.ns && tid == 255) rw_s[a.k] = 1.0f;
-        __syncthreads();
-        if (blockIdx.x == (unsigned) t % G && tid < a.k) {   // one writer per token publishes the routing
-            a.ind[(size_t) t * a.k + tid] = ri_s[tid];
-            a.wt[(size_t) t * a.k + tid] = rw_s[tid];
+        if (a.ns && lane == a.k) rw_s[a.k] = 1.0f;
+        if (blockIdx.x == (unsigned) t % G && lane < a.k) {   // one writer per token publishes the routing
+            a.ind[(size_t) t * a.k + lane] = ri_s[lane];
+            a.wt[(size_t) t * a.k + lane] = rw_s[lane];
         }
     };
 
@@ -344,6 +353,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         if (item == (int) blockIdx.x) STAMP(8);
         const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
+        route_weights(t);
         if (staged != t) {
             __syncthreads();
             stage_input(a.x + (size_t) t * a.xs, a.d, xl, a.nw, a.nw ? rn_s[t] : 1.0f);
@@ -360,7 +370,10 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         if (tid == 0 && atomicAdd(&pairc[p * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&pairc[p * 96 + 32], 1u);   // the pair's A is complete
     }
     // tokens whose routing nobody needed here still get published by their designated workgroup
-    for (int t = (int) blockIdx.x; t < a.T; t += (int) G) route(t);
+    for (int t = (int) blockIdx.x; t < a.T; t += (int) G) {
+        route(t);
+        route_weights(t);
+    }
     STAMP(3);
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
@@ -371,6 +384,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
         route(t);
         d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, tile * a.it_d / a.ntile_d * a.rpid, min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d));
+        route_weights(t);
     }
     // No grid barrier here: a down item needs its own pair's A only, so it waits for that pair's gate+up items (every
     // workgroup finishes its gate+up items before it waits, and the whole grid is resident, so the wait ends; bounded anyway).
@@ -379,6 +393,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         route(t);
         const int v0 = tile * a.it_d / a.ntile_d * a.rpid, v1 = min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d);
         if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
+        route_weights(t);
         if (tid == 0) {
             uint32_t spins = 0;
             while (ld_agent(&pairc[p * 96 + 32]) == 0u) {
