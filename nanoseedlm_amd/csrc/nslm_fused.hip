@@ -167,14 +167,40 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
 }
 
 // n floats of a row staged chunk-padded into LDS by the whole workgroup; coherent: agent-scope loads (the row was
-// written by other workgroups of this launch)
+// written by other workgroups of this launch).  Eight loads a thread are requested before the first is used (clamped
+// indices, so they are unconditional): one load and one LDS store a round is one memory round trip a round.
 __device__ __forceinline__ void stage_row(const float* src, int n, float* xl, bool coherent) {
-    for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = coherent ? ld_agent(src + i) : src[i];
+    for (int i0 = threadIdx.x; i0 < n; i0 += 256 * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(i0 + 256 * u, n - 1);
+            v[u] = coherent ? ld_agent(src + i) : src[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + 256 * u;
+            if (i < n) xl[(i >> 6) * XPAD + (i & 63)] = v[u];
+        }
+    }
 }
 // an input row, normalised on the way when nw is given: the values kq4_norm1p would have stored
 __device__ __forceinline__ void stage_input(const float* src, int n, float* xl, const float* nw, float rn) {
     if (!nw) { stage_row(src, n, xl, false); return; }
-    for (int i = threadIdx.x; i < n; i += 256) xl[(i >> 6) * XPAD + (i & 63)] = src[i] * rn * (1.0f + nw[i]);
+    for (int i0 = threadIdx.x; i0 < n; i0 += 256 * 8) {
+        float v[8], w[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = min(i0 + 256 * u, n - 1);
+            v[u] = src[i];
+            w[u] = nw[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + 256 * u;
+            if (i < n) xl[(i >> 6) * XPAD + (i & 63)] = v[u] * rn * (1.0f + w[u]);
+        }
+    }
 }
 
 #ifdef NSLM_FUSED_STAMPS
@@ -221,24 +247,42 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         const uint16_t* wr = a.rw + (size_t) e * a.d;
         const float* xr = a.x + (size_t) t * a.xs;
         float acc = 0.0f;
-        for (int j = lane; j < a.d / 8; j += 64) {
-            const uint4 q = *(const uint4*) (wr + (size_t) j * 8);
-            float4 x0 = *(const float4*) (xr + (size_t) j * 8), x1 = *(const float4*) (xr + (size_t) j * 8 + 4);
-            if (a.nw) {
-                const float4 w0 = *(const float4*) (a.nw + (size_t) j * 8), w1 = *(const float4*) (a.nw + (size_t) j * 8 + 4);
-                const float rn = rn_s[t];
-                x0.x = x0.x * rn * (1.0f + w0.x); x0.y = x0.y * rn * (1.0f + w0.y); x0.z = x0.z * rn * (1.0f + w0.z); x0.w = x0.w * rn * (1.0f + w0.w);
-                x1.x = x1.x * rn * (1.0f + w1.x); x1.y = x1.y * rn * (1.0f + w1.y); x1.z = x1.z * rn * (1.0f + w1.z); x1.w = x1.w * rn * (1.0f + w1.w);
+        const int nb = a.d / 8;
+        // four of the lane's blocks a round, every load of the round requested before the first use (clamped indices, so
+        // the loads are unconditional): a loop that loads and uses one block a round is one memory round trip a round
+        for (int j0 = lane; j0 < nb; j0 += 256) {
+            uint4 q[4];
+            float4 x0[4], x1[4], w0[4], w1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const size_t j = (size_t) min(j0 + 64 * u, nb - 1);
+                q[u] = *(const uint4*) (wr + j * 8);
+                x0[u] = *(const float4*) (xr + j * 8);
+                x1[u] = *(const float4*) (xr + j * 8 + 4);
+                if (a.nw) {
+                    w0[u] = *(const float4*) (a.nw + j * 8);
+                    w1[u] = *(const float4*) (a.nw + j * 8 + 4);
+                }
             }
-            float dd = bf(q.x & 0xFFFFu) * x0.x;
-            dd = fmaf(bf(q.x >> 16), x0.y, dd);
-            dd = fmaf(bf(q.y & 0xFFFFu), x0.z, dd);
-            dd = fmaf(bf(q.y >> 16), x0.w, dd);
-            dd = fmaf(bf(q.z & 0xFFFFu), x1.x, dd);
-            dd = fmaf(bf(q.z >> 16), x1.y, dd);
-            dd = fmaf(bf(q.w & 0xFFFFu), x1.z, dd);
-            dd = fmaf(bf(q.w >> 16), x1.w, dd);
-            acc = fmaf(dd, 1.0f, acc);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (j0 + 64 * u >= nb) break;
+                float4 y0 = x0[u], y1 = x1[u];
+                if (a.nw) {
+                    const float rn = rn_s[t];
+                    y0.x = y0.x * rn * (1.0f + w0[u].x); y0.y = y0.y * rn * (1.0f + w0[u].y); y0.z = y0.z * rn * (1.0f + w0[u].z); y0.w = y0.w * rn * (1.0f + w0[u].w);
+                    y1.x = y1.x * rn * (1.0f + w1[u].x); y1.y = y1.y * rn * (1.0f + w1[u].y); y1.z = y1.z * rn * (1.0f + w1[u].z); y1.w = y1.w * rn * (1.0f + w1[u].w);
+                }
+                float dd = bf(q[u].x & 0xFFFFu) * y0.x;
+                dd = fmaf(bf(q[u].x >> 16), y0.y, dd);
+                dd = fmaf(bf(q[u].y & 0xFFFFu), y0.z, dd);
+                dd = fmaf(bf(q[u].y >> 16), y0.w, dd);
+                dd = fmaf(bf(q[u].z & 0xFFFFu), y1.x, dd);
+                dd = fmaf(bf(q[u].z >> 16), y1.y, dd);
+                dd = fmaf(bf(q[u].w & 0xFFFFu), y1.z, dd);
+                dd = fmaf(bf(q[u].w >> 16), y1.w, dd);
+                acc = fmaf(dd, 1.0f, acc);
+            }
         }
         for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
         if (lane == 0) st_agent(a.logits + item, bfr(acc));
