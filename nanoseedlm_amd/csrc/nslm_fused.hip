@@ -204,7 +204,7 @@ __device__ __forceinline__ void stage_input(const float* src, int n, float* xl, 
 }
 
 #ifdef NSLM_FUSED_STAMPS
-__device__ unsigned long long g_fstamp[1024 * 16];
+__device__ unsigned long long g_fstamp[1024 * 32];
 #endif
 template <int P, bool SHFL_G, bool SHFL_D>
 __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five waves a SIMD: at most 96 registers
@@ -223,10 +223,12 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
     // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
     unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
 #ifdef NSLM_FUSED_STAMPS   // development builds: every workgroup's timeline
-#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } } while (0)
-    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 16 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + (i)] = wall_clock64(); } } while (0)
+#define DSTAMP(i) do { if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + (i)] = wall_clock64(); } while (0)
+    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
 #else
-#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
+#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)   // i < 6: the stamps share the error word's line
+#define DSTAMP(i) do { } while (0)
 #endif
     STAMP(0);
     load_tables(tab);
@@ -366,7 +368,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         __syncthreads();
 #ifdef NSLM_FUSED_STAMPS
         tq[3] = wall_clock64();
-        if (tid == 0 && blockIdx.x < 1024) for (int q = 0; q < 4; ++q) g_fstamp[blockIdx.x * 16 + 11 + q] = tq[q];
+        if (tid == 0 && blockIdx.x < 1024) for (int q = 0; q < 4; ++q) g_fstamp[blockIdx.x * 32 + 11 + q] = tq[q];
 #endif
         weighted = false;
     };
@@ -394,7 +396,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
-        if (item == (int) blockIdx.x) STAMP(8);
+        if (item == (int) blockIdx.x) DSTAMP(8);
         const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
         route_weights(t);
@@ -404,11 +406,11 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
             staged = t;
             __syncthreads();
         }
-        if (item == (int) blockIdx.x) STAMP(9);
+        if (item == (int) blockIdx.x) DSTAMP(9);
         float* Ap = a.A + (size_t) p * a.ff;
         rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
                                    [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
-        if (item == (int) blockIdx.x) STAMP(10);
+        if (item == (int) blockIdx.x) DSTAMP(10);
         wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
         __syncthreads();
         if (tid == 0 && atomicAdd(&pairc[p * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&pairc[p * 96 + 32], 1u);   // the pair's A is complete
@@ -454,13 +456,16 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         stage_row(a.A + (size_t) p * a.ff, a.ff, xl, true);
         staged = -1;
         __syncthreads();
+        if (item == (int) blockIdx.x) DSTAMP(16);
         float* Dp = a.D + (size_t) p * a.d;
         rows_pass<P, false, SHFL_D>(d0, sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1, tab, xl, part,
                                     [&](int r, float s, float) { st_agent(Dp + r, bfr(s)); });
+        if (item == (int) blockIdx.x) DSTAMP(17);
         wg_release();
         __syncthreads();
         if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.kk - 1);
         __syncthreads();
+        if (item == (int) blockIdx.x) DSTAMP(18);
         if (s_flag) {   // all k experts' rows of this tile are written: out = 0.5 * 0 + sum_j wt_j D_j, in j order
             wg_acquire();
             for (int r = v0 + tid; r < v1; r += 256) {
@@ -479,6 +484,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
     }
     STAMP(5);
 #undef STAMP
+#undef DSTAMP
 }
 
 int cu_count() {
@@ -582,6 +588,6 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
 
 #ifdef NSLM_FUSED_STAMPS
 extern "C" int kc_moe_decode_stamps(unsigned long long* host) {
-    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 16);
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 32);
 }
 #endif

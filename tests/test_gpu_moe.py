@@ -154,18 +154,21 @@ def test_whole_expert_block_in_one_launch(T):
     st.close()
 
 
+@pytest.mark.parametrize("E", [16, 200, 320])
 @pytest.mark.parametrize("case", ["pairs", "all_equal"])
-def test_fused_step_equal_logits(oracle, case):
+def test_fused_step_equal_logits(oracle, case, E):
     """Equal router logits (BF16 logits tie often): the persistent kernel orders them as the separate router does,
-    ties to the higher expert id (k_q4_route, engine/kernels_qwen4.cu:385-422)."""
+    ties to the higher expert id (k_q4_route, engine/kernels_qwen4.cu:385-422).  16 and 200 experts take the register
+    path of the kernel's ranking, 320 the path for more than 256 experts."""
     from nanoseedlm_amd import moe
-    rng = np.random.default_rng(5)
-    E, k, d, ff, T = 16, 4, 256, 128, 3
+    rng = np.random.default_rng(5 + E)
+    k, d, ff, T = 4, 256, 128, 3
     st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=8)
     gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, d, ff, eb=-20)
     W = (rng.standard_normal((E, d)) * 0.05).astype(np.float32)
-    for grp in ((3, 7, 12), (0, 15), (5, 6)):      # identical router rows -> identical logits for every input
-        W[list(grp)] = W[grp[0]]
+    groups = ((3, 7, 12), (0, E - 1), (5, 6), (E // 2, E // 2 + 1, E - 2))
+    for grp in groups:      # identical router rows -> identical logits for every input
+        W[list(grp)] = 3.0 * W[grp[0]]      # large, so that the groups reach the top k for some inputs
     rw = packs.f32_to_bf16_bits(W)
     st.set_layer(0, gate, up, down, rw)
     st.finalize()
@@ -192,7 +195,7 @@ def test_fused_step_equal_logits(oracle, case):
     # the groups really tie on the GPU: members of a group that are both chosen appear in descending id order
     for t in range(T):
         sel = outs[0][0][t].tolist()
-        for grp in ((3, 7, 12), (0, 15), (5, 6)):
+        for grp in groups:
             pos = [sel.index(g) for g in grp if g in sel]
             ids = [g for g in grp if g in sel]
             assert pos == sorted(pos, reverse=True) or len(ids) < 2, (sel, grp)
