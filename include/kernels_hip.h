@@ -242,7 +242,7 @@ void kc_fill_random(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);
 void kc_fill_bf16(kc_stream_t s, uint16_t* p, size_t n, uint64_t seed, float scale);
 void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);   /* random E4M3 codes the cache's encoder can write (no 0x7F / 0xFF) */
 
-/* A whole routed-expert decode step for T <= MV_MAXT tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
+/* A whole routed-expert decode step for T <= kc_moe_decode_max_rows() tokens in ONE persistent kernel: router logits bf16(W x) on a BF16
  * router weight [n_exp][d], softmax top-k, gate + up + SwiGLU gather, down gather, out[t] = sum_j wt_j y_j - the same
  * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.
  * Scratch (caller-owned device memory): logits [T][n_exp], ind / wt [T][top_k] (the routing, also an output), A [T*k][ff],
@@ -250,8 +250,14 @@ void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);   
  * consistent from launch to launch; sync[kc_moe_decode_error_word()] != 0 afterwards reports a grid barrier that gave up,
  * after which the caller must zero sync again).
  * The grid spans the whole device and its workgroups wait for each other: nothing else may run on the GPU beside it.
+ * Up to MV_MAXT tokens every (token, expert) pair is a pass of its own (the reference's decode composition, bit for bit);
+ * above that and up to kc_moe_decode_max_rows() the pairs of one expert share each decoded block, two at a time, with
+ * the same per-token arithmetic (exact weights, the row-sum order of kc_mv_sel) - where the reference switches to its grouped
+ * GEMM on BF16-rounded weights (engine/mova_cuda.c:1308-1317), so results there differ from the GEMM path's by that rounding
+ * (shapes whose gate+up row sums do not fit a wave shuffle are refused above MV_MAXT tokens: the grouped GEMMs are faster there).
  * Returns 0, or -1 when the shape has no fused kernel (nothing launched: use the separate launchers). */
 size_t kc_moe_decode_sync_words(int T, int d);
+int kc_moe_decode_max_rows(void);
 int kc_moe_decode_error_word(void);
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                   int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,

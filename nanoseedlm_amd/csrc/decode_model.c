@@ -350,7 +350,7 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
         /* ---- experts: x = bf16(x + bf16(sum_k wt_k y_k + shared(xn))) ---- */
         const WSlice* st = m->shared_tab + (size_t) l * 3;
         const float* nw2 = m->norm + (size_t) (2 * l + 1) * d;
-        if (!big && !par && ffs == c->ff) {   /* norm + routed + shared + residual: the whole expert block in the one persistent launch */
+        if (T <= kc_moe_decode_max_rows() && !par && ffs == c->ff) {   /* norm + routed + shared + residual: the whole expert block in the one persistent launch */
             const WSlice sh3[3] = {dn[NSLM_W_SG].w, dn[NSLM_W_SU].w, dn[NSLM_W_SD].w};
             const int rc = nslm_moe_step_layer(m->moe, s, l, m->x, T, sh3, m->x, m->x, nw2, c->eps);
             if (rc < 0) return -1;

@@ -23,7 +23,7 @@ struct NslmMoe {
     MmTile* tiles;
     int max_tiles;
     uint32_t* sync;             /* device: the fused decode kernel's barrier words */
-    int fused;                  /* 1: T <= MV_MAXT steps of the softmax composition take kc_moe_decode */
+    int fused;                  /* 1: steps of the softmax composition up to kc_moe_decode_max_rows() rows take kc_moe_decode */
 };
 
 static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
@@ -91,7 +91,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     bad |= nh_malloc((void**) &m->perm, 4 * (size_t) P);
     bad |= nh_malloc((void**) &m->tiles, sizeof(MmTile) * (size_t) m->max_tiles);
     bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 3));
-    bad |= nh_malloc((void**) &m->sync, 4 * kc_moe_decode_sync_words(MV_MAXT, c->d));
+    bad |= nh_malloc((void**) &m->sync, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d));
     m->fused = 1;
     m->unit_host = (uint8_t*) calloc(1, cur);
     m->eb = (int32_t*) calloc((size_t) m->units * 3, 4);
@@ -101,7 +101,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
         return NULL;
     }
     nh_memset(m->zero, 0, 4 * (size_t) c->max_rows * c->d);
-    nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(MV_MAXT, c->d));
+    nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d));
     nh_memset(m->rb, 0, 2 * (size_t) c->n_layer * c->n_exp);
     return m;
 }
@@ -227,7 +227,7 @@ int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, i
     if (!m->final || T < 1 || T > c->max_rows || layer < 0 || layer >= c->n_layer) return -1;
     const int E = c->n_exp;
     const WSlice* tab = m->pool.tab + (size_t) layer * 3 * E;
-    if (!(m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= MV_MAXT)) return 1;
+    if (!(m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows())) return 1;
     if (kc_moe_decode_layer(s, c->fmt, m->rw + (size_t) layer * E * c->d, tab, tab + E, tab + 2 * E, E, c->top_k, c->d, c->ff, xn, c->d, T, out,
                             c->d, m->logit, m->ind, m->wt, m->A, m->D, m->sync, shared, res, norm_w, norm_eps))
         return 1;
@@ -241,7 +241,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
     const WSlice* gate = m->pool.tab + ((size_t) layer * 3 + 0) * E;
     const WSlice* up = m->pool.tab + ((size_t) layer * 3 + 1) * E;
     const WSlice* down = m->pool.tab + ((size_t) layer * 3 + 2) * E;
-    if (m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= MV_MAXT &&
+    if (m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows() &&
         !kc_moe_decode(s, c->fmt, m->rw + (size_t) layer * E * d, gate, up, down, E, k, d, ff, xn, d, T, io, d, m->logit, m->ind,
                        m->wt, m->A, m->D, m->sync))
         return kc_last_error() ? -1 : 0;   /* the whole step in one persistent kernel */

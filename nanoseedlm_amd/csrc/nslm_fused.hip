@@ -16,6 +16,7 @@
 // Grid barriers: the grid is sized to the number of workgroups the device can hold at once (occupancy query), every
 // workgroup arrives on a counter in caller-provided scratch and spins until all have; the spin is bounded, and a
 // workgroup that gives up sets an error word and runs on to the end, so every wave always exits.
+#include <math.h>
 #include <stdlib.h>
 
 #include "nslm_mv_dev.h"
@@ -203,6 +204,52 @@ __device__ __forceinline__ void stage_input(const float* src, int n, float* xl, 
     }
 }
 
+// The k best of E logits already in LDS (rv, padded to a multiple of four with -inf): ri[r] = the expert of rank r, where
+// rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order.  Called by
+// the whole workgroup after a barrier; the caller's next barrier publishes ri.  scratch: 512 words of LDS.
+// The logits are BF16 values (phase 1 rounds them), so the upper half of a float's order-preserving integer image holds
+// all of a logit and the lower half is free for the expert's index: one 32-bit key whose integer order is the routing
+// order, and no two keys are equal.  rank(e) = number of larger keys.  Up to 256 experts: thread (e, part) counts over its
+// part of the experts (keys read four at a time as LDS broadcasts: two instructions a compare) and the parts' counts are
+// added.  Every instruction counts here, scalar ones too: the workgroups of a CU rank at the same moment, and wave-wide
+// compares with scalar population counts took 3 to 6 us of every workgroup's time.
+__device__ __forceinline__ void rank_logits(const float* rv, int E, int k, uint32_t* scratch, int* ri) {
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, E4 = (E + 3) & ~3;
+    auto key_of = [&](int o) {
+        const uint32_t b = __float_as_uint(rv[o] + 0.0f);   // -0 counts as +0, as in a float compare
+        return ((b ^ ((uint32_t) ((int32_t) b >> 31) | 0x80000000u)) & 0xFFFF0000u) | (uint32_t) o;
+    };
+    if (E <= 256) {
+        uint32_t* pk = scratch;              // keys (0 = absent, below every real key)
+        int* gp = (int*) scratch + 256;      // the parts' counts, [part][expert]
+        pk[tid] = tid < E ? key_of(tid) : 0u;
+        __syncthreads();
+        const int epad = E <= 64 ? 64 : E <= 128 ? 128 : 256, len = epad * epad / 256;
+        const int e = tid & (epad - 1), o0 = tid / epad * len;
+        const uint32_t ke = pk[e];
+        int g = 0;
+#pragma unroll 4
+        for (int o = o0; o < o0 + len; o += 4) {
+            const uint4 q = *(const uint4*) &pk[o];
+            g += (q.x > ke ? 1 : 0) + (q.y > ke ? 1 : 0) + (q.z > ke ? 1 : 0) + (q.w > ke ? 1 : 0);
+        }
+        gp[tid] = g;
+        __syncthreads();
+        if (tid < E) {
+            int rank = 0;
+            for (int q = tid; q < 256; q += epad) rank += gp[q];
+            if (rank < k) ri[rank] = tid;
+        }
+    } else {   // a wave takes the experts one at a time
+        for (int e = wv; e < E; e += 4) {
+            const uint32_t ke = __builtin_amdgcn_readfirstlane(key_of(e));
+            int rank = 0;
+            for (int o = lane; o < E4 + 63; o += 64) rank += __popcll(__ballot(o < E && key_of(o < 1024 ? o : 1023) > ke));
+            if (rank < k && lane == 0) ri[rank] = e;
+        }
+    }
+}
+
 #ifdef NSLM_FUSED_STAMPS
 __device__ unsigned long long g_fstamp[1024 * 32];
 #endif
@@ -314,45 +361,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
 #ifdef NSLM_FUSED_STAMPS
         tq[0] = wall_clock64();
 #endif
-        // The logits are BF16 values (phase 1 rounds them), so the upper half of a float's order-preserving integer image
-        // holds all of a logit and the lower half is free for the expert's index: one 32-bit key whose integer order is the
-        // routing order, and no two keys are equal.  rank(e) = number of larger keys.  Up to 256 experts: thread (e, part)
-        // counts over its part of the experts (keys read four at a time as LDS broadcasts: two instructions a compare) and
-        // the parts' counts are added.  Every instruction counts here, scalar ones too: the workgroups of a CU rank at the
-        // same moment, and wave-wide compares with scalar population counts took 3 to 6 us of every workgroup's time.
-        auto key_of = [&](int o) {
-            const uint32_t b = __float_as_uint(rv[o] + 0.0f);   // -0 counts as +0, as in a float compare
-            return ((b ^ ((uint32_t) ((int32_t) b >> 31) | 0x80000000u)) & 0xFFFF0000u) | (uint32_t) o;
-        };
-        if (a.E <= 256) {
-            uint32_t* pk = (uint32_t*) &part[0][0];   // keys (0 = absent, below every real key)
-            int* gp = (int*) &part[1][0];             // the parts' counts, [part][expert]
-            pk[tid] = tid < a.E ? key_of(tid) : 0u;
-            __syncthreads();
-            const int epad = a.E <= 64 ? 64 : a.E <= 128 ? 128 : 256, len = epad * epad / 256;
-            const int e = tid & (epad - 1), o0 = tid / epad * len;
-            const uint32_t ke = pk[e];
-            int g = 0;
-#pragma unroll 4
-            for (int o = o0; o < o0 + len; o += 4) {
-                const uint4 q = *(const uint4*) &pk[o];
-                g += (q.x > ke ? 1 : 0) + (q.y > ke ? 1 : 0) + (q.z > ke ? 1 : 0) + (q.w > ke ? 1 : 0);
-            }
-            gp[tid] = g;
-            __syncthreads();
-            if (tid < a.E) {
-                int rank = 0;
-                for (int q = tid; q < 256; q += epad) rank += gp[q];
-                if (rank < a.k) ri_s[rank] = tid;
-            }
-        } else {   // a wave takes the experts one at a time
-            for (int e = wv; e < a.E; e += 4) {
-                const uint32_t ke = __builtin_amdgcn_readfirstlane(key_of(e));
-                int rank = 0;
-                for (int o = lane; o < E4 + 63; o += 64) rank += __popcll(__ballot(o < a.E && key_of(o < 1024 ? o : 1023) > ke));
-                if (rank < a.k && lane == 0) ri_s[rank] = e;
-            }
-        }
+        rank_logits(rv, a.E, a.k, (uint32_t*) &part[0][0], ri_s);
 #ifdef NSLM_FUSED_STAMPS
         tq[1] = wall_clock64();
 #endif
@@ -487,6 +496,319 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
 #undef DSTAMP
 }
 
+// ---- 9 to 16 tokens: the pairs of one expert share its decoded blocks ---------------------------------------------------
+// With more tokens than experts-per-token slots, several (token, expert) pairs meet on the same expert, and the decode of
+// a block (nine tenths of the work) can serve them all.  Pairs are grouped by expert in runs of at most NT; an item is a
+// (group, row tile); a thread decodes its chunk once and multiplies it with the NT rows of activations staged side by side
+// in LDS (chunk_dot<P, NT>: per token the same chain of operations as the one-token kernel, hence the same bits).  The
+// groups must be the same in every workgroup, so the routing is done once (workgroup t routes token t) and published, a
+// second grid barrier follows, and every workgroup builds the same table from the published selection: position of a pair
+// among the pairs of its expert in pair order, groups numbered in expert order.  Pair p = (token p / kk, slot p % kk),
+// slots >= k are the always-on experts (expert ids E, E + 1, ...).
+#define FG_MAXT 16
+#define FG_MAXP 512    // pairs a launch: T * kk
+#define FG_RN_WORDS 64   // the rows' RMSNorm scales behind the pairs' words of the sync area
+
+template <int P, bool GATEUP, bool SHFL, int NT, typename Emit>
+__device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1,
+                                            const uint32_t* tab, const float* xl, int xstride, int nt, float* part, Emit emit) {
+    const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
+    const bool active = lr < rpi;
+    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
+    auto fetch = [&](int vv) {
+        const bool ok = active && vv < v1;
+        const int r = GATEUP ? vv >> 1 : vv;
+        const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
+        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
+    };
+    int par = 0;
+    for (int vb = v0; vb < v1; vb += rpi, par ^= 1) {
+        const int v = vb + lr;
+        const Chunk nxt = fetch(v + rpi);
+        float acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+        const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
+        if (active && v < v1) chunk_dot<P, NT, true>(cur, eb, tab, xl + ch * XPAD, xstride, nt, acc);
+        if (SHFL) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                float s = acc[t];
+                for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+                if (GATEUP) {
+                    const float other = __shfl_xor(s, L);
+                    if (t < nt && active && ch == 0 && !(v & 1) && v < v1) emit(t, v >> 1, s * NSLM_R32, other * NSLM_R32);
+                } else if (t < nt && active && ch == 0 && v < v1) emit(t, v, s * NSLM_R32, 0.0f);
+            }
+        } else {
+            float* pp = part + par * NT * 256;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) pp[t * 256 + tid] = acc[t];
+            __syncthreads();   // one barrier per iteration: part is double-buffered by iteration parity
+            const int nrow = min(rpi, v1 - vb);
+            if (GATEUP) {
+                const int nr2 = nrow / 2;
+                for (int w = tid; w < nr2 * nt; w += 256) {   // (token, row) sums: more than 256 when rows are short
+                    const int t = w / nr2, r = w - t * nr2;
+                    float gs = 0.0f, us = 0.0f;
+                    for (int j = 0; j < L; ++j) gs += pp[t * 256 + (2 * r) * L + j];
+                    for (int j = 0; j < L; ++j) us += pp[t * 256 + (2 * r + 1) * L + j];
+                    emit(t, (vb >> 1) + r, gs * NSLM_R32, us * NSLM_R32);
+                }
+            } else {
+                for (int w = tid; w < nrow * nt; w += 256) {
+                    const int t = w / nrow, r = w - t * nrow;
+                    float sm = 0.0f;
+                    for (int j = 0; j < L; ++j) sm += pp[t * 256 + r * L + j];
+                    emit(t, vb + r, sm * NSLM_R32, 0.0f);
+                }
+            }
+        }
+        cur = nxt;
+    }
+    if (!SHFL) __syncthreads();   // part may be reused by the next pass
+}
+
+template <int P, int NT, bool SHFL_G, bool SHFL_D>
+__global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
+    extern __shared__ float xl[];   // NT rows of max(d, ff) activations, chunk-padded, side by side
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    __shared__ float part[2 * NT * 256];
+    __shared__ __attribute__((aligned(16))) float rv[1024];
+    __shared__ float rw_s[33];
+    __shared__ int ri_s[33];
+    __shared__ WSlice sl_s[3];
+    __shared__ int s_flag, s_ng;
+    __shared__ float rn_s[FG_MAXT], nred[4];
+    __shared__ __attribute__((aligned(16))) uint16_t pe[FG_MAXP + 8];   // a pair's expert
+    __shared__ uint16_t gof[FG_MAXP], gm[FG_MAXP * NT], cnt_s[1024 + 32], base_s[1024 + 32];   // position; members; per expert: pairs, first group
+    __shared__ uint8_t gn[FG_MAXP];   // a group's number of members
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const uint32_t G = (uint32_t) a.grid;
+    const int P_ = a.T * a.kk, NE = a.E + a.ns;
+    const int xsg = a.Lg * XPAD, xsd = a.Ld * XPAD;   // LDS floats between two rows of activations
+    uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
+    uint32_t* grpc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [group][3][32]: arrivals, ready, done
+    float* rnpub = (float*) (grpc + (size_t) a.T * 33 * 96);
+    load_tables(tab);
+
+    // ---- phase 1: router logits, one wave per (token, expert) -------------------------------------------------------------
+    if (a.nw) {   // the scales of the rows whose logits this workgroup forms (uniform over the workgroup)
+        for (int base = (int) blockIdx.x * 4; base < a.T * a.E; base += (int) G * 4) {
+            const int t0 = base / a.E, t1 = min(base + 3, a.T * a.E - 1) / a.E;
+            for (int t = t0; t <= t1; ++t) {
+                const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
+                if (tid == 0) rn_s[t] = r;
+            }
+        }
+        __syncthreads();
+    }
+    for (int item = (int) blockIdx.x * 4 + wv; item < a.T * a.E; item += (int) G * 4) {
+        const int t = item / a.E, e = item - t * a.E;
+        const uint16_t* wr = a.rw + (size_t) e * a.d;
+        const float* xr = a.x + (size_t) t * a.xs;
+        float acc = 0.0f;
+        const int nb = a.d / 8;
+        for (int j0 = lane; j0 < nb; j0 += 256) {
+            uint4 q[4];
+            float4 x0[4], x1[4], w0[4], w1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const size_t j = (size_t) min(j0 + 64 * u, nb - 1);
+                q[u] = *(const uint4*) (wr + j * 8);
+                x0[u] = *(const float4*) (xr + j * 8);
+                x1[u] = *(const float4*) (xr + j * 8 + 4);
+                if (a.nw) {
+                    w0[u] = *(const float4*) (a.nw + j * 8);
+                    w1[u] = *(const float4*) (a.nw + j * 8 + 4);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (j0 + 64 * u >= nb) break;
+                float4 y0 = x0[u], y1 = x1[u];
+                if (a.nw) {
+                    const float rn = rn_s[t];
+                    y0.x = y0.x * rn * (1.0f + w0[u].x); y0.y = y0.y * rn * (1.0f + w0[u].y); y0.z = y0.z * rn * (1.0f + w0[u].z); y0.w = y0.w * rn * (1.0f + w0[u].w);
+                    y1.x = y1.x * rn * (1.0f + w1[u].x); y1.y = y1.y * rn * (1.0f + w1[u].y); y1.z = y1.z * rn * (1.0f + w1[u].z); y1.w = y1.w * rn * (1.0f + w1[u].w);
+                }
+                float dd = bf(q[u].x & 0xFFFFu) * y0.x;
+                dd = fmaf(bf(q[u].x >> 16), y0.y, dd);
+                dd = fmaf(bf(q[u].y & 0xFFFFu), y0.z, dd);
+                dd = fmaf(bf(q[u].y >> 16), y0.w, dd);
+                dd = fmaf(bf(q[u].z & 0xFFFFu), y1.x, dd);
+                dd = fmaf(bf(q[u].z >> 16), y1.y, dd);
+                dd = fmaf(bf(q[u].w & 0xFFFFu), y1.z, dd);
+                dd = fmaf(bf(q[u].w >> 16), y1.w, dd);
+                acc = fmaf(dd, 1.0f, acc);
+            }
+        }
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+        if (lane == 0) st_agent(a.logits + item, bfr(acc));
+    }
+    grid_barrier(a.sync, G);
+
+    // ---- routing, once per token: workgroup t % G ranks token t and publishes selection, weights and the row's scale ----
+    for (int t = (int) blockIdx.x; t < a.T; t += (int) G) {
+        __syncthreads();
+        const int E4 = (a.E + 3) & ~3;
+        for (int e = tid; e < E4; e += 256) rv[e] = e < a.E ? ld_agent(a.logits + (size_t) t * a.E + e) : __uint_as_float(0xFF800000u);
+        __syncthreads();
+        rank_logits(rv, a.E, a.k, (uint32_t*) part, ri_s);
+        __syncthreads();
+        if (wv == 0) {
+            if (lane < a.k) rw_s[lane] = expf(rv[ri_s[lane]] - rv[ri_s[0]]);
+            if (lane < a.k) {
+                float top = 0.0f;
+                for (int r = 0; r < a.k; ++r) top += rw_s[r];
+                st_agent((uint32_t*) a.ind + (size_t) t * a.k + lane, (uint32_t) ri_s[lane]);
+                st_agent(a.wt + (size_t) t * a.k + lane, rw_s[lane] / top);
+            }
+        }
+        if (a.nw) {
+            const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
+            if (tid == 0) st_agent(rnpub + t, r);
+        }
+    }
+    grid_barrier(a.sync, G);
+
+    // ---- the groups: the same table in every workgroup ----------------------------------------------------------------------
+    for (int i = tid; i < NE; i += 256) cnt_s[i] = 0;
+    for (int p = tid; p < P_ + 8; p += 256) {
+        const int pc = min(p, P_ - 1), t = pc / a.kk, j = pc - t * a.kk;
+        const int e = j < a.k ? (int) ld_agent((const uint32_t*) a.ind + (size_t) t * a.k + j) : a.E + (j - a.k);
+        if (p < FG_MAXP + 8) pe[p] = (uint16_t) (p < P_ ? e : 0xFFFF);   // the table is read eight at a time: pad with "no expert"
+    }
+    if (a.nw && tid < a.T) rn_s[tid] = ld_agent(rnpub + tid);
+    __syncthreads();
+    for (int p = tid; p < P_; p += 256) {   // position among the pairs of the same expert (in pair order), and their number
+        const uint32_t e = pe[p];
+        int before = 0, all = 0;
+        for (int q0 = 0; q0 < P_; q0 += 8) {
+            const uint4 w = *(const uint4*) &pe[q0];
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int m0 = (ww[u] & 0xFFFFu) == e ? 1 : 0, m1 = (ww[u] >> 16) == e ? 1 : 0;
+                all += m0 + m1;
+                before += (q0 + 2 * u < p ? m0 : 0) + (q0 + 2 * u + 1 < p ? m1 : 0);
+            }
+        }
+        gof[p] = (uint16_t) before;
+        cnt_s[e] = (uint16_t) all;   // every pair of the expert writes the same number
+    }
+    __syncthreads();
+    {   // groups before expert e: exclusive sums of ceil(cnt / NT), five experts a thread
+        int own[5], sum = 0;
+#pragma unroll
+        for (int u = 0; u < 5; ++u) {
+            const int e = tid * 5 + u;
+            own[u] = e < NE ? (cnt_s[e] + NT - 1) / NT : 0;
+            sum += own[u];
+        }
+        int inc = sum;
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(inc, o);
+            if (lane >= o) inc += v;
+        }
+        if (lane == 63) ri_s[wv] = inc;   // the waves' totals (ri_s is free after the routing)
+        __syncthreads();
+        int off = inc - sum;
+        for (int w = 0; w < wv; ++w) off += ri_s[w];
+#pragma unroll
+        for (int u = 0; u < 5; ++u) {
+            const int e = tid * 5 + u;
+            if (e < NE) base_s[e] = (uint16_t) off;
+            off += own[u];
+        }
+        if (tid == 255) s_ng = off;
+    }
+    __syncthreads();
+    for (int p = tid; p < P_; p += 256) {
+        const int e = pe[p], pos = gof[p], g = base_s[e] + pos / NT;
+        gm[g * NT + pos % NT] = (uint16_t) p;
+        if (pos % NT == 0) gn[g] = (uint8_t) min(NT, (int) cnt_s[e] - pos);
+    }
+    __syncthreads();
+    const int NG = s_ng, items_g = NG * a.ntile_g, items_d = NG * a.ntile_d;
+
+    // ---- gate + up + SwiGLU: items (group, row tile) ---------------------------------------------------------------------------
+    int staged_g = -1;
+    for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
+        const int g = item / a.ntile_g, tile = item - g * a.ntile_g, nt = gn[g], e = pe[gm[g * NT]];
+        const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
+        __syncthreads();
+        if (tid < 2) sl_s[tid] = e < a.E ? (tid == 0 ? a.gate : a.up)[e] : a.sh[tid];
+        __syncthreads();
+        const Chunk c0 = first_chunk<P, true>(sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1);
+        if (staged_g != g) {
+            for (int m = 0; m < nt; ++m) {
+                const int t = gm[g * NT + m] / a.kk;
+                stage_input(a.x + (size_t) t * a.xs, a.d, xl + m * xsg, a.nw, a.nw ? rn_s[t] : 1.0f);
+            }
+            staged_g = g;
+            __syncthreads();
+        }
+        rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part,
+                                         [&](int m, int r, float gs, float us) {
+                                             st_agent(a.A + (size_t) gm[g * NT + m] * a.ff + r, bfr(silu_bf(bfr(gs)) * bfr(us)));
+                                         });
+        wg_release();   // this item's rows of A are written: one more of the group's gate+up items is done
+        __syncthreads();
+        if (tid == 0 && atomicAdd(&grpc[g * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&grpc[g * 96 + 32], 1u);
+    }
+
+    // ---- down, then the last workgroup of a (token, row tile) sums the token's experts ------------------------------------
+    for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
+        const int g = item / a.ntile_d, tile = item - g * a.ntile_d, nt = gn[g], e = pe[gm[g * NT]];
+        const int v0 = tile * a.it_d / a.ntile_d * a.rpid, v1 = min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d);
+        __syncthreads();
+        if (tid == 0) sl_s[2] = e < a.E ? a.down[e] : a.sh[2];
+        __syncthreads();
+        const Chunk d0 = first_chunk<P, false>(sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1);
+        if (tid == 0) {   // the group's A is complete when its last gate+up item has said so (bounded wait)
+            uint32_t spins = 0;
+            while (ld_agent(&grpc[g * 96 + 32]) == 0u) {
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > SPIN_LIMIT) {
+                    atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        wg_acquire();
+        for (int m = 0; m < nt; ++m) stage_row(a.A + (size_t) gm[g * NT + m] * a.ff, a.ff, xl + m * xsd, true);
+        staged_g = -1;
+        __syncthreads();
+        rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part,
+                                          [&](int m, int r, float sm, float) { st_agent(a.D + (size_t) gm[g * NT + m] * a.d + r, bfr(sm)); });
+        wg_release();
+        for (int m = 0; m < nt; ++m) {   // one ticket per member's (token, row tile); the token's last arrival sums its experts
+            const int t = gm[g * NT + m] / a.kk;
+            __syncthreads();
+            if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.kk - 1);
+            if (tid < a.kk) rw_s[tid] = tid < a.k ? ld_agent(a.wt + (size_t) t * a.k + tid) : 1.0f;
+            __syncthreads();
+            if (s_flag) {
+                wg_acquire();
+                for (int r = v0 + tid; r < v1; r += 256) {
+                    float acc = 0.0f;
+                    for (int jj = 0; jj < a.kk; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.kk + jj) * a.d + r), acc);
+                    a.out[(size_t) t * a.os + r] = a.res ? bfr(a.res[(size_t) t * a.os + r] + bfr(acc)) : acc;
+                }
+                if (tid == 0) st_agent(&tick[t * a.ntile_d + tile], 0u);
+            }
+        }
+        // the group's last down item leaves its three words at zero for the next launch
+        if (tid == 0 && atomicAdd(&grpc[g * 96 + 64], 1u) == (uint32_t) (a.ntile_d - 1)) {
+            st_agent(&grpc[g * 96], 0u);
+            st_agent(&grpc[g * 96 + 32], 0u);
+            st_agent(&grpc[g * 96 + 64], 0u);
+        }
+    }
+}
+
 int cu_count() {
     static int n = 0;
     if (!n) {
@@ -549,11 +871,57 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     return 0;
 }
 
+
+template <int P, int NT>
+int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
+    void (*kern)(FusedArgs) = sg ? (sd ? k_moe_decode_grouped<P, NT, true, true> : k_moe_decode_grouped<P, NT, true, false>)
+                                 : (sd ? k_moe_decode_grouped<P, NT, false, true> : k_moe_decode_grouped<P, NT, false, false>);
+    const int lmax = a.Lg > a.Ld ? a.Lg : a.Ld;
+    const size_t lds = (size_t) NT * lmax * XPAD * sizeof(float);
+    static int cached[2][2] = {{0, 0}, {0, 0}};   // resident workgroups per CU, by kernel variant, for the largest request seen
+    static size_t cached_lds[2][2] = {{0, 0}, {0, 0}};
+    int& per_cu = cached[sg][sd];
+    if (!per_cu || lds > cached_lds[sg][sd]) {
+        if (lds > 48 * 1024 && hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return -1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds) != hipSuccess || per_cu < 1) {
+            per_cu = 0;
+            return -1;
+        }
+        cached_lds[sg][sd] = lds;
+    }
+    // The groups are formed on the device; the host sizes the items for the number it expects from a uniform routing:
+    // the experts that receive a pair at all, plus the always-on experts' runs of NT tokens.
+    const double pairs = (double) a.T * a.k;
+    int groups = (int) (a.E * (1.0 - pow(1.0 - 1.0 / a.E, pairs)) + 0.5) + a.ns * ((a.T + NT - 1) / NT);
+    if (groups < 1) groups = 1;
+    const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count();
+    auto pick = [&](int iters) {
+        int best = 1;
+        long best_cost = -1;
+        for (int n = 1; n <= iters; ++n) {
+            const long rounds = ((long) groups * n + gmax - 1) / gmax, per = (iters + n - 1) / n;
+            const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
+            if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }
+        }
+        return best;
+    };
+    a.ntile_g = pick(a.it_g);
+    a.ntile_d = pick(a.it_d);
+    const long items = (long) groups * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
+    int grid = items < gmax ? (int) items : gmax;
+    if (grid < a.T) grid = a.T < gmax ? a.T : gmax;
+    a.grid = grid;
+    hipLaunchKernelGGL(kern, dim3((unsigned) grid), dim3(256), lds, st, a);
+    host_note_launch();
+    return 0;
+}
+
 }   // namespace
 
 extern "C" {
 
-size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1) + (size_t) T * 33 * 96; }
+size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1) + (size_t) T * 33 * 96 + FG_RN_WORDS; }
+int kc_moe_decode_max_rows(void) { return FG_MAXT; }
 int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
 
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
@@ -566,7 +934,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                         int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res, const float* norm_w,
                         float norm_eps) {
-    if (T < 1 || T > MV_MAXT || top_k < 1 || top_k > 32 || n_exp > 1024 || n_exp < top_k) return -1;
+    if (T < 1 || T > FG_MAXT || top_k < 1 || top_k > 32 || n_exp > 1024 || n_exp < top_k) return -1;
+    if (T > MV_MAXT && T * (top_k + (shared ? 1 : 0)) > FG_MAXP) return -1;
     if (fmt != MF_SEED4P4 && fmt != MF_SEED4) return -1;
     if (host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u)) return -1;
     FusedArgs a = {};
@@ -579,6 +948,14 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     for (int i = 0; i < 3 && shared; ++i) a.sh[i] = shared[i];
     a.it_g = (2 * ff + a.rpig - 1) / a.rpig;
     a.it_d = (d + a.rpid - 1) / a.rpid;
+    if (T > MV_MAXT) {
+        // More rows than the per-pair kernel takes: pairs grouped by expert, two to a decode.  Measured against the grouped
+        // GEMMs of the separate launches (C2, 16 rows: 236 against 268 us); with four to a decode (17 to 32 rows: 402 against
+        // 338 us at 32) and where the gate+up row sums go through LDS (C3's 45 chunks a row: 1129 against 753 us) the GEMMs
+        // win, so those shapes are left to them.
+        if (!sg) return -1;
+        return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
+    }
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);

@@ -90,7 +90,10 @@ def test_moe_step(oracle, router, T, slots):
             assert all(len(set(ind[t])) == k for t in range(T))
             # the layer output from the GPU's own routing
             for t in range(T):
-                ys = np.stack([expert_ref(oracle, gate, up, down, int(ind[t, j]), xn[t], gemm=T > 8) for j in range(k)])
+                # above 8 rows the separate launches take the grouped GEMM (BF16-rounded weights); the persistent kernel
+                # (softmax routing, every expert resident) keeps the exact weights of the decode path up to 16 rows
+                gemm = T > 8 and not (router == 0 and slots == 0 and T <= 16)
+                ys = np.stack([expert_ref(oracle, gate, up, down, int(ind[t, j]), xn[t], gemm=gemm) for j in range(k)])
                 if router == 0:
                     want = (wt[t].astype(np.float64)[:, None] * ys).sum(0)
                     tol = 2e-2 * np.abs(wt[t].astype(np.float64)[:, None] * ys).sum(0) + 1e-6
@@ -109,7 +112,7 @@ def test_moe_step(oracle, router, T, slots):
     st.close()
 
 
-@pytest.mark.parametrize("T", [1, 3, 8])
+@pytest.mark.parametrize("T", [1, 3, 8, 12, 16])
 def test_whole_expert_block_in_one_launch(T):
     """nslm_moe_step_layer (input RMSNorm + routed experts + shared expert + residual inside the persistent kernel) writes the
     same bits as kq4_norm1p + nslm_moe_step + kc_mv_gu / kc_mv (shared expert) + kc_residual_add."""
@@ -119,7 +122,7 @@ def test_whole_expert_block_in_one_launch(T):
     L, K = backend.hip(), backend.kt()
     rng = np.random.default_rng(77 + T)
     E, k, d, ff = 16, 4, 256, 128
-    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=8)
+    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=32)
     gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-12), packs.seed4p4(rng, E, ff, d, eb=-12), packs.seed4p4(rng, E, d, ff, eb=-12)
     st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.3).astype(np.float32)))
     st.finalize()
@@ -200,4 +203,43 @@ def test_fused_step_equal_logits(oracle, case, E):
             ids = [g for g in grp if g in sel]
             assert pos == sorted(pos, reverse=True) or len(ids) < 2, (sel, grp)
     assert np.mean([len(set(outs[0][0][t]) & set(oi[t])) / k for t in range(T)]) >= 0.75
+    st.close()
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("E", [16, 64])
+@pytest.mark.parametrize("T", [9, 13, 16])
+def test_grouped_step_equals_per_pair_steps(T, E, fmt):
+    """More than 8 rows: the persistent kernel groups the pairs of an expert, and every row comes out as the per-pair kernel
+    computes it in steps of at most 8 rows - routing, weights and outputs bit for bit (16 experts: many pairs an expert,
+    several groups; 64 experts: mostly one or two)."""
+    from nanoseedlm_amd import moe
+    rng = np.random.default_rng(900 + T + E)
+    k, d, ff = 4, 256, 192
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=16)
+    gate, up, down = mk(rng, E, ff, d, eb=-21), mk(rng, E, ff, d, eb=-21), mk(rng, E, d, ff, eb=-20)
+    st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+    st.finalize()
+    xn = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
+    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf.from_array(np.zeros((T, d), dtype=np.float32))
+    for rep in range(2):      # twice: the second launch finds the counters as the first left them
+        st.step(None, 0, dx.ptr, T, dio.ptr)
+        assert st.fused_error() == 0
+    ind, wt = st.last_routing(T)
+    out = dio.to_array(np.float32, (T, d))
+    dx.free(); dio.free()
+    assert np.abs(out).max() > 0
+    for r0 in range(0, T, 8):
+        n = min(8, T - r0)
+        dx, dio = moe.DevBuf.from_array(xn[r0:r0 + n]), moe.DevBuf.from_array(np.zeros((n, d), dtype=np.float32))
+        st.step(None, 0, dx.ptr, n, dio.ptr)
+        i2, w2 = st.last_routing(n)
+        o2 = dio.to_array(np.float32, (n, d))
+        dx.free(); dio.free()
+        assert np.array_equal(ind[r0:r0 + n], i2)
+        assert np.array_equal(wt[r0:r0 + n].view(np.uint32), w2.view(np.uint32))
+        bad = np.argwhere(out[r0:r0 + n].view(np.uint32) != o2.view(np.uint32))
+        assert len(bad) == 0, (r0, len(bad), bad[:6].tolist())
+    assert st.fused_error() == 0
     st.close()
