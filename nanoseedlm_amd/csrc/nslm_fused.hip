@@ -749,10 +749,14 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             staged_g = g;
             __syncthreads();
         }
-        rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part,
-                                         [&](int m, int r, float gs, float us) {
-                                             st_agent(a.A + (size_t) gm[g * NT + m] * a.ff + r, bfr(silu_bf(bfr(gs)) * bfr(us)));
-                                         });
+        auto put_a = [&](int m, int r, float gs, float us) {
+            st_agent(a.A + (size_t) gm[g * NT + m] * a.ff + r, bfr(silu_bf(bfr(gs)) * bfr(us)));
+        };
+        if (nt == 1)   // a group of one: the one-token loop, no second row of multiply-adds
+            rows_pass<P, true, SHFL_G>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, (float (*)[256]) part,
+                                       [&](int r, float gs, float us) { put_a(0, r, gs, us); });
+        else
+            rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part, put_a);
         wg_release();   // this item's rows of A are written: one more of the group's gate+up items is done
         __syncthreads();
         if (tid == 0 && atomicAdd(&grpc[g * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&grpc[g * 96 + 32], 1u);
@@ -781,8 +785,12 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         for (int m = 0; m < nt; ++m) stage_row(a.A + (size_t) gm[g * NT + m] * a.ff, a.ff, xl + m * xsd, true);
         staged_g = -1;
         __syncthreads();
-        rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part,
-                                          [&](int m, int r, float sm, float) { st_agent(a.D + (size_t) gm[g * NT + m] * a.d + r, bfr(sm)); });
+        auto put_d = [&](int m, int r, float sm, float) { st_agent(a.D + (size_t) gm[g * NT + m] * a.d + r, bfr(sm)); };
+        if (nt == 1)
+            rows_pass<P, false, SHFL_D>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, (float (*)[256]) part,
+                                        [&](int r, float sm, float) { put_d(0, r, sm, 0.0f); });
+        else
+            rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part, put_d);
         wg_release();
         for (int m = 0; m < nt; ++m) {   // one ticket per member's (token, row tile); the token's last arrival sums its experts
             const int t = gm[g * NT + m] / a.kk;
