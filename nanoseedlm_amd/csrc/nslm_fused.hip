@@ -1,5 +1,6 @@
-// nslm_fused.hip - one persistent kernel for a whole routed-expert decode step at T <= 8 tokens: router logits, softmax
-// top-k, fused gate + up + SwiGLU gather, down gather, weighted combine.  No counterpart in the reference, which launches
+// nslm_fused.hip - one persistent kernel for a whole routed-expert decode step at T <= 8 tokens (k_moe_decode; 9 to 16
+// tokens: k_moe_decode_grouped further down): router logits, softmax top-k, fused gate + up + SwiGLU gather, down gather,
+// weighted combine.  No counterpart in the reference, which launches
 // these as five kernels (engine/qwen4_cuda.c:1023-1083); on MI355X each launch and each dependent global read costs
 // microseconds that a ~20 us step cannot afford, so the phases run inside one grid separated by grid-wide barriers.
 //
