@@ -33,6 +33,7 @@ struct MvArgs {
     float* y;
     const int32_t* sel;
     int K, R, xdiv, xs, ys, add, nt, f32out;
+    int ttot;             // dense modes with NT > 1: tokens of the launch; workgroup row blockIdx.y takes tokens NT y .. (nt = NT)
     int L, rpi, rows_per_wg;   // fast path: chunks per row, rows per iteration, virtual rows per workgroup
     // MULTI: up to MV_MAXJ dense matrices over the same x in one launch; job j owns workgroups [wg0[j], wg0[j + 1])
     WSlice wj[4];
@@ -63,7 +64,12 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
         wg -= a.wg0[job];
     }
     const int R = MODE == MULTI ? a.Rj[job] : a.R, ys = MODE == MULTI ? a.ysj[job] : a.ys, add = MODE == MULTI ? a.addj[job] : a.add;
-    float* const yb = MODE == MULTI ? a.yj[job] : a.y;
+    // staged dense passes: the launch's tokens are dealt to grid.y in runs of NT, so a workgroup stages NT rows however
+    // many tokens there are (16 rows in one workgroup's LDS left room for one workgroup a CU)
+    constexpr bool TGRP = DN && NT > 1;
+    const int tg0 = TGRP ? (int) blockIdx.y * NT : 0, nt_ = TGRP ? min(NT, a.ttot - tg0) : a.nt;
+    const float* const xbase = a.x + (size_t) tg0 * a.xs;
+    float* const yb = (MODE == MULTI ? a.yj[job] : a.y) + (size_t) tg0 * (MODE == MULTI ? a.ysj[job] : a.ys);
     const int V = MODE == GATEUP ? 2 * R : R;   // virtual rows: gate row r = 2r, up row r = 2r + 1
     const int v0 = wg * a.rows_per_wg, v1 = min(v0 + a.rows_per_wg, V);
     WSlice wA = MODE == MULTI ? a.wj[job] : a.wd, wB = wA;
@@ -121,19 +127,19 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
         // run-time count waits for every load in turn).
         __shared__ float rn_s[NT];
         if (prenorm) {
-            for (int t = 0; t < a.nt; ++t) {
-                const float rn = row_rnorm(a.x + (size_t) t * a.xs, a.K, a.neps, nred);
+            for (int t = 0; t < nt_; ++t) {
+                const float rn = row_rnorm(xbase + (size_t) t * a.xs, a.K, a.neps, nred);
                 if (tid == 0) rn_s[t] = rn;
             }
             __syncthreads();
         }
-        const int K4 = a.K / 4, tot = a.nt * K4;
+        const int K4 = a.K / 4, tot = nt_ * K4;
         for (int base = tid; base < tot; base += 256 * 8) {
             float4 q[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int idx = min(base + 256 * j, tot - 1), t = idx / K4, i = idx - t * K4;
-                q[j] = ((const float4*) (a.x + (size_t) t * a.xs))[i];
+                q[j] = ((const float4*) (xbase + (size_t) t * a.xs))[i];
             }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -163,12 +169,12 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
         const int eb = (MODE == GATEUP && (v & 1)) ? eB : eA;
         if (active && v < v1) {
             if (NT == 1) chunk_dot<P, NT>(cur, eb, tab, xreg, 0, 1, acc);
-            else chunk_dot<P, NT>(cur, eb, tab, xl + ch * XPAD, L * XPAD, a.nt, acc);
+            else chunk_dot<P, NT>(cur, eb, tab, xl + ch * XPAD, L * XPAD, nt_, acc);
         }
         if (SHFL) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                if (NT > 1 && t >= a.nt) break;
+                if (NT > 1 && t >= nt_) break;
                 float s = acc[t];
                 for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
                 if (MODE == GATEUP) {
@@ -197,11 +203,13 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                     float* yo = yb + (size_t) pair * ys + ((vb >> 1) + tid);
                     *yo = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                 }
-            } else if (tid < nrow * (NT > 1 ? a.nt : 1)) {
-                const int t = tid / nrow, r = tid - t * nrow;
-                float s = 0.0f;
-                for (int j = 0; j < L; ++j) s += part[par][t][r * L + j];
-                store_y(yb + (size_t) (DN ? t : pair) * ys + (vb + r), s * NSLM_R32, add, a.f32out);
+            } else {
+                for (int w = tid; w < nrow * (NT > 1 ? nt_ : 1); w += 256) {   // (token, row) sums: more than 256 with many tokens of short rows
+                    const int t = w / nrow, r = w - t * nrow;
+                    float s = 0.0f;
+                    for (int j = 0; j < L; ++j) s += part[par][t][r * L + j];
+                    store_y(yb + (size_t) (DN ? t : pair) * ys + (vb + r), s * NSLM_R32, add, a.f32out);
+                }
             }
         }
         cur = nxt;
@@ -491,9 +499,7 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
 
 void note_launch() { nslm::host_note_launch(); }
 
-#define MV_TG 4   // tokens per pass of the multi-token fast path (activations staged in LDS); MV_TG2 when more than MV_TG remain
-#define MV_TG2 8
-#define MV_TG3 16   // one pass of 16 when the rows fit the LDS (K <= 2176): small matrices leave one workgroup a CU anyway
+#define MV_TG 4   // tokens a workgroup of the multi-token fast path stages in LDS
 #define MV_MULTI_MAXT 64
 
 }   // namespace
@@ -529,22 +535,21 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(R, rpi, 1);
         const dim3 grid((unsigned) ((R + a.rows_per_wg - 1) / a.rows_per_wg), 1);
-        // Tokens go in passes of at most MV_TG; a token's arithmetic is the same in every pass size.  Rows too long for
-        // the LDS staging take one pass per token with the activations in registers.
-        const bool stage = T > 1 && L <= 96;
-        const bool wide8 = stage && (size_t) MV_TG2 * L * XPAD * sizeof(float) <= 72 * 1024;   // two workgroups a CU still fit
-        for (int t0 = 0; t0 < T;) {
-            MvArgs b = a;
-            b.x = x + (size_t) t0 * xs;
-            b.y = y + (size_t) t0 * ys;
-            const bool wide16 = wide8 && (size_t) MV_TG3 * L * XPAD * sizeof(float) <= 150 * 1024;
-            const int tg = !stage ? 1 : (wide16 && T - t0 > MV_TG2) ? MV_TG3 : (wide8 && T - t0 > MV_TG) ? MV_TG2 : MV_TG;
-            b.nt = T - t0 < tg ? T - t0 : tg;
-            if (tg == MV_TG3) launch_seed_fmt<DENSE, MV_TG3>(st, fmt, b, shfl, grid, (size_t) MV_TG3 * L * XPAD * sizeof(float));
-            else if (tg == MV_TG2) launch_seed_fmt<DENSE, MV_TG2>(st, fmt, b, shfl, grid, (size_t) MV_TG2 * L * XPAD * sizeof(float));
-            else if (stage) launch_seed_fmt<DENSE, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
-            else launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid, 0);
-            t0 += tg;
+        // Several tokens: their activations staged in LDS, MV_TG tokens a workgroup, the runs of MV_TG tokens dealt to grid.y
+        // (a token's arithmetic does not depend on the run it is in).  One workgroup for all of 16 tokens needed 139 KB of
+        // LDS, i.e. one workgroup a CU: 2048 x 2048 at 16 tokens 21.5 us, in runs of four 14.1 us (8 tokens: 12.6 -> 9.9).
+        // Rows too long for the staging take one launch per token with the activations in registers.
+        if (T > 1 && L <= 96) {
+            a.ttot = T;
+            launch_seed_fmt<DENSE, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG), (size_t) MV_TG * L * XPAD * sizeof(float));
+        } else {
+            for (int t0 = 0; t0 < T; ++t0) {
+                MvArgs b = a;
+                b.x = x + (size_t) t0 * xs;
+                b.y = y + (size_t) t0 * ys;
+                b.nt = 1;
+                launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid, 0);
+            }
         }
         note_launch();
         return;
@@ -573,19 +578,14 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     }
     const dim3 grid((unsigned) a.wg0[n], 1);
     hipStream_t st = (hipStream_t) s;
-    const bool wide8 = (size_t) MV_TG2 * L * XPAD * sizeof(float) <= 72 * 1024;
-    for (int t0 = 0; t0 < T;) {   // passes of tokens as kc_mv's: a token's arithmetic is the same in every pass size
-        MvArgs b = a;
-        b.x = x + (size_t) t0 * xs;
-        for (int j = 0; j < n; ++j) b.yj[j] = y[j] + (size_t) t0 * ys[j];
-        const bool wide16 = wide8 && (size_t) MV_TG3 * L * XPAD * sizeof(float) <= 150 * 1024;
-        const int tg = T == 1 ? 1 : (wide16 && T - t0 > MV_TG2) ? MV_TG3 : (wide8 && T - t0 > MV_TG) ? MV_TG2 : MV_TG;
-        b.nt = T - t0 < tg ? T - t0 : tg;
-        if (tg == MV_TG3) launch_seed_fmt<MULTI, MV_TG3>(st, fmt, b, shfl, grid, (size_t) MV_TG3 * L * XPAD * sizeof(float));
-        else if (tg == MV_TG2) launch_seed_fmt<MULTI, MV_TG2>(st, fmt, b, shfl, grid, (size_t) MV_TG2 * L * XPAD * sizeof(float));
-        else if (tg == MV_TG) launch_seed_fmt<MULTI, MV_TG>(st, fmt, b, shfl, grid, (size_t) MV_TG * L * XPAD * sizeof(float));
-        else launch_seed_fmt<MULTI, 1>(st, fmt, b, shfl, grid, 0);
-        t0 += tg;
+    if (T == 1) {
+        a.nt = 1;
+        for (int j = 0; j < n; ++j) a.yj[j] = y[j];
+        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, 0);
+    } else {   // runs of MV_TG tokens over grid.y, as kc_mv's
+        a.ttot = T;
+        for (int j = 0; j < n; ++j) a.yj[j] = y[j];
+        launch_seed_fmt<MULTI, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG), (size_t) MV_TG * L * XPAD * sizeof(float));
     }
     note_launch();
     return 0;
