@@ -33,7 +33,6 @@ struct MvArgs {
     float* y;
     const int32_t* sel;
     int K, R, xdiv, xs, ys, add, nt, f32out;
-    int ttot;             // dense modes with NT > 1: tokens of the launch; workgroup row blockIdx.y takes tokens NT y .. (nt = NT)
     int L, rpi, rows_per_wg;   // fast path: chunks per row, rows per iteration, virtual rows per workgroup
     // MULTI: up to MV_MAXJ dense matrices over the same x in one launch; job j owns workgroups [wg0[j], wg0[j + 1])
     WSlice wj[4];
@@ -41,6 +40,9 @@ struct MvArgs {
     int Rj[4], ysj[4], addj[4], wg0[5], nj;
     const float* nw;      // non-null (dense modes): x is normalised first, xn_k = x_k r (1 + nw_k), r = rsqrt(mean(x^2) + neps)
     float neps;
+    int ttot;             // dense modes with NT > 1: tokens of the launch; workgroup row blockIdx.y takes tokens NT y .. (nt = NT)
+                          // (last, so that the one-token kernels read their arguments where they always did: a field
+                          // added in the middle cost them a second round of argument loads, 0.3 us a launch)
 };
 #define MV_MAXJ 4
 
