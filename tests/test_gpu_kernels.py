@@ -383,7 +383,7 @@ def test_cache_copy_moves_units(be):
 
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
-@pytest.mark.parametrize("T", [1, 3, 8])
+@pytest.mark.parametrize("T", [1, 3, 8, 13, 16])
 def test_mv_multi_equals_separate_matvecs(fmt, T):
     """kc_mv_multi: several dense seed matrices over the same x in one launch, bit-equal to one kc_mv each (ragged row
     counts, one job accumulating into y)."""
@@ -434,3 +434,40 @@ def test_mv_multi_equals_separate_matvecs(fmt, T):
     for j, R in enumerate(Rs):
         a, b = yc[j].to_array(np.float32, (T, R)), yd[j].to_array(np.float32, (T, R))
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32)) and not np.array_equal(a, ya[j].to_array(np.float32, (T, R))), j
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("K,R", [(768, 300), (2048, 96), (256, 1000)])
+@pytest.mark.parametrize("T", [5, 16, 23, 64])
+def test_mv_many_tokens_equal_single_token_calls(fmt, K, R, T):
+    """kc_mv over T tokens (runs of four tokens dealt to grid.y) gives every token the bits of a one-token call: batch
+    invariance beyond the reference's 8 tokens (engine/kernels_moe.cu:239-240).  K = 768: 12 chunks a row, row sums through
+    LDS with more (token, row) sums than threads at four tokens; add = 1 accumulates into y."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(7 * T + K)
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    p = mk(rng, 1, R, K, eb=-20)
+    words = p["coefs"] if fmt == packs.MF_SEED4P4 else p["nibs"]
+    bufs = [moe.DevBuf.from_array(p["seeds"][0]), moe.DevBuf.from_array(words[0])]
+    w = backend.WSlice()
+    w.p[0], w.p[1], w.eb = bufs[0].ptr.value, bufs[1].ptr.value, int(p["eb"][0])
+    if fmt == packs.MF_SEED4P4:
+        bufs.append(moe.DevBuf.from_array(p["codes"][0]))
+        w.p[3] = bufs[2].ptr.value
+    x = packs.round_bf16(rng.standard_normal((T, K)).astype(np.float32))
+    y0 = packs.round_bf16(rng.standard_normal((T, R)).astype(np.float32))
+    dx = moe.DevBuf.from_array(x)
+    for add in (0, 1):
+        ya, yb = moe.DevBuf.from_array(y0), moe.DevBuf.from_array(y0)
+        L.kc_mv(None, fmt, w, K, R, dx.ptr, K, ya.ptr, R, T, add, None)
+        for t in range(T):
+            L.kc_mv(None, fmt, w, K, R, dx.at(4 * t * K), K, yb.at(4 * t * R), R, 1, add, None)
+        moe.device_sync()
+        assert L.kc_last_error() == 0
+        a, b = ya.to_array(np.float32, (T, R)), yb.to_array(np.float32, (T, R))
+        bad = np.argwhere(a.view(np.uint32) != b.view(np.uint32))
+        assert not np.array_equal(a, y0) and len(bad) == 0, (add, len(bad), bad[:6].tolist())
+        ya.free(); yb.free()
