@@ -207,15 +207,15 @@ def test_fused_step_equal_logits(oracle, case, E):
 
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
-@pytest.mark.parametrize("E", [16, 64])
+@pytest.mark.parametrize("E,k", [(16, 4), (64, 4), (200, 8), (300, 6)])
 @pytest.mark.parametrize("T", [9, 13, 16])
-def test_grouped_step_equals_per_pair_steps(T, E, fmt):
+def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
     """More than 8 rows: the persistent kernel groups the pairs of an expert, and every row comes out as the per-pair kernel
     computes it in steps of at most 8 rows - routing, weights and outputs bit for bit (16 experts: many pairs an expert,
     several groups; 64 experts: mostly one or two)."""
     from nanoseedlm_amd import moe
     rng = np.random.default_rng(900 + T + E)
-    k, d, ff = 4, 256, 192
+    d, ff = 256, 192
     mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
     st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=16)
     gate, up, down = mk(rng, E, ff, d, eb=-21), mk(rng, E, ff, d, eb=-21), mk(rng, E, d, ff, eb=-20)
