@@ -279,7 +279,6 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
 #define DSTAMP(i) do { } while (0)
 #endif
     STAMP(0);
-    load_tables(tab);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
     uint32_t* pairc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [pair][3][32]: arrivals, ready, done
@@ -337,6 +336,9 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
         if (lane == 0) st_agent(a.logits + item, bfr(acc));
     }
+    // The decode tables are first needed after the barrier: loaded here, behind the logits (the workgroups that form logits
+    // are the last to reach the barrier; tables first was one more memory round trip on their way).
+    load_tables(tab);
     // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
     if ((int) blockIdx.x < items_g) {
         staged = ((int) blockIdx.x / a.ntile_g) / a.kk;
