@@ -56,8 +56,9 @@ struct FusedArgs {
 //                        poll: polling the counter's line would slow the arrivals), finished down items
 // Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
 // counters and only each group's last arrival touches the shared one; waiters poll their own group's sense word.  The
-// barrier is sense-reversing (each group's word flips from its own value, so launches with different numbers of groups
-// and any number of barriers a launch can follow each other) and resets its own counters: no clean-up between launches.
+// barrier's sense words hold a generation number, the same in all of them (whoever opens a barrier writes the next number to
+// every word), so launches with different numbers of groups and any number of barriers a launch can follow each other;
+// the counters are reset by the last arrival: no clean-up between launches.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
 #define FUSED_SYNC_WORDS (32 * (2 * BAR_GROUPS + 2))
@@ -84,15 +85,13 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G) {
             if (atomicAdd(sync + 32 * BAR_GROUPS, 1u) == ng - 1) {
                 st_agent(sync + 32 * BAR_GROUPS, 0u);
                 wg_release();   // every counter is back at zero before anyone is let through
-                // Each group's word flips from ITS OWN value: launches of different grid sizes use different numbers of
-                // groups, so after an odd number of barriers the words need not agree with each other.
-                // (all the words are read before any is written: 32 independent loads, then 32 stores)
-                uint32_t cur[BAR_GROUPS];
+                // All BAR_GROUPS words always hold the same number: whoever opens a barrier writes s + 1 to every one of
+                // them, whatever the number of groups of its launch (s = its own group's word, read before its arrival,
+                // and no barrier can have opened since).  Launches of different grid sizes and any number of barriers a
+                // launch can therefore follow each other, and opening costs no loads.  (Flipping only the words of the
+                // launch's groups left stale values behind a smaller grid; reading all words first cost a round trip.)
 #pragma unroll
-                for (uint32_t i = 0; i < BAR_GROUPS; ++i) cur[i] = ld_agent(sync + 32 * (BAR_GROUPS + 1 + i));
-#pragma unroll
-                for (uint32_t i = 0; i < BAR_GROUPS; ++i)
-                    if (i < ng) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), cur[i] ^ 1u);
+                for (uint32_t i = 0; i < BAR_GROUPS; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), s + 1u);
             }
         }
         uint32_t spins = 0;
