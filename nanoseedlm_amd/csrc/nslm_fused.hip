@@ -47,9 +47,9 @@ struct FusedArgs {
 };
 
 // Barrier words (uint32; every counter sits alone on a 128-byte line = 32 words):
-//   [32 g]              arrivals of group g = blockIdx.x % BAR_GROUPS
-//   [32 BAR_GROUPS]     groups that are complete
-//   [32 (BAR_GROUPS+1+g)] group g's sense word: flipped when the barrier opens
+//   [32 g], [32 g + 1]   arrivals of group g = blockIdx.x % BAR_GROUPS, for barriers of even / odd generation
+//   [32 BAR_GROUPS], [.. + 1] groups that are complete (even / odd generation)
+//   [32 (BAR_GROUPS+1+g)] group g's sense word: the generation, advanced when the barrier opens
 //   [32 (2 BAR_GROUPS+1)] error word
 //   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile); behind them (at T (d + 1)) three words per pair, each on
 //                        its own line: finished gate+up items (atomics only), the pair's ready flag (what waiters
@@ -58,7 +58,8 @@ struct FusedArgs {
 // counters and only each group's last arrival touches the shared one; waiters poll their own group's sense word.  The
 // barrier's sense words hold a generation number, the same in all of them (whoever opens a barrier writes the next number to
 // every word), so launches with different numbers of groups and any number of barriers a launch can follow each other;
-// the counters are reset by the last arrival: no clean-up between launches.
+// the counters are reset by the last arrival (two sets by generation parity, so that the reset needs no wait): no clean-up
+// between launches.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
 #define FUSED_SYNC_WORDS (32 * (2 * BAR_GROUPS + 2))
@@ -72,24 +73,31 @@ __device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) { __hip_atomic
 __device__ __forceinline__ void wg_release() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
 __device__ __forceinline__ void wg_acquire() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
-// every workgroup of the grid arrives and waits (bounded); data written before it by any workgroup is visible after it
-__device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G) {
+// The generation the next barrier of this launch starts from (thread 0 keeps it; requested at the start of the kernel so
+// that the load is not on the way of the first barrier's last arrival).
+__device__ __forceinline__ uint32_t barrier_generation(const uint32_t* sync) {
+    return threadIdx.x == 0 ? ld_agent(sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS)) : 0u;
+}
+// every workgroup of the grid arrives and waits (bounded); data written before it by any workgroup is visible after it.
+// gen: the generation before this barrier (barrier_generation() for the first one); advanced on return.
+__device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G, uint32_t& gen) {
     wg_release();
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t g = blockIdx.x % BAR_GROUPS, ng = G < BAR_GROUPS ? G : BAR_GROUPS, mine = (G - g + BAR_GROUPS - 1) / BAR_GROUPS;
+        const uint32_t s = gen, set = s & 1u;   // two sets of counters, by generation parity (second word of the same lines)
         uint32_t* sense = sync + 32 * (BAR_GROUPS + 1 + g);
-        const uint32_t s = ld_agent(sense);   // read before arriving: the barrier cannot open without this arrival
-        if (atomicAdd(sync + 32 * g, 1u) == mine - 1) {
-            st_agent(sync + 32 * g, 0u);
-            if (atomicAdd(sync + 32 * BAR_GROUPS, 1u) == ng - 1) {
-                st_agent(sync + 32 * BAR_GROUPS, 0u);
-                wg_release();   // every counter is back at zero before anyone is let through
+        if (atomicAdd(sync + 32 * g + set, 1u) == mine - 1) {
+            // The counters go back to zero without a wait: the next barrier counts in the other set, and nobody can reach
+            // the barrier after that one before this workgroup has arrived at the next, which it does only after its
+            // stores have completed (the release fence at the top).
+            st_agent(sync + 32 * g + set, 0u);
+            if (atomicAdd(sync + 32 * BAR_GROUPS + set, 1u) == ng - 1) {
+                st_agent(sync + 32 * BAR_GROUPS + set, 0u);
                 // All BAR_GROUPS words always hold the same number: whoever opens a barrier writes s + 1 to every one of
-                // them, whatever the number of groups of its launch (s = its own group's word, read before its arrival,
-                // and no barrier can have opened since).  Launches of different grid sizes and any number of barriers a
-                // launch can therefore follow each other, and opening costs no loads.  (Flipping only the words of the
-                // launch's groups left stale values behind a smaller grid; reading all words first cost a round trip.)
+                // them, whatever the number of groups of its launch.  Launches of different grid sizes and any number of
+                // barriers a launch can therefore follow each other, and opening costs no loads.  (Flipping only the words
+                // of the launch's groups left stale values behind a smaller grid; reading all words first cost a round trip.)
 #pragma unroll
                 for (uint32_t i = 0; i < BAR_GROUPS; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), s + 1u);
             }
@@ -102,6 +110,7 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G) {
                 break;
             }
         }
+        gen = s + 1u;
     }
     __syncthreads();
     wg_acquire();
@@ -278,6 +287,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
 #define DSTAMP(i) do { } while (0)
 #endif
     STAMP(0);
+    uint32_t bar_gen = barrier_generation(a.sync);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
     uint32_t* pairc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [pair][3][32]: arrivals, ready, done
@@ -344,7 +354,7 @@ __global__ void __launch_bounds__(256, 5) k_moe_decode(FusedArgs a) {   // five 
         stage_input(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
     }
     STAMP(1);
-    grid_barrier(a.sync, G);
+    grid_barrier(a.sync, G, bar_gen);
     STAMP(2);
 
     // ---- route: every workgroup ranks the logits of the token it needs (cheap, and saves a grid barrier) ----------------
@@ -592,6 +602,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
     uint32_t* grpc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [group][3][32]: arrivals, ready, done
     float* rnpub = (float*) (grpc + (size_t) a.T * 33 * 96);
+    uint32_t bar_gen = barrier_generation(a.sync);
     load_tables(tab);
 
     // ---- phase 1: router logits, one wave per (token, expert) -------------------------------------------------------------
@@ -648,7 +659,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
         if (lane == 0) st_agent(a.logits + item, bfr(acc));
     }
-    grid_barrier(a.sync, G);
+    grid_barrier(a.sync, G, bar_gen);
 
     // ---- routing, once per token: workgroup t % G ranks token t and publishes selection, weights and the row's scale ----
     for (int t = (int) blockIdx.x; t < a.T; t += (int) G) {
@@ -672,7 +683,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             if (tid == 0) st_agent(rnpub + t, r);
         }
     }
-    grid_barrier(a.sync, G);
+    grid_barrier(a.sync, G, bar_gen);
 
     // ---- the groups: the same table in every workgroup ----------------------------------------------------------------------
     for (int i = tid; i < NE; i += 256) cnt_s[i] = 0;

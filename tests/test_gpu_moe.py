@@ -243,3 +243,32 @@ def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
         assert len(bad) == 0, (r0, len(bad), bad[:6].tolist())
     assert st.fused_error() == 0
     st.close()
+
+
+def test_steps_of_changing_size_share_the_barrier_words():
+    """Launches with one grid barrier (up to 8 rows) and two (9 to 16 rows), of different grid sizes, follow each other on
+    one set of barrier words: no barrier gives up, and every step returns what the same step returned the first time."""
+    from nanoseedlm_amd import moe
+    rng = np.random.default_rng(4242)
+    E, k, d, ff = 32, 4, 256, 192
+    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=16)
+    gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, d, ff, eb=-20)
+    st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+    st.finalize()
+    xn = packs.round_bf16(rng.standard_normal((16, d)).astype(np.float32))
+    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf(4 * 16 * d)
+    first = {}
+    for rep in range(6):
+        for T in (1, 12, 3, 16, 8, 9, 9, 2, 13, 1, 1, 16):
+            st.step(None, 0, dx.ptr, T, dio.ptr)
+            out = dio.to_array(np.float32, (16, d))[:T].copy()
+            assert st.fused_error() == 0, (rep, T)
+            if T not in first:
+                first[T] = out
+                assert np.abs(out).max() > 0
+            assert np.array_equal(out.view(np.uint32), first[T].view(np.uint32)), (rep, T)
+    # rows are the same whatever the step size they came in
+    assert np.array_equal(first[16][:8].view(np.uint32), first[8].view(np.uint32))
+    assert np.array_equal(first[13][:1].view(np.uint32), first[1].view(np.uint32))
+    dx.free(); dio.free()
+    st.close()
