@@ -146,7 +146,9 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
         const Chunk nxt = fetch(v + rpi);
         float acc[1] = {0.0f};
         const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
-        if (active && v < v1) chunk_dot<P, 1, true>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
+        // (two blocks at a time in phase order where three workgroups a CU compute at once; the down pass, whose waves mostly
+        // run alone behind their pair's readiness, keeps the compiler's order)
+        if (active && v < v1) chunk_dot<P, 1, GATEUP>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
         if (SHFL) {
             float s = acc[0];
             for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
