@@ -51,6 +51,10 @@ struct FusedArgs {
 //   [32 BAR_GROUPS], [.. + 1] groups that are complete (even / odd generation)
 //   [32 (BAR_GROUPS+1+g)] group g's sense word: the generation, advanced when the barrier opens
 //   [32 (2 BAR_GROUPS+1)] error word
+//   [FUSED_LOGIT_WORDS ..] the per-pair kernel's router logits [MV_MAXT][E], each a 64-bit word: the BF16 value's float
+//                        bits below, the launch's generation + 1 above.  A reader polls until the upper half is its own
+//                        launch's: the logits need no grid barrier.  Every launch rewrites all MV_MAXT rows (rows it does
+//                        not use with zero), so a stale word is always the preceding launch's and never matches.
 //   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile); behind them (at T (d + 1)) three words per pair, each on
 //                        its own line: finished gate+up items (atomics only), the pair's ready flag (what waiters
 //                        poll: polling the counter's line would slow the arrivals), finished down items
@@ -62,13 +66,16 @@ struct FusedArgs {
 // between launches.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
-#define FUSED_SYNC_WORDS (32 * (2 * BAR_GROUPS + 2))
+#define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // MV_MAXT x 1024 router logits, 64 bits each: value | generation << 32
+#define FUSED_SYNC_WORDS (FUSED_LOGIT_WORDS + 2 * MV_MAXT * 1024)
 #define SPIN_LIMIT (1u << 21)
 
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ unsigned long long ld_agent(const unsigned long long* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_agent(unsigned long long* p, unsigned long long v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 // this workgroup's earlier memory operations have completed / later ones start after this point
 __device__ __forceinline__ void wg_release() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
 __device__ __forceinline__ void wg_acquire() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
@@ -114,6 +121,21 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G, uint32_
     }
     __syncthreads();
     wg_acquire();
+}
+
+// A launch without a grid barrier still moves the generation on: every workgroup arrives (nobody waits), the last arrival
+// writes the next number.  Called by thread 0 after every wave of the workgroup has read the generation.
+__device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t G, uint32_t gen) {
+    const uint32_t g = blockIdx.x % BAR_GROUPS, ng = G < BAR_GROUPS ? G : BAR_GROUPS, mine = (G - g + BAR_GROUPS - 1) / BAR_GROUPS;
+    const uint32_t set = gen & 1u;
+    if (atomicAdd(sync + 32 * g + set, 1u) == mine - 1) {
+        st_agent(sync + 32 * g + set, 0u);
+        if (atomicAdd(sync + 32 * BAR_GROUPS + set, 1u) == ng - 1) {
+            st_agent(sync + 32 * BAR_GROUPS + set, 0u);
+#pragma unroll
+            for (uint32_t i = 0; i < BAR_GROUPS; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), gen + 1u);
+        }
+    }
 }
 
 // The first chunk of a pass over rows [v0, v1): issued as early as the slices are known, so its latency hides behind
@@ -274,6 +296,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     __shared__ int ri_s[33];        // route: expert by rank
     __shared__ WSlice sl_s[3][33];  // route: the chosen experts' gate / up / down slices (+ the shared expert's)
     __shared__ int s_flag;
+    __shared__ uint32_t s_tag;
     __shared__ float rn_s[MV_MAXT], nred[4];   // the rows' RMSNorm scales when the kernel normalises its input
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t G = (uint32_t) a.grid;
@@ -289,7 +312,9 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 #define DSTAMP(i) do { } while (0)
 #endif
     STAMP(0);
-    uint32_t bar_gen = barrier_generation(a.sync);
+    // the generation: lane 0 of every wave reads it (all sense words are equal); the workgroup arrives further down
+    const uint32_t my_gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
+    unsigned long long* lg64 = (unsigned long long*) (a.sync + FUSED_LOGIT_WORDS);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
     uint32_t* pairc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [pair][3][32]: arrivals, ready, done
@@ -345,7 +370,12 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             }
         }
         for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-        if (lane == 0) st_agent(a.logits + item, bfr(acc));
+        const float lv = bfr(acc);
+        if (lane == 0) {
+            st_agent(a.logits + item, lv);
+            st_agent(lg64 + item, (unsigned long long) __float_as_uint(lv) | (unsigned long long) (my_gen + 1u) << 32);
+        }
+        if (t == 0 && lane >= a.T && lane < MV_MAXT) st_agent(lg64 + (size_t) lane * a.E + e, 0ull);   // rows this launch does not use
     }
     // The decode tables are first needed after the barrier: loaded here, behind the logits (the workgroups that form logits
     // are the last to reach the barrier; tables first was one more memory round trip on their way).
@@ -356,7 +386,12 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         stage_input(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
     }
     STAMP(1);
-    grid_barrier(a.sync, G, bar_gen);
+    // No grid barrier: what the other workgroups produce here are the logits, and those say themselves when they are there.
+    __syncthreads();   // every wave has used its copy of the generation
+    if (tid == 0) {
+        s_tag = my_gen + 1u;
+        grid_arrive(a.sync, G, my_gen);
+    }
     STAMP(2);
 
     // ---- route: every workgroup ranks the logits of the token it needs (cheap, and saves a grid barrier) ----------------
@@ -368,7 +403,22 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         routed = t;
         __syncthreads();
         const int E4 = (a.E + 3) & ~3;
-        for (int e = tid; e < E4; e += 256) rv[e] = e < a.E ? ld_agent(a.logits + (size_t) t * a.E + e) : __uint_as_float(0xFF800000u);
+        const uint32_t tag = s_tag;
+        for (int e = tid; e < E4; e += 256) {
+            float v = __uint_as_float(0xFF800000u);
+            if (e < a.E) {   // the logit's word carries this launch's tag once its wave has stored it (bounded wait)
+                unsigned long long w = ld_agent(lg64 + (size_t) t * a.E + e);
+                for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(lg64 + (size_t) t * a.E + e)) {
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > SPIN_LIMIT) {
+                        atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                        break;
+                    }
+                }
+                v = __uint_as_float((uint32_t) w);
+            }
+            rv[e] = v;
+        }
         __syncthreads();
         unsigned long long tq[4] = {0, 0, 0, 0};
         (void) tq;
