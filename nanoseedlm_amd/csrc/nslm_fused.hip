@@ -2,7 +2,9 @@
 // tokens: k_moe_decode_grouped further down): router logits, softmax top-k, fused gate + up + SwiGLU gather, down gather,
 // weighted combine.  No counterpart in the reference, which launches
 // these as five kernels (engine/qwen4_cuda.c:1023-1083); on MI355X each launch and each dependent global read costs
-// microseconds that a ~20 us step cannot afford, so the phases run inside one grid separated by grid-wide barriers.
+// microseconds that a ~20 us step cannot afford, so the phases run inside one grid: the data that crosses workgroups says
+// itself when it is there (generation-tagged router logits, one ready flag per pair), and the kernel for 9 to 16 tokens
+// adds two grid-wide barriers.
 //
 // Arithmetic is the stand-alone kernels', instruction for instruction (k_mv_any's BF16 row dot, k_q4_route's selection
 // and weights, k_mv_seed's chunk products and row-sum order, k_q4_moe_combine's sum), so the fused step returns the same
@@ -14,9 +16,10 @@
 // ordering against the barrier counters is a workgroup-scope release / acquire, i.e. a wait for outstanding memory
 // operations.
 //
-// Grid barriers: the grid is sized to the number of workgroups the device can hold at once (occupancy query), every
-// workgroup arrives on a counter in caller-provided scratch and spins until all have; the spin is bounded, and a
-// workgroup that gives up sets an error word and runs on to the end, so every wave always exits.
+// Waiting: the grid is sized to the number of workgroups the device can hold at once (occupancy query), because
+// workgroups wait for each other's data (and, in the grouped kernel, for each other at its barriers: every workgroup
+// arrives on a counter in caller-provided scratch and spins until all have); every wait is bounded, and a workgroup that
+// gives up sets an error word and runs on to the end, so every wave always exits.
 #include <math.h>
 #include <stdlib.h>
 
