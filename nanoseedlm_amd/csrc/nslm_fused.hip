@@ -127,11 +127,16 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G, uint32_
 }
 
 // A launch without a grid barrier still moves the generation on: every workgroup arrives (nobody waits), the last arrival
-// writes the next number.  Called by thread 0 after every wave of the workgroup has read the generation.
-__device__ __forceinline__ void grid_arrive(uint32_t* sync, uint32_t G, uint32_t gen) {
+// writes the next number.  By thread 0, after every wave of the workgroup has read the generation.  In two halves, so
+// that the atomic's round trip lies under other work: arrive_issue() returns what the group's counter held, and
+// arrive_finish() acts on it later.
+__device__ __forceinline__ uint32_t arrive_issue(uint32_t* sync, uint32_t gen) {
+    return atomicAdd(sync + 32 * (blockIdx.x % BAR_GROUPS) + (gen & 1u), 1u);
+}
+__device__ __forceinline__ void arrive_finish(uint32_t* sync, uint32_t G, uint32_t gen, uint32_t old) {
     const uint32_t g = blockIdx.x % BAR_GROUPS, ng = G < BAR_GROUPS ? G : BAR_GROUPS, mine = (G - g + BAR_GROUPS - 1) / BAR_GROUPS;
     const uint32_t set = gen & 1u;
-    if (atomicAdd(sync + 32 * g + set, 1u) == mine - 1) {
+    if (old == mine - 1) {
         st_agent(sync + 32 * g + set, 0u);
         if (atomicAdd(sync + 32 * BAR_GROUPS + set, 1u) == ng - 1) {
             st_agent(sync + 32 * BAR_GROUPS + set, 0u);
@@ -391,9 +396,10 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     STAMP(1);
     // No grid barrier: what the other workgroups produce here are the logits, and those say themselves when they are there.
     __syncthreads();   // every wave has used its copy of the generation
+    uint32_t arrived = 0;
     if (tid == 0) {
         s_tag = my_gen + 1u;
-        grid_arrive(a.sync, G, my_gen);
+        arrived = arrive_issue(a.sync, my_gen);
     }
     STAMP(2);
 
@@ -496,6 +502,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         route(t);
         route_weights(t);
     }
+    if (tid == 0) arrive_finish(a.sync, G, my_gen, arrived);   // here most workgroups are about to wait for their pair anyway
     STAMP(3);
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
