@@ -247,7 +247,7 @@ void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);   
  * bits as kc_mv(MF_BF16) + kq4_route + kc_mv_gu + kc_mv_sel + kq4_moe_combine(sh = 0), without the four launch gaps.
  * Scratch (caller-owned device memory): logits [T][n_exp], ind / wt [T][top_k] (the routing, also an output), A [T*k][ff],
  * D [T*k][d], sync: kc_moe_decode_sync_words(T, d) uint32 that must be zero before the first call (the kernel keeps them
- * consistent from launch to launch; sync[kc_moe_decode_error_word()] != 0 afterwards reports a grid barrier that gave up,
+ * consistent from launch to launch; sync[kc_moe_decode_error_word()] != 0 afterwards reports a wait between workgroups that gave up,
  * after which the caller must zero sync again).
  * The grid spans the whole device and its workgroups wait for each other: nothing else may run on the GPU beside it.
  * Up to MV_MAXT tokens every (token, expert) pair is a pass of its own (the reference's decode composition, bit for bit);

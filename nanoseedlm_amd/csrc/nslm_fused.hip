@@ -49,28 +49,32 @@ struct FusedArgs {
     int grid;
 };
 
-// Barrier words (uint32; every counter sits alone on a 128-byte line = 32 words):
-//   [32 g], [32 g + 1]   arrivals of group g = blockIdx.x % BAR_GROUPS, for barriers of even / odd generation
+// Words of the sync area (uint32; every counter sits alone on a 128-byte line = 32 words):
+//   [32 g], [32 g + 1]   arrivals of group g = blockIdx.x % BAR_GROUPS, for launches of even / odd generation
 //   [32 BAR_GROUPS], [.. + 1] groups that are complete (even / odd generation)
-//   [32 (BAR_GROUPS+1+g)] group g's sense word: the generation, advanced when the barrier opens
+//   [32 (BAR_GROUPS+1+g)] the generation, the same number in all BAR_GROUPS words: a launch reads it at its start and its
+//                        last arrival writes the next number to every word
 //   [32 (2 BAR_GROUPS+1)] error word
-//   [FUSED_LOGIT_WORDS ..] the per-pair kernel's router logits [MV_MAXT][E], each a 64-bit word: the BF16 value's float
-//                        bits below, the launch's generation + 1 above.  A reader polls until the upper half is its own
-//                        launch's: the logits need no grid barrier.  Every launch rewrites all MV_MAXT rows (rows it does
-//                        not use with zero), so a stale word is always the preceding launch's and never matches.
+//   [FUSED_LOGIT_WORDS ..] the router logits [FG_MAXT][E], each a 64-bit word: the BF16 value's float bits below, the
+//                        launch's generation + 1 above.  A reader polls until the upper half is its own launch's: the
+//                        logits need no grid barrier.  Every launch rewrites all FG_MAXT rows (rows it does not use with
+//                        zero), so a stale word is always the preceding launch's and never matches.
+//   [FUSED_IND_WORDS ..]  the grouped kernel's published selection [FG_MAXT][32], tagged the same way (the weights and the
+//                        row's scale are stored before it)
 //   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile); behind them (at T (d + 1)) three words per pair, each on
 //                        its own line: finished gate+up items (atomics only), the pair's ready flag (what waiters
 //                        poll: polling the counter's line would slow the arrivals), finished down items
 // Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
-// counters and only each group's last arrival touches the shared one; waiters poll their own group's sense word.  The
-// barrier's sense words hold a generation number, the same in all of them (whoever opens a barrier writes the next number to
-// every word), so launches with different numbers of groups and any number of barriers a launch can follow each other;
-// the counters are reset by the last arrival (two sets by generation parity, so that the reset needs no wait): no clean-up
-// between launches.
+// counters and only each group's last arrival touches the shared one.  Earlier versions of these kernels separated their
+// phases by grid barriers on the same words (arrive, then poll the group's generation word): 3.3 us behind the last
+// arrival when the opener read and flipped 32 sense words, 1.2 us with generation numbers, and none now that the data
+// carries the generation itself.  No clean-up between launches: every counter is reset by the launch that used it.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
-#define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // MV_MAXT x 1024 router logits, 64 bits each: value | generation << 32
-#define FUSED_SYNC_WORDS (FUSED_LOGIT_WORDS + 2 * MV_MAXT * 1024)
+#define FG_MAXT 16      // rows of the grouped kernel
+#define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // FG_MAXT x 1024 router logits, 64 bits each: value | generation << 32
+#define FUSED_IND_WORDS (FUSED_LOGIT_WORDS + 2 * FG_MAXT * 1024)   // FG_MAXT x 32 published selections, tagged the same way
+#define FUSED_SYNC_WORDS (FUSED_IND_WORDS + 2 * FG_MAXT * 32)
 #define SPIN_LIMIT (1u << 21)
 
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -83,51 +87,9 @@ __device__ __forceinline__ void st_agent(unsigned long long* p, unsigned long lo
 __device__ __forceinline__ void wg_release() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
 __device__ __forceinline__ void wg_acquire() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
-// The generation the next barrier of this launch starts from (thread 0 keeps it; requested at the start of the kernel so
-// that the load is not on the way of the first barrier's last arrival).
-__device__ __forceinline__ uint32_t barrier_generation(const uint32_t* sync) {
-    return threadIdx.x == 0 ? ld_agent(sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS)) : 0u;
-}
-// every workgroup of the grid arrives and waits (bounded); data written before it by any workgroup is visible after it.
-// gen: the generation before this barrier (barrier_generation() for the first one); advanced on return.
-__device__ __forceinline__ void grid_barrier(uint32_t* sync, uint32_t G, uint32_t& gen) {
-    wg_release();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const uint32_t g = blockIdx.x % BAR_GROUPS, ng = G < BAR_GROUPS ? G : BAR_GROUPS, mine = (G - g + BAR_GROUPS - 1) / BAR_GROUPS;
-        const uint32_t s = gen, set = s & 1u;   // two sets of counters, by generation parity (second word of the same lines)
-        uint32_t* sense = sync + 32 * (BAR_GROUPS + 1 + g);
-        if (atomicAdd(sync + 32 * g + set, 1u) == mine - 1) {
-            // The counters go back to zero without a wait: the next barrier counts in the other set, and nobody can reach
-            // the barrier after that one before this workgroup has arrived at the next, which it does only after its
-            // stores have completed (the release fence at the top).
-            st_agent(sync + 32 * g + set, 0u);
-            if (atomicAdd(sync + 32 * BAR_GROUPS + set, 1u) == ng - 1) {
-                st_agent(sync + 32 * BAR_GROUPS + set, 0u);
-                // All BAR_GROUPS words always hold the same number: whoever opens a barrier writes s + 1 to every one of
-                // them, whatever the number of groups of its launch.  Launches of different grid sizes and any number of
-                // barriers a launch can therefore follow each other, and opening costs no loads.  (Flipping only the words
-                // of the launch's groups left stale values behind a smaller grid; reading all words first cost a round trip.)
-#pragma unroll
-                for (uint32_t i = 0; i < BAR_GROUPS; ++i) st_agent(sync + 32 * (BAR_GROUPS + 1 + i), s + 1u);
-            }
-        }
-        uint32_t spins = 0;
-        while (ld_agent(sense) == s) {
-            __builtin_amdgcn_s_sleep(4);
-            if (++spins > SPIN_LIMIT) {
-                atomicExch(&sync[FUSED_ERR_WORD], 1u);
-                break;
-            }
-        }
-        gen = s + 1u;
-    }
-    __syncthreads();
-    wg_acquire();
-}
-
-// A launch without a grid barrier still moves the generation on: every workgroup arrives (nobody waits), the last arrival
-// writes the next number.  By thread 0, after every wave of the workgroup has read the generation.  In two halves, so
+// The generation moves on once per launch: every workgroup arrives (nobody waits), the last arrival writes the next number
+// to all sense words (two sets of counters, by generation parity: the next launch counts in the other set, so the reset of
+// this launch's set needs no wait).  By thread 0, after every wave of the workgroup has read the generation.  In two halves, so
 // that the atomic's round trip lies under other work: arrive_issue() returns what the group's counter held, and
 // arrive_finish() acts on it later.
 __device__ __forceinline__ uint32_t arrive_issue(uint32_t* sync, uint32_t gen) {
@@ -383,7 +345,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             st_agent(a.logits + item, lv);
             st_agent(lg64 + item, (unsigned long long) __float_as_uint(lv) | (unsigned long long) (my_gen + 1u) << 32);
         }
-        if (t == 0 && lane >= a.T && lane < MV_MAXT) st_agent(lg64 + (size_t) lane * a.E + e, 0ull);   // rows this launch does not use
+        if (t == 0 && lane >= a.T && lane < FG_MAXT) st_agent(lg64 + (size_t) lane * a.E + e, 0ull);   // rows this launch does not use
     }
     // The decode tables are first needed after the barrier: loaded here, behind the logits (the workgroups that form logits
     // are the last to reach the barrier; tables first was one more memory round trip on their way).
@@ -579,7 +541,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 // second grid barrier follows, and every workgroup builds the same table from the published selection: position of a pair
 // among the pairs of its expert in pair order, groups numbered in expert order.  Pair p = (token p / kk, slot p % kk),
 // slots >= k are the always-on experts (expert ids E, E + 1, ...).
-#define FG_MAXT 16
 #define FG_MAXP 512    // pairs a launch: T * kk
 #define FG_RN_WORDS 64   // the rows' RMSNorm scales behind the pairs' words of the sync area
 
@@ -664,7 +625,11 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
     uint32_t* grpc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [group][3][32]: arrivals, ready, done
     float* rnpub = (float*) (grpc + (size_t) a.T * 33 * 96);
-    uint32_t bar_gen = barrier_generation(a.sync);
+    // the generation (all sense words are equal); the workgroup arrives, without waiting, further down
+    const uint32_t my_gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
+    const uint32_t tag = my_gen + 1u;
+    unsigned long long* lg64 = (unsigned long long*) (a.sync + FUSED_LOGIT_WORDS);
+    unsigned long long* ind64 = (unsigned long long*) (a.sync + FUSED_IND_WORDS);
     load_tables(tab);
 
     // ---- phase 1: router logits, one wave per (token, expert) -------------------------------------------------------------
@@ -719,17 +684,46 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             }
         }
         for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-        if (lane == 0) st_agent(a.logits + item, bfr(acc));
+        const float lv = bfr(acc);
+        if (lane == 0) {
+            st_agent(a.logits + item, lv);
+            st_agent(lg64 + item, (unsigned long long) __float_as_uint(lv) | (unsigned long long) tag << 32);
+        }
+        if (t == 0 && lane >= a.T && lane < FG_MAXT) st_agent(lg64 + (size_t) lane * a.E + e, 0ull);   // rows this launch does not use
     }
-    grid_barrier(a.sync, G, bar_gen);
+    // No grid barriers: the logits and the published routing carry the launch's generation and are polled where they are
+    // needed.  The generation moves on with the workgroups' arrivals, which nobody waits for.
+    __syncthreads();   // every wave has its copy of the generation
+    uint32_t arrived = 0;
+    if (tid == 0) arrived = arrive_issue(a.sync, my_gen);
 
     // ---- routing, once per token: workgroup t % G ranks token t and publishes selection, weights and the row's scale ----
     for (int t = (int) blockIdx.x; t < a.T; t += (int) G) {
         __syncthreads();
         const int E4 = (a.E + 3) & ~3;
-        for (int e = tid; e < E4; e += 256) rv[e] = e < a.E ? ld_agent(a.logits + (size_t) t * a.E + e) : __uint_as_float(0xFF800000u);
+        for (int e = tid; e < E4; e += 256) {
+            float v = __uint_as_float(0xFF800000u);
+            if (e < a.E) {   // bounded wait for the logit's wave
+                unsigned long long w = ld_agent(lg64 + (size_t) t * a.E + e);
+                for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(lg64 + (size_t) t * a.E + e)) {
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > SPIN_LIMIT) {
+                        atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                        break;
+                    }
+                }
+                v = __uint_as_float((uint32_t) w);
+            }
+            rv[e] = v;
+        }
         __syncthreads();
         rank_logits(rv, a.E, a.k, (uint32_t*) part, ri_s);
+        __syncthreads();
+        if (a.nw) {
+            const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
+            if (tid == 0) st_agent(rnpub + t, r);
+        }
+        wg_release();   // the scale is stored before the selection that announces it
         __syncthreads();
         if (wv == 0) {
             if (lane < a.k) rw_s[lane] = expf(rv[ri_s[lane]] - rv[ri_s[0]]);
@@ -739,21 +733,32 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
                 st_agent((uint32_t*) a.ind + (size_t) t * a.k + lane, (uint32_t) ri_s[lane]);
                 st_agent(a.wt + (size_t) t * a.k + lane, rw_s[lane] / top);
             }
-        }
-        if (a.nw) {
-            const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
-            if (tid == 0) st_agent(rnpub + t, r);
+            wg_release();   // weights before the tagged selection
+            if (lane < a.k) st_agent(ind64 + (size_t) t * 32 + lane, (unsigned long long) (uint32_t) ri_s[lane] | (unsigned long long) tag << 32);
         }
     }
-    grid_barrier(a.sync, G, bar_gen);
 
     // ---- the groups: the same table in every workgroup ----------------------------------------------------------------------
     for (int i = tid; i < NE; i += 256) cnt_s[i] = 0;
     for (int p = tid; p < P_ + 8; p += 256) {
         const int pc = min(p, P_ - 1), t = pc / a.kk, j = pc - t * a.kk;
-        const int e = j < a.k ? (int) ld_agent((const uint32_t*) a.ind + (size_t) t * a.k + j) : a.E + (j - a.k);
+        int e = a.E + (j - a.k);
+        if (j < a.k) {   // bounded wait for the token's routing
+            unsigned long long w = ld_agent(ind64 + (size_t) t * 32 + j);
+            for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(ind64 + (size_t) t * 32 + j)) {
+                __builtin_amdgcn_s_sleep(2);
+                if (++spins > SPIN_LIMIT) {
+                    atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                    w = 0;   // expert 0: the results are void, the indices stay in range
+                    break;
+                }
+            }
+            e = (int) (uint32_t) w;
+        }
         if (p < FG_MAXP + 8) pe[p] = (uint16_t) (p < P_ ? e : 0xFFFF);   // the table is read eight at a time: pad with "no expert"
     }
+    __syncthreads();
+    wg_acquire();   // the selections have been seen: the scales and weights stored before them are there
     if (a.nw && tid < a.T) rn_s[tid] = ld_agent(rnpub + tid);
     __syncthreads();
     for (int p = tid; p < P_; p += 256) {   // position among the pairs of the same expert (in pair order), and their number
@@ -836,6 +841,8 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         __syncthreads();
         if (tid == 0 && atomicAdd(&grpc[g * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&grpc[g * 96 + 32], 1u);
     }
+
+    if (tid == 0) arrive_finish(a.sync, G, my_gen, arrived);
 
     // ---- down, then the last workgroup of a (token, row tile) sums the token's experts ------------------------------------
     for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {
