@@ -61,9 +61,16 @@ struct FusedArgs {
 //                        zero), so a stale word is always the preceding launch's and never matches.
 //   [FUSED_IND_WORDS ..]  the grouped kernel's published selection [FG_MAXT][32], tagged the same way (the weights and the
 //                        row's scale are stored before it)
-//   [FUSED_SYNC_WORDS ..] one ticket per (token, down row tile); behind them (at T (d + 1)) three words per pair, each on
-//                        its own line: finished gate+up items (atomics only), the pair's ready flag (what waiters
-//                        poll: polling the counter's line would slow the arrivals), finished down items
+//   [FUSED_PAIR_WORDS ..] the per-pair kernel's two words per pair, each on its own line: finished gate+up items (atomics
+//                        only; the last arrival puts it back to zero) and the pair's ready word, set to the launch's
+//                        generation + 1 by that last arrival (what the pair's down items poll: polling the counter's
+//                        line would slow the arrivals, and a word per item - 96 polls a workgroup - was slower too)
+//   [FUSED_DFLAG_WORDS ..] a word per down item, set to the generation + 1 when its rows are stored; the down item of a
+//                        token's last expert polls the words of the other experts' items of its row tile and sums (a
+//                        ticket per (token, row tile) cost an atomic's round trip more before the sum)
+//   [FUSED_SYNC_WORDS ..] the grouped kernel's words: one ticket per (token, down row tile); behind them (at T (d + 1))
+//                        three words per group, each on its own line: finished gate+up items (atomics only), the group's
+//                        ready flag (what waiters poll), finished down items; then the rows' scales
 // Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
 // counters and only each group's last arrival touches the shared one.  Earlier versions of these kernels separated their
 // phases by grid barriers on the same words (arrive, then poll the group's generation word): 3.3 us behind the last
@@ -74,7 +81,10 @@ struct FusedArgs {
 #define FG_MAXT 16      // rows of the grouped kernel
 #define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // FG_MAXT x 1024 router logits, 64 bits each: value | generation << 32
 #define FUSED_IND_WORDS (FUSED_LOGIT_WORDS + 2 * FG_MAXT * 1024)   // FG_MAXT x 32 published selections, tagged the same way
-#define FUSED_SYNC_WORDS (FUSED_IND_WORDS + 2 * FG_MAXT * 32)
+#define FUSED_TILES 256   // most items a pair in a pass of the per-pair kernel
+#define FUSED_PAIR_WORDS (FUSED_IND_WORDS + 2 * FG_MAXT * 32)        // per-pair kernel: [MV_MAXT * 33 pairs][64]: arrivals, ready word
+#define FUSED_DFLAG_WORDS (FUSED_PAIR_WORDS + MV_MAXT * 33 * 64)     // per-pair kernel: [MV_MAXT][FUSED_TILES][33] finished down items
+#define FUSED_SYNC_WORDS (FUSED_DFLAG_WORDS + MV_MAXT * FUSED_TILES * 33)
 #define SPIN_LIMIT (1u << 21)
 
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -265,7 +275,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     __shared__ float rw_s[33];      // route: weight by rank (+ the shared expert's 1)
     __shared__ int ri_s[33];        // route: expert by rank
     __shared__ WSlice sl_s[3][33];  // route: the chosen experts' gate / up / down slices (+ the shared expert's)
-    __shared__ int s_flag;
+    // (no workgroup-wide flag: every wait of this kernel is a poll of its own threads)
     __shared__ uint32_t s_tag;
     __shared__ float rn_s[MV_MAXT], nred[4];   // the rows' RMSNorm scales when the kernel normalises its input
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -287,7 +297,8 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     unsigned long long* lg64 = (unsigned long long*) (a.sync + FUSED_LOGIT_WORDS);
     const int items_g = P_ * a.ntile_g, items_d = P_ * a.ntile_d;
     int staged = -1;
-    uint32_t* pairc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [pair][3][32]: arrivals, ready, done
+    uint32_t* pairw = a.sync + FUSED_PAIR_WORDS;    // [pair][64]: arrivals, ready word
+    uint32_t* dflag = a.sync + FUSED_DFLAG_WORDS;   // [token][FUSED_TILES][33]
     if (a.nw) {   // uniform: every workgroup forms every row's scale (T rows of d values from L2)
         for (int t = 0; t < a.T; ++t) {
             const float r = row_rnorm(a.x + (size_t) t * a.xs, a.d, a.neps, nred);
@@ -457,7 +468,10 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         if (item == (int) blockIdx.x) DSTAMP(10);
         wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
         __syncthreads();
-        if (tid == 0 && atomicAdd(&pairc[p * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&pairc[p * 96 + 32], 1u);   // the pair's A is complete
+        if (tid == 0 && atomicAdd(&pairw[p * 64], 1u) == (uint32_t) (a.ntile_g - 1)) {
+            st_agent(&pairw[p * 64], 0u);
+            st_agent(&pairw[p * 64 + 32], s_tag);   // the pair's A is complete
+        }
     }
     // tokens whose routing nobody needed here still get published by their designated workgroup
     for (int t = (int) blockIdx.x; t < a.T; t += (int) G) {
@@ -469,7 +483,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
     // the first down item's records do not depend on phase 2: they are fetched before the barrier
-    uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
     Chunk d0;
     if ((int) blockIdx.x < items_d) {
         const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
@@ -485,9 +498,10 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         const int v0 = tile * a.it_d / a.ntile_d * a.rpid, v1 = min((tile + 1) * a.it_d / a.ntile_d * a.rpid, a.d);
         if (item != (int) blockIdx.x) d0 = first_chunk<P, false>(sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1);
         route_weights(t);
-        if (tid == 0) {
+        if (tid == 0) {   // the pair's A is complete when its last gate+up item has said so (bounded wait)
+            const uint32_t tag = s_tag;
             uint32_t spins = 0;
-            while (ld_agent(&pairc[p * 96 + 32]) == 0u) {
+            while (ld_agent(&pairw[p * 64 + 32]) != tag) {
                 __builtin_amdgcn_s_sleep(2);
                 if (++spins > SPIN_LIMIT) {
                     atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
@@ -508,23 +522,28 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         if (item == (int) blockIdx.x) DSTAMP(17);
         wg_release();
         __syncthreads();
-        if (tid == 0) s_flag = atomicAdd(&tick[t * a.ntile_d + tile], 1u) == (uint32_t) (a.kk - 1);
-        __syncthreads();
-        if (item == (int) blockIdx.x) DSTAMP(18);
-        if (s_flag) {   // all k experts' rows of this tile are written: out = 0.5 * 0 + sum_j wt_j D_j, in j order
+        if (j != a.kk - 1) {
+            if (tid == 0) st_agent(&dflag[((size_t) t * FUSED_TILES + tile) * 33 + j], s_tag);
+        } else {   // the token's last expert sums: out = 0.5 * 0 + sum_j wt_j D_j, in j order, once the others' rows are there
+            if (tid < a.kk - 1) {
+                const uint32_t tag = s_tag;
+                uint32_t spins = 0;
+                while (ld_agent(&dflag[((size_t) t * FUSED_TILES + tile) * 33 + tid]) != tag) {
+                    __builtin_amdgcn_s_sleep(2);
+                    if (++spins > SPIN_LIMIT) {
+                        atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                        break;
+                    }
+                }
+            }
+            __syncthreads();
             wg_acquire();
+            if (item == (int) blockIdx.x) DSTAMP(18);
             for (int r = v0 + tid; r < v1; r += 256) {
                 float acc = 0.0f;
                 for (int jj = 0; jj < a.kk; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.kk + jj) * a.d + r), acc);
                 a.out[(size_t) t * a.os + r] = a.res ? bfr(a.res[(size_t) t * a.os + r] + bfr(acc)) : acc;
             }
-            if (tid == 0) st_agent(&tick[t * a.ntile_d + tile], 0u);
-        }
-        // the pair's last down item leaves its three words at zero for the next launch (everyone has read them by then)
-        if (tid == 0 && atomicAdd(&pairc[p * 96 + 64], 1u) == (uint32_t) (a.ntile_d - 1)) {
-            st_agent(&pairc[p * 96], 0u);
-            st_agent(&pairc[p * 96 + 32], 0u);
-            st_agent(&pairc[p * 96 + 64], 0u);
         }
     }
     STAMP(5);
@@ -948,7 +967,7 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     auto pick = [&](int iters) {
         int best = 1;
         long best_cost = -1;
-        for (int n = 1; n <= iters; ++n) {
+        for (int n = 1; n <= iters && n <= FUSED_TILES; ++n) {
             const long rounds = ((long) P_ * n + gmax - 1) / gmax, per = (iters + n - 1) / n;
             const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
             if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }   // ties: more, shorter items
