@@ -3,8 +3,8 @@
 // weighted combine.  No counterpart in the reference, which launches
 // these as five kernels (engine/qwen4_cuda.c:1023-1083); on MI355X each launch and each dependent global read costs
 // microseconds that a ~20 us step cannot afford, so the phases run inside one grid: the data that crosses workgroups says
-// itself when it is there (generation-tagged router logits, one ready flag per pair), and the kernel for 9 to 16 tokens
-// adds two grid-wide barriers.
+// itself when it is there (router logits, published routing, ready words and finished-item words, all tagged with the
+// launch's generation), so no phase needs a grid-wide barrier.
 //
 // Arithmetic is the stand-alone kernels', instruction for instruction (k_mv_any's BF16 row dot, k_q4_route's selection
 // and weights, k_mv_seed's chunk products and row-sum order, k_q4_moe_combine's sum), so the fused step returns the same
@@ -13,13 +13,12 @@
 // Data that one workgroup writes and another reads inside the launch (logits, A, D) moves with agent-scope relaxed
 // atomic stores and loads: on this GPU every XCD has its own L2, and those accesses go through to the coherent level, so
 // no device-scope fence (an L2 write-back / invalidate per workgroup, which costs far more than the step) is needed;
-// ordering against the barrier counters is a workgroup-scope release / acquire, i.e. a wait for outstanding memory
-// operations.
+// ordering against the counters and tagged words is a workgroup-scope release / acquire, i.e. a wait for outstanding
+// memory operations.
 //
 // Waiting: the grid is sized to the number of workgroups the device can hold at once (occupancy query), because
-// workgroups wait for each other's data (and, in the grouped kernel, for each other at its barriers: every workgroup
-// arrives on a counter in caller-provided scratch and spins until all have); every wait is bounded, and a workgroup that
-// gives up sets an error word and runs on to the end, so every wave always exits.
+// workgroups wait for each other's data; every wait is a bounded poll, and a workgroup that gives up sets an error word
+// and runs on to the end, so every wave always exits.
 #include <math.h>
 #include <stdlib.h>
 
@@ -119,7 +118,7 @@ __device__ __forceinline__ void arrive_finish(uint32_t* sync, uint32_t G, uint32
 }
 
 // The first chunk of a pass over rows [v0, v1): issued as early as the slices are known, so its latency hides behind
-// whatever comes before the pass (a grid barrier, the staging of the activations).
+// whatever comes before the pass (a wait for other workgroups, the staging of the activations).
 template <int P, bool GATEUP>
 __device__ __forceinline__ Chunk first_chunk(const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1) {
     const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L, vv = v0 + lr;
@@ -358,8 +357,8 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         }
         if (t == 0 && lane >= a.T && lane < FG_MAXT) st_agent(lg64 + (size_t) lane * a.E + e, 0ull);   // rows this launch does not use
     }
-    // The decode tables are first needed after the barrier: loaded here, behind the logits (the workgroups that form logits
-    // are the last to reach the barrier; tables first was one more memory round trip on their way).
+    // The decode tables are first needed in phase 2: loaded here, behind the logits (everybody waits for the workgroups
+    // that form logits; tables first was one more memory round trip on their way).
     load_tables(tab);
     // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
     if ((int) blockIdx.x < items_g) {
@@ -376,7 +375,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     }
     STAMP(2);
 
-    // ---- route: every workgroup ranks the logits of the token it needs (cheap, and saves a grid barrier) ----------------
+    // ---- route: every workgroup ranks the logits of the token it needs itself (cheap, and nobody waits for a router) ----
     // rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order
     int routed = -1;
     bool weighted = true;
@@ -482,7 +481,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     STAMP(3);
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
-    // the first down item's records do not depend on phase 2: they are fetched before the barrier
+    // the first down item's records do not depend on phase 2: they are requested before the wait for the pair
     Chunk d0;
     if ((int) blockIdx.x < items_d) {
         const int p = (int) blockIdx.x / a.ntile_d, tile = (int) blockIdx.x - p * a.ntile_d, t = p / a.kk, j = p - t * a.kk;
@@ -557,7 +556,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 // (group, row tile); a thread decodes its chunk once and multiplies it with the NT rows of activations staged side by side
 // in LDS (chunk_dot<P, NT>: per token the same chain of operations as the one-token kernel, hence the same bits).  The
 // groups must be the same in every workgroup, so the routing is done once (workgroup t routes token t) and published, a
-// second grid barrier follows, and every workgroup builds the same table from the published selection: position of a pair
+// every workgroup polls the published selection (tagged with the generation) and builds the same table from it: position of a pair
 // among the pairs of its expert in pair order, groups numbered in expert order.  Pair p = (token p / kk, slot p % kk),
 // slots >= k are the always-on experts (expert ids E, E + 1, ...).
 #define FG_MAXP 512    // pairs a launch: T * kk
@@ -956,7 +955,7 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
         per_cu = 0;
         return -1;
     }
-    // The grid must be resident at once (the kernel has a grid barrier): at most what the device holds, and no more than
+    // The grid must be resident at once (workgroups wait for each other's data): at most what the device holds, and no more than
     // five workgroups a CU (the most that was tried).  Items per pair (an item = a run of a pair's iterations, as
     // equal as whole iterations allow): the count that gives the busiest workgroup the least to do, an item's set-up priced
     // at a third of an iteration and unequal items at half an iteration (workgroups i, i + 256, ... share a CU, so the long
