@@ -555,9 +555,9 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 // a block (nine tenths of the work) can serve them all.  Pairs are grouped by expert in runs of at most NT; an item is a
 // (group, row tile); a thread decodes its chunk once and multiplies it with the NT rows of activations staged side by side
 // in LDS (chunk_dot<P, NT>: per token the same chain of operations as the one-token kernel, hence the same bits).  The
-// groups must be the same in every workgroup, so the routing is done once (workgroup t routes token t) and published, a
-// every workgroup polls the published selection (tagged with the generation) and builds the same table from it: position of a pair
-// among the pairs of its expert in pair order, groups numbered in expert order.  Pair p = (token p / kk, slot p % kk),
+// groups must be the same in every workgroup, so the routing is done once (workgroup t routes token t) and published;
+// every workgroup polls the published selection (tagged with the generation) and builds the same table from it: position
+// of a pair among the pairs of its expert in pair order, groups numbered in expert order.  Pair p = (token p / kk, slot p % kk),
 // slots >= k are the always-on experts (expert ids E, E + 1, ...).
 #define FG_MAXP 512    // pairs a launch: T * kk
 #define FG_RN_WORDS 64   // the rows' RMSNorm scales behind the pairs' words of the sync area
