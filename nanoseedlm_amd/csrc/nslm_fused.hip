@@ -78,6 +78,7 @@ struct FusedArgs {
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
 #define FG_MAXT 16      // rows of the grouped kernel
+#define FG_MINT_SHARED 6   // with an always-on expert (every row a pair on the same expert) it also takes 6 to 8 rows
 #define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // FG_MAXT x 1024 router logits, 64 bits each: value | generation << 32
 #define FUSED_IND_WORDS (FUSED_LOGIT_WORDS + 2 * FG_MAXT * 1024)   // FG_MAXT x 32 published selections, tagged the same way
 #define FUSED_TILES 256   // most items a pair in a pass of the per-pair kernel
@@ -940,6 +941,36 @@ bool shape_of(int K, bool gateup, int* L, int* rpi, bool* shfl) {
     return true;
 }
 
+// Items per pair (or group) of a phase of `iters` iterations, `units` pairs, at most gmax workgroups.
+// one_round: the count that gives the busiest workgroup the least to do when every workgroup takes its items one after the
+// other (an item's set-up priced at a third of an iteration, unequal items at half an iteration: workgroups i, i + 256, ...
+// share a CU, so the long items of a regular pattern meet on the same CUs); up to `slack` items more than the workgroups still
+// count as one round.
+int pick_one_round(int units, int iters, int gmax, int nmax, int slack = 0) {
+    int best = 1;
+    long best_cost = -1;
+    for (int n = 1; n <= iters && n <= nmax; ++n) {
+        const long over = (long) units * n - slack, rounds = over <= gmax ? 1 : (over + gmax - 1) / gmax, per = (iters + n - 1) / n;
+        const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
+        if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }   // ties: more, shorter items
+    }
+    return best;
+}
+// by_cu_load: the count that gives the busiest CU the least to do (items go round the workgroups, the workgroups round the
+// CUs, and a CU's waves share its issue slots, so a CU is as late as the sum of its items, plus one item for the end of
+// the phase, when the CU is no longer full), with fewer than five workgroups a CU priced for the latencies they no longer hide.
+int pick_by_cu_load(int units, int iters, int cus, int nmax) {
+    static const int thin[6] = {200, 160, 130, 115, 103, 100};
+    int best = 1;
+    long best_cost = -1;
+    for (int n = 1; n <= iters && n <= nmax; ++n) {
+        const long items = (long) units * n, per = (iters + n - 1) / n, on_cu = (items + cus - 1) / cus;
+        const long cost = (on_cu * (6 * per + (iters % n ? 3 : 0) + 2) + 2 * per) * thin[items / cus < 5 ? items / cus : 5];
+        if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }
+    }
+    return best;
+}
+
 template <int P>
 int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // One token is at most a few hundred items more than three workgroups a CU hold (C2: 784): that launch may use the
@@ -957,24 +988,16 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     }
     // The grid must be resident at once (workgroups wait for each other's data): at most what the device holds, and no more than
     // five workgroups a CU (the most that was tried).  Items per pair (an item = a run of a pair's iterations, as
-    // equal as whole iterations allow): the count that gives the busiest workgroup the least to do, an item's set-up priced
-    // at a third of an iteration and unequal items at half an iteration (workgroups i, i + 256, ... share a CU, so the long
-    // items of a regular pattern meet on the same CUs).  Measured on C2: one token, 96 x 2 gate+up iterations and 98 x 1 down
-    // iterations a pair on 784 workgroups, 40.1 us (96 unequal down items on 768 workgroups: 42.9); 8 tokens, 20 items a
-    // pair on 1280 workgroups, 139.6 us (768 workgroups, 24 and 13 items of 8 iterations: 163.7).
+    // equal as whole iterations allow).  Down items, and every item of one token: one round (measured on C2, one token: 96 x 2
+    // gate+up iterations and 98 x 1 down iterations a pair on 784 workgroups, 40.1 us; 96 unequal down items on 768
+    // workgroups: 42.9; 8 tokens with 32 instead of 20 down items a pair: 144 against 131 us - a down item waits for its
+    // pair, and a second round of them waits behind the first).  Gate+up items of several tokens: by the CUs' load, which
+    // takes more, shorter items than one round holds (C2, items a pair -> us; 4 tokens: 24 -> 82.2, 40 -> 79.6, 64 -> 78.0;
+    // 6 tokens: 24 -> 120.2, 32 -> 111.4, 48 -> 115.2; 8 tokens: 20 -> 135.4, 32 -> 131.2, 48 -> 138.9); where the row sums go
+    // through LDS (C3) one round stayed ahead.
     const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
-    auto pick = [&](int iters) {
-        int best = 1;
-        long best_cost = -1;
-        for (int n = 1; n <= iters && n <= FUSED_TILES; ++n) {
-            const long rounds = ((long) P_ * n + gmax - 1) / gmax, per = (iters + n - 1) / n;
-            const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
-            if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }   // ties: more, shorter items
-        }
-        return best;
-    };
-    a.ntile_g = pick(a.it_g);
-    a.ntile_d = pick(a.it_d);
+    a.ntile_g = few || !sg ? pick_one_round(P_, a.it_g, gmax, FUSED_TILES) : pick_by_cu_load(P_, a.it_g, cu_count(), FUSED_TILES);
+    a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES);
     const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     int grid = items < gmax ? (int) items : gmax;
     if (grid < 1) grid = 1;
@@ -1003,23 +1026,16 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
         cached_lds[sg][sd] = lds;
     }
     // The groups are formed on the device; the host sizes the items for the number it expects from a uniform routing:
-    // the experts that receive a pair at all, plus the always-on experts' runs of NT tokens.
+    // the experts that receive a pair at all, plus the always-on experts' runs of NT tokens.  Four workgroups a CU are
+    // resident, and items for about five were fastest (C2, 16 rows, 81 groups on 1024 workgroups, gate+up items a group
+    // -> us: 12 -> 228, 14 -> 223, 16 -> 212, 18 -> 216, 20 -> 230; down items: 10 -> 207, 14 -> 202, 24 -> 208, 49 -> 214):
+    // one round that may run over by three eighths.
     const double pairs = (double) a.T * a.k;
     int groups = (int) (a.E * (1.0 - pow(1.0 - 1.0 / a.E, pairs)) + 0.5) + a.ns * ((a.T + NT - 1) / NT);
     if (groups < 1) groups = 1;
     const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count();
-    auto pick = [&](int iters) {
-        int best = 1;
-        long best_cost = -1;
-        for (int n = 1; n <= iters; ++n) {
-            const long rounds = ((long) groups * n + gmax - 1) / gmax, per = (iters + n - 1) / n;
-            const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
-            if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }
-        }
-        return best;
-    };
-    a.ntile_g = pick(a.it_g);
-    a.ntile_d = pick(a.it_d);
+    a.ntile_g = pick_one_round(groups, a.it_g, gmax, a.it_g, 3 * gmax / 8);
+    a.ntile_d = pick_one_round(groups, a.it_d, gmax, a.it_d, 3 * gmax / 8);
     const long items = (long) groups * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     int grid = items < gmax ? (int) items : gmax;
     if (grid < a.T) grid = a.T < gmax ? a.T : gmax;
@@ -1061,11 +1077,13 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     for (int i = 0; i < 3 && shared; ++i) a.sh[i] = shared[i];
     a.it_g = (2 * ff + a.rpig - 1) / a.rpig;
     a.it_d = (d + a.rpid - 1) / a.rpid;
-    if (T > MV_MAXT) {
+    if (T > MV_MAXT || (shared && T >= FG_MINT_SHARED && sg && T * a.kk <= FG_MAXP)) {
         // More rows than the per-pair kernel takes: pairs grouped by expert, two to a decode.  Measured against the grouped
-        // GEMMs of the separate launches (C2, 16 rows: 236 against 268 us); with four to a decode (17 to 32 rows: 402 against
+        // GEMMs of the separate launches (C2, 16 rows: 199 against 268 us); with four to a decode (17 to 32 rows: 402 against
         // 338 us at 32) and where the gate+up row sums go through LDS (C3's 45 chunks a row: 1129 against 753 us) the GEMMs
-        // win, so those shapes are left to them.
+        // win, so those shapes are left to them.  With an always-on expert every row brings a pair on the same expert, and
+        // the grouped kernel is already ahead of the per-pair one at 6 rows (whole model, 8 rows: 5.37 against 5.70 ms); without
+        // one the two are level at 8 rows (130 us) and the per-pair kernel is ahead below.
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
