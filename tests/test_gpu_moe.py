@@ -208,6 +208,41 @@ def test_fused_step_equal_logits(oracle, case, E):
 
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("d,ff", [(2880, 2880), (2816, 2880), (4480, 5760)])
+def test_fused_step_rows_that_do_not_fill_a_workgroup(d, ff, fmt):
+    """Rows of 44, 45, 70 or 90 chunks (hidden 2880 = the mixed-format configuration): whole rows do not fill a workgroup's
+    256 threads, the row sums go through LDS in both passes, and 2816 rows are 563.2 iterations of 5, so the last item
+    ends inside an iteration.  Same bits as the separate launches, at 1, 3 and 8 rows."""
+    from nanoseedlm_amd import moe
+    rng = np.random.default_rng(d + ff + fmt)
+    E, k = 6, 2
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=8)
+    gate, up, down = mk(rng, E, ff, d, eb=-23), mk(rng, E, ff, d, eb=-23), mk(rng, E, d, ff, eb=-22)
+    st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+    st.finalize()
+    for T in (1, 3, 8):
+        xn = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
+        dx = moe.DevBuf.from_array(xn)
+        outs = []
+        for fused in (1, 0):
+            st.set_fused(fused)
+            dio = moe.DevBuf.from_array(np.zeros((T, d), dtype=np.float32))
+            st.step(None, 0, dx.ptr, T, dio.ptr)
+            outs.append((st.last_routing(T), dio.to_array(np.float32, (T, d))))
+            dio.free()
+            assert st.fused_error() == 0
+        dx.free()
+        (i1, w1), o1 = outs[0]
+        (i0, w0), o0 = outs[1]
+        assert np.abs(o0).max() > 0
+        assert np.array_equal(i1, i0) and np.array_equal(w1.view(np.uint32), w0.view(np.uint32))
+        bad = np.argwhere(o1.view(np.uint32) != o0.view(np.uint32))
+        assert len(bad) == 0, (T, len(bad), bad[:6].tolist())
+    st.close()
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
 @pytest.mark.parametrize("E,k", [(16, 4), (64, 4), (200, 8), (300, 6)])
 @pytest.mark.parametrize("T", [9, 13, 16])
 def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
