@@ -139,6 +139,9 @@ void kq4_route(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int32_t* i
 void kq4_route_ld(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int ld, int32_t* ind, float* wt, int T);
 /* engine/kernels_cuda.h:124-125, engine/kernels_moe.cu:2408-2413 */
 void kc_swiglu(kc_stream_t s, const float* g, const float* u, float* a, int n);
+/* kc_swiglu + kc_pack_input_bf16 in one pass (no counterpart in the reference): y = the BF16 bits of kc_swiglu's values,
+ * n % 8 == 0, g / u / y 16-byte aligned, y distinct from g and u */
+void kc_swiglu_pack(kc_stream_t s, const float* g, const float* u, uint16_t* y, size_t n);
 void kc_moe_combine(kc_stream_t s, const float* D, const float* w, const float* shared, float* x, int d, int k, int T);
 /* engine/kernels_qwen4.h:71, engine/kernels_qwen4.cu:514-516 */
 void kq4_moe_combine(kc_stream_t s, int d, int k, const float* D, const float* wt, const float* sh, const float* sg,

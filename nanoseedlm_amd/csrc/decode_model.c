@@ -378,8 +378,11 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
                 dense(m, s, &dn[NSLM_W_SG], m->xn, m->px, d, m->gs, T, 0);
                 dense(m, s, &dn[NSLM_W_SU], m->xn, m->px, d, m->us, T, 0);
             }
-            kc_swiglu(s, m->gs, m->us, m->as, T * ffs);
-            if (bigd) kc_pack_input_bf16(s, m->as, m->pa, (size_t) T * ffs);
+            if (bigd && ffs % 8 == 0) kc_swiglu_pack(s, m->gs, m->us, m->pa, (size_t) T * ffs);   /* the GEMM reads the BF16 view only */
+            else {
+                kc_swiglu(s, m->gs, m->us, m->as, T * ffs);
+                if (bigd) kc_pack_input_bf16(s, m->as, m->pa, (size_t) T * ffs);
+            }
             dense(m, s, &dn[NSLM_W_SD], m->as, m->pa, ffs, m->sh, T, 0);
         }
         kc_residual_add(s, m->x, m->mo, m->sh, (size_t) T * d);

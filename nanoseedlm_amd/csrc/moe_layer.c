@@ -275,16 +275,15 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         kc_mv_sel(s, c->fmt, down, ff, d, m->A, ff, m->D, d, m->ind, P, 1, NULL);
     } else {              /* batched: pairs grouped by expert, three grouped GEMMs (engine/mova_cuda.c:1308-1317) */
         /* BF16 views of the activations feed the MFMA path, as the reference's packed_layer() case does
-           (engine/mova_cuda.c:1012-1035,1229,1308-1317): SwiGLU has consumed G, so G's storage holds A's view */
+           (engine/mova_cuda.c:1012-1035,1229,1308-1317): SwiGLU writes A as that view directly */
         const int packed = d % 8 == 0 && ff % 8 == 0;
         kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
         if (packed) {
             if (c->router != NSLM_ROUTE_SOFTMAX) kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);   /* else: made for the router */
             kc_mm_grouped_packed(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
             kc_mm_grouped_packed(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
-            kc_swiglu(s, m->G, m->U, m->A, P * ff);
-            kc_pack_input_bf16(s, m->A, (uint16_t*) m->G, (size_t) P * ff);
-            kc_mm_grouped_packed(s, c->fmt, down, ff, d, (const uint16_t*) m->G, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
+            kc_swiglu_pack(s, m->G, m->U, (uint16_t*) m->A, (size_t) P * ff);
+            kc_mm_grouped_packed(s, c->fmt, down, ff, d, (const uint16_t*) m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
                                  m->max_tiles, NULL);
         } else {
             kc_mm_grouped_dev(s, c->fmt, gate, d, ff, xn, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);

@@ -127,6 +127,18 @@ __global__ void k_swiglu(const float* g, const float* u, float* a, int n) {
     const int i = (int) (blockIdx.x * blockDim.x + threadIdx.x);
     if (i < n) a[i] = bfr(silu_bf(g[i]) * u[i]);
 }
+// the same values as BF16 bits (they are BF16 values already), eight a thread: k_swiglu + k_pack_input_bf16 in one pass for
+// the GEMMs that take a BF16 view of their activations
+__global__ void k_swiglu_pack(const float* g, const float* u, uint16_t* y, size_t n) {
+    const size_t b = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= n / 8) return;
+    const float4 g0 = ((const float4*) g)[2 * b], g1 = ((const float4*) g)[2 * b + 1];
+    const float4 u0 = ((const float4*) u)[2 * b], u1 = ((const float4*) u)[2 * b + 1];
+    ((uint4*) y)[b] = make_uint4(pack_bf2(bfr(silu_bf(g0.x) * u0.x), bfr(silu_bf(g0.y) * u0.y)),
+                                 pack_bf2(bfr(silu_bf(g0.z) * u0.z), bfr(silu_bf(g0.w) * u0.w)),
+                                 pack_bf2(bfr(silu_bf(g1.x) * u1.x), bfr(silu_bf(g1.y) * u1.y)),
+                                 pack_bf2(bfr(silu_bf(g1.z) * u1.z), bfr(silu_bf(g1.w) * u1.w)));
+}
 // x[t][c] = bf16(x + bf16(bf16(sum_j bf16(D[t,j][c] * bf16(w[t,j]))) + shared[t][c]))
 __global__ void k_moe_combine(const float* D, const float* w, const float* shared, float* x, int d, int k) {
     const int c = (int) (blockIdx.x * blockDim.x + threadIdx.x), t = (int) blockIdx.y;
@@ -362,6 +374,10 @@ void kq4_route(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int32_t* i
 void kc_swiglu(kc_stream_t s, const float* g, const float* u, float* a, int n) {
     if (n < 1) return;
     hipLaunchKernelGGL(k_swiglu, dim3((unsigned) (n + 255) / 256), dim3(256), 0, (hipStream_t) s, g, u, a, n);
+}
+void kc_swiglu_pack(kc_stream_t s, const float* g, const float* u, uint16_t* y, size_t n) {
+    if (n < 8) return;
+    hipLaunchKernelGGL(k_swiglu_pack, dim3((unsigned) ((n / 8 + 255) / 256)), dim3(256), 0, (hipStream_t) s, g, u, y, n);
 }
 void kc_moe_combine(kc_stream_t s, const float* D, const float* w, const float* shared, float* x, int d, int k, int T) {
     if (T < 1) return;

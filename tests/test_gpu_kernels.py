@@ -325,6 +325,29 @@ def test_routers(be, oracle):
     assert np.array_equal(ind, oi) and np.allclose(wt, ow, rtol=1e-5)
 
 
+def test_swiglu_pack_equals_swiglu_then_pack():
+    """kc_swiglu_pack writes the BF16 bits of exactly the values kc_swiglu stores (which are BF16 values already)."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(99)
+    n = 8 * 777
+    g = packs.round_bf16(rng.standard_normal(n).astype(np.float32) * 3)
+    u = packs.round_bf16(rng.standard_normal(n).astype(np.float32))
+    dg, du, da, dp = moe.DevBuf.from_array(g), moe.DevBuf.from_array(u), moe.DevBuf(4 * n), moe.DevBuf(2 * n)
+    L.kc_swiglu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+    L.kc_swiglu_pack.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    L.kc_swiglu(None, dg.ptr, du.ptr, da.ptr, n)
+    L.kc_swiglu_pack(None, dg.ptr, du.ptr, dp.ptr, n)
+    moe.device_sync()
+    a, p = da.to_array(np.float32, (n,)), dp.to_array(np.uint16, (n,))
+    for b in (dg, du, da, dp):
+        b.free()
+    assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32) & 0xFFFF, np.zeros(n, dtype=np.uint32))
+    assert np.array_equal((a.view(np.uint32) >> 16).astype(np.uint16), p)
+
+
 def test_swiglu_and_combines(be, oracle):
     rng = np.random.default_rng(12)
     r = packs.round_bf16
