@@ -208,12 +208,12 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part)
         ind.free(); A.free()
     else:
-        # Batched steps: 9 to 16 rows of C2 are one launch of the grouped persistent kernel; beyond that (and for C3) three
+        # Batched steps: 9 to 24 rows of C2 are one launch of the grouped persistent kernel; beyond that (and for C3) three
         # grouped GEMM launches over tiles of a few pairs each dominate, and what they spend is the records' expansion, not
         # matrix flops: priced against HBM on the records the step has to read.
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
                                frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=None,
-                               kernel=("k_moe_decode_grouped (one launch per step)" if T <= 16 and name[:2] == "c2" else
+                               kernel=("k_moe_decode_grouped (one launch per step)" if T <= 24 and name[:2] == "c2" else
                                        "k_mm_stream<1, 4, 3> grouped (three launches of the step, with its glue kernels)"),
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
     desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",

@@ -1,4 +1,4 @@
-// nslm_fused.hip - one persistent kernel for a whole routed-expert decode step at T <= 8 tokens (k_moe_decode; 9 to 16
+// nslm_fused.hip - one persistent kernel for a whole routed-expert decode step at T <= 8 tokens (k_moe_decode; 9 to 24
 // tokens: k_moe_decode_grouped further down): router logits, softmax top-k, fused gate + up + SwiGLU gather, down gather,
 // weighted combine.  No counterpart in the reference, which launches
 // these as five kernels (engine/qwen4_cuda.c:1023-1083); on MI355X each launch and each dependent global read costs
@@ -77,7 +77,7 @@ struct FusedArgs {
 // carries the generation itself.  No clean-up between launches: every counter is reset by the launch that used it.
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
-#define FG_MAXT 16      // rows of the grouped kernel
+#define FG_MAXT 24      // rows of the grouped kernel
 #define FG_MINT_SHARED 6   // with an always-on expert (every row a pair on the same expert) it also takes 6 to 8 rows
 #define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // FG_MAXT x 1024 router logits, 64 bits each: value | generation << 32
 #define FUSED_IND_WORDS (FUSED_LOGIT_WORDS + 2 * FG_MAXT * 1024)   // FG_MAXT x 32 published selections, tagged the same way
@@ -551,7 +551,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 #undef DSTAMP
 }
 
-// ---- 9 to 16 tokens: the pairs of one expert share its decoded blocks ---------------------------------------------------
+// ---- 9 to 24 tokens: the pairs of one expert share its decoded blocks ---------------------------------------------------
 // With more tokens than experts-per-token slots, several (token, expert) pairs meet on the same expert, and the decode of
 // a block (nine tenths of the work) can serve them all.  Pairs are grouped by expert in runs of at most NT; an item is a
 // (group, row tile); a thread decodes its chunk once and multiplies it with the NT rows of activations staged side by side
@@ -1079,8 +1079,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     a.it_d = (d + a.rpid - 1) / a.rpid;
     if (T > MV_MAXT || (shared && T >= FG_MINT_SHARED && sg && T * a.kk <= FG_MAXP)) {
         // More rows than the per-pair kernel takes: pairs grouped by expert, two to a decode.  Measured against the grouped
-        // GEMMs of the separate launches (C2, 16 rows: 199 against 268 us); with four to a decode (17 to 32 rows: 402 against
-        // 338 us at 32) and where the gate+up row sums go through LDS (C3's 45 chunks a row: 1129 against 753 us) the GEMMs
+        // GEMMs of the separate launches (C2, 16 rows: 199 against 268 us; 20 rows: 242 against 295; 24 rows: 278 against 305;
+        // 28 rows: 335 against 327, so the limit is 24); with four to a decode (402 against 338 us at 32 rows) and where the gate+up row sums go through LDS (C3's 45 chunks a row: 1129 against 753 us) the GEMMs
         // win, so those shapes are left to them.  With an always-on expert every row brings a pair on the same expert, and
         // the grouped kernel is already ahead of the per-pair one at 6 rows (whole model, 8 rows: 5.37 against 5.70 ms); without
         // one the two are level at 8 rows (130 us) and the per-pair kernel is ahead below.

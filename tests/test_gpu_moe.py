@@ -35,7 +35,7 @@ def expert_ref(orc, gate, up, down, e, x, gemm):
 
 
 @pytest.mark.parametrize("router", [0, 1])
-@pytest.mark.parametrize("T", [1, 5, 8, 20])
+@pytest.mark.parametrize("T", [1, 5, 8, 20, 27])
 @pytest.mark.parametrize("slots", [0, 20])
 def test_moe_step(oracle, router, T, slots):
     from nanoseedlm_amd import moe
@@ -91,8 +91,8 @@ def test_moe_step(oracle, router, T, slots):
             # the layer output from the GPU's own routing
             for t in range(T):
                 # above 8 rows the separate launches take the grouped GEMM (BF16-rounded weights); the persistent kernel
-                # (softmax routing, every expert resident) keeps the exact weights of the decode path up to 16 rows
-                gemm = T > 8 and not (router == 0 and slots == 0 and T <= 16)
+                # (softmax routing, every expert resident) keeps the exact weights of the decode path up to 24 rows
+                gemm = T > 8 and not (router == 0 and slots == 0 and T <= 24)
                 ys = np.stack([expert_ref(oracle, gate, up, down, int(ind[t, j]), xn[t], gemm=gemm) for j in range(k)])
                 if router == 0:
                     want = (wt[t].astype(np.float64)[:, None] * ys).sum(0)
@@ -112,7 +112,7 @@ def test_moe_step(oracle, router, T, slots):
     st.close()
 
 
-@pytest.mark.parametrize("T", [1, 3, 5, 6, 7, 8, 12, 16])
+@pytest.mark.parametrize("T", [1, 3, 5, 6, 7, 8, 12, 16, 19, 24])
 def test_whole_expert_block_in_one_launch(T):
     """nslm_moe_step_layer (input RMSNorm + routed experts + shared expert + residual inside the persistent kernel) writes the
     same bits as kq4_norm1p + nslm_moe_step + kc_mv_gu / kc_mv (shared expert) + kc_residual_add.  With the shared expert
@@ -244,7 +244,7 @@ def test_fused_step_rows_that_do_not_fill_a_workgroup(d, ff, fmt):
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
 @pytest.mark.parametrize("E,k", [(16, 4), (64, 4), (200, 8), (300, 6)])
-@pytest.mark.parametrize("T", [9, 13, 16])
+@pytest.mark.parametrize("T", [9, 13, 16, 21, 24])
 def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
     """More than 8 rows: the persistent kernel groups the pairs of an expert, and every row comes out as the per-pair kernel
     computes it in steps of at most 8 rows - routing, weights and outputs bit for bit (16 experts: many pairs an expert,
@@ -253,7 +253,7 @@ def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
     rng = np.random.default_rng(900 + T + E)
     d, ff = 256, 192
     mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
-    st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=16)
+    st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=24)
     gate, up, down = mk(rng, E, ff, d, eb=-21), mk(rng, E, ff, d, eb=-21), mk(rng, E, d, ff, eb=-20)
     st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
     st.finalize()
@@ -282,22 +282,22 @@ def test_grouped_step_equals_per_pair_steps(T, E, k, fmt):
 
 
 def test_steps_of_changing_size_share_the_barrier_words():
-    """Launches with one grid barrier (up to 8 rows) and two (9 to 16 rows), of different grid sizes, follow each other on
-    one set of barrier words: no barrier gives up, and every step returns what the same step returned the first time."""
+    """Launches of the per-pair kernel (up to 8 rows) and of the grouped kernel (9 to 24 rows), of different grid sizes, follow
+    each other on one set of sync words: no wait gives up, and every step returns what the same step returned the first time."""
     from nanoseedlm_amd import moe
     rng = np.random.default_rng(4242)
     E, k, d, ff = 32, 4, 256, 192
-    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=16)
+    st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=24)
     gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, d, ff, eb=-20)
     st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
     st.finalize()
-    xn = packs.round_bf16(rng.standard_normal((16, d)).astype(np.float32))
-    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf(4 * 16 * d)
+    xn = packs.round_bf16(rng.standard_normal((24, d)).astype(np.float32))
+    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf(4 * 24 * d)
     first = {}
     for rep in range(6):
-        for T in (1, 12, 3, 16, 8, 9, 9, 2, 13, 1, 1, 16):
+        for T in (1, 12, 3, 24, 16, 8, 9, 19, 9, 2, 13, 1, 24, 1, 16):
             st.step(None, 0, dx.ptr, T, dio.ptr)
-            out = dio.to_array(np.float32, (16, d))[:T].copy()
+            out = dio.to_array(np.float32, (24, d))[:T].copy()
             assert st.fused_error() == 0, (rep, T)
             if T not in first:
                 first[T] = out
@@ -305,6 +305,8 @@ def test_steps_of_changing_size_share_the_barrier_words():
             assert np.array_equal(out.view(np.uint32), first[T].view(np.uint32)), (rep, T)
     # rows are the same whatever the step size they came in
     assert np.array_equal(first[16][:8].view(np.uint32), first[8].view(np.uint32))
+    assert np.array_equal(first[24][:16].view(np.uint32), first[16].view(np.uint32))
+    assert np.array_equal(first[19][:9].view(np.uint32), first[9].view(np.uint32))
     assert np.array_equal(first[13][:1].view(np.uint32), first[1].view(np.uint32))
     dx.free(); dio.free()
     st.close()
