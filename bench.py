@@ -225,14 +225,14 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     return res
 
 
-def model_workload(name, steps, warmup, no_graph, branches=False):
+def model_workload(name, steps, warmup, no_graph, branches=False, splits=32):
     """Config 4: greedy decode of the whole synthetic model (24 layers of MLA attention over an FP8 latent cache + 128 seeded
     experts top-8 + a shared expert, tied BF16 LM head over 151936 ids), the cache pre-filled so that the timed steps end at
     the 4096th position.  A step = one token for each of the batch's sequences, all of its launches in one hipGraph."""
     from nanoseedlm_amd import backend, model, moe
     T = int(name[3:])
     cfg = dict(n_layer=24, d=2048, n_head=16, head_dim=128, r=512, rope=64, n_exp=128, top_k=8, ff=768, ff_shared=768, vocab=151936,
-               max_ctx=4096, max_rows=T, kv_fmt=backend.KV_FP8, n_splits=32, eps=1e-6, rope_theta=10000.0)
+               max_ctx=4096, max_rows=T, kv_fmt=backend.KV_FP8, n_splits=splits, eps=1e-6, rope_theta=10000.0)
     if steps + warmup + 8 > cfg["max_ctx"]:
         sys.exit("bench.py: c4 decodes towards position 4096; --steps + --warmup must stay below 4088")
     m = model.DecodeModel(**cfg)
@@ -430,6 +430,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="plain stream launches even for multi-launch steps")
     ap.add_argument("--graph", action="store_true", help="one hipGraph per step even when the step is a single launch")
+    ap.add_argument("--splits", type=int, default=32, help="c4: pieces the attention of a (row, head group) is split into over the context")
     ap.add_argument("--branches", action="store_true", help="c4: independent launches of a layer on side streams (parallel graph branches; measured slower)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="after the workload, run 20 device-to-device copies of this size: a copy kernel of known traffic "
@@ -445,7 +446,7 @@ def main():
         single = int(a.workload[3:]) <= 8 and a.workload[:2] == "c2"
         r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or (single and not a.graph))
     elif a.workload[:2] == "c4":
-        r = model_workload(a.workload, a.steps, a.warmup, a.no_graph, a.branches)
+        r = model_workload(a.workload, a.steps, a.warmup, a.no_graph, a.branches, a.splits)
     else:
         r = dense_workload(a.workload, a.steps, a.warmup)
     gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6
