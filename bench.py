@@ -71,14 +71,20 @@ class Q4Projections:
         self.q, self.kk, self.v, self.o, self.a, self.g, self.u, self.sh = (f(T * d) for _ in range(8))
         self.px, self.pa = moe.DevBuf(2 * T * d), moe.DevBuf(2 * T * d)
         self.sel0 = moe.DevBuf.from_array(np.zeros(max(T, 1), dtype=np.int32))
+        self.R3, self.add3 = (C.c_int * 3)(d, d, d), (C.c_int * 3)(0, 0, 0)
+        self.y3 = (C.c_void_p * 3)(self.q.ptr.value, self.kk.ptr.value, self.v.ptr.value)
+        self.L.kc_mv_multi.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(backend.WSlice), C.POINTER(C.c_int), C.POINTER(C.c_void_p),
+                                       C.POINTER(C.c_int), C.POINTER(C.c_int), C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_float]
 
     def run(self, stream, layer, x_ptr):
         from nanoseedlm_amd import packs
         L, d, T, Q4 = self.L, self.d, self.T, packs.MF_Q4
         arr, tab = self.layers[layer]
         if T <= 8:
-            for i, y in enumerate((self.q, self.kk, self.v)):
-                L.kc_mv(stream, Q4, arr[i], d, d, x_ptr, d, y.ptr, d, T, 0, None)
+            # q, k, v over the same input: one launch (kc_mv_multi; the same bits as one kc_mv each), else the three launches
+            if L.kc_mv_multi(stream, Q4, 3, arr, self.R3, self.y3, self.R3, self.add3, d, x_ptr, d, T, None, C.c_float(0.0)):
+                for i, y in enumerate((self.q, self.kk, self.v)):
+                    L.kc_mv(stream, Q4, arr[i], d, d, x_ptr, d, y.ptr, d, T, 0, None)
             L.kc_mv(stream, Q4, arr[3], d, d, self.q.ptr, d, self.o.ptr, d, T, 0, None)
             # shared expert: the gather entry points with every pair on slice 0 (as engine/qwen4_cuda.c:1029 does)
             L.kc_mv_gu(stream, Q4, tab.at(4 * C.sizeof(arr[0])), tab.at(5 * C.sizeof(arr[0])), d, d, x_ptr, d, self.a.ptr, d,

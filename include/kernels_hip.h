@@ -77,7 +77,9 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
  * the same T <= 64 rows of x in ONE launch per 8 rows, y[j][t * ys[j] + r] (+)= as kc_mv writes it, bit for bit.  0, or -1 when the
  * shapes are outside the seed fast path (K % 64, K > 6144, unaligned x): nothing is launched, call kc_mv per matrix.
  * norm_w (f32 [K], K <= 4096) or NULL: the rows of x are normalised first, exactly as kq4_norm1p(x, K, K, norm_w, norm_eps) would
- * have stored them (each workgroup recomputes the row's scale; the launch of the norm is saved). */
+ * have stored them (each workgroup recomputes the row's scale; the launch of the norm is saved).
+ * BF16 / Q8 / Q4 matrices (fmt as for kc_mv): the same in one launch for T <= MV_MAXT rows, K % 8 == 0, x 16-byte aligned,
+ * without norm_w (-1 with it). */
 int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,
                 const float* x, int xs, int T, const float* norm_w, float norm_eps);
 void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,

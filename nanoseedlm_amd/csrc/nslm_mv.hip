@@ -354,20 +354,33 @@ template <int FMT, int MODE>
 __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
     extern __shared__ __attribute__((aligned(16))) float xw[];   // [nt][K]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int pair = MODE == DENSE ? 0 : (int) blockIdx.y;
+    constexpr bool DNW = MODE == DENSE || MODE == MULTI;   // all tokens against the rows of one matrix (MULTI: of up to MV_MAXJ)
+    const int pair = DNW ? 0 : (int) blockIdx.y;
     WSlice wA = a.wd, wB = a.wd;
-    if (MODE != DENSE) {
+    if (!DNW) {
         const int sl = a.sel[pair];
         wA = a.ws[sl];
         if (MODE == GATEUP) wB = a.wu[sl];
     }
-    const float* xrow = a.x + (size_t) (MODE == DENSE ? 0 : pair / a.xdiv) * a.xs;
-    const int nbk = a.K / 8, nt = MODE == DENSE ? a.nt : 1;
-    const bool alA = ((uintptr_t) wA.p[0] & 15u) == 0, alB = ((uintptr_t) wB.p[0] & 15u) == 0;
+    const float* xrow = a.x + (size_t) (DNW ? 0 : pair / a.xdiv) * a.xs;
+    const int nbk = a.K / 8, nt = DNW ? a.nt : 1;
+    bool alA = ((uintptr_t) wA.p[0] & 15u) == 0;
+    const bool alB = ((uintptr_t) wB.p[0] & 15u) == 0;
+    int total = a.R;
+    if (MODE == MULTI) {
+        total = 0;
+        for (int j = 0; j < a.nj; ++j) total += a.Rj[j];
+    }
     for (int t = 0; t < nt; ++t)
         for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[(size_t) t * (a.K / 4) + i] = ((const float4*) (xrow + (size_t) t * a.xs))[i];
     __syncthreads();
-    for (int r = (int) blockIdx.x * 4 + wv; r < a.R; r += (int) gridDim.x * 4) {
+    for (int rr = (int) blockIdx.x * 4 + wv; rr < total; rr += (int) gridDim.x * 4) {
+        int r = rr, job = 0;
+        if (MODE == MULTI) {   // the matrix this row belongs to (the rows of the matrices follow each other)
+            while (job + 1 < a.nj && r >= a.Rj[job]) r -= a.Rj[job++];
+            wA = a.wj[job];
+            alA = ((uintptr_t) wA.p[0] & 15u) == 0;
+        }
         float acc[MV_MAXT], accu = 0.0f;
 #pragma unroll
         for (int t = 0; t < MV_MAXT; ++t) acc[t] = 0.0f;
@@ -408,7 +421,8 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
                 for (int o = 32; o > 0; o >>= 1) u += __shfl_xor(u, o);
                 if (lane == 0) a.y[(size_t) pair * a.ys + r] = a.f32out ? (s / (1.0f + expf(-s))) * u : bfr(silu_bf(bfr(s)) * bfr(u));
             } else if (lane == 0) {
-                store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + r, s, a.add, a.f32out);
+                if (MODE == MULTI) store_y(a.yj[job] + (size_t) t * a.ysj[job] + r, s, a.addj[job], a.f32out);
+                else store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + r, s, a.add, a.f32out);
             }
         }
     }
@@ -482,9 +496,14 @@ bool wide_ok(int fmt, int K, const void* x, int xs, int nt) {
 }
 template <int MODE>
 void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
-    const size_t lds = (size_t) (MODE == DENSE ? a.nt : 1) * a.K * sizeof(float);
+    const size_t lds = (size_t) (MODE == DENSE || MODE == MULTI ? a.nt : 1) * a.K * sizeof(float);
     // about 8 small workgroups a CU when the rows allow it; a wave then walks its rows with a grid stride
-    int gx = (a.R + 3) / 4;
+    int rows = a.R;
+    if (MODE == MULTI) {
+        rows = 0;
+        for (int j = 0; j < a.nj; ++j) rows += a.Rj[j];
+    }
+    int gx = (rows + 3) / 4;
     const int cap = (8 * cu_count() + ny - 1) / ny;
     if (gx > cap) gx = cap < 1 ? 1 : cap;
     const dim3 grid((unsigned) gx, (unsigned) ny);
@@ -564,6 +583,18 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
 
 int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,
                 const float* x, int xs, int T, const float* norm_w, float norm_eps) {
+    if (n >= 1 && n <= MV_MAXJ && T >= 1 && T <= MV_MAXT && !norm_w && wide_ok(fmt, K, x, xs, T)) {
+        // BF16 / Q8 / Q4: a wave a row, the rows of the n matrices one after the other (the same row sums as kc_mv's)
+        MvArgs a = {};
+        a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.nj = n; a.nt = T;
+        for (int j = 0; j < n; ++j) {
+            if (R[j] < 1) return -1;
+            a.wj[j] = w[j]; a.Rj[j] = R[j]; a.ysj[j] = ys[j]; a.addj[j] = add[j]; a.yj[j] = y[j];
+        }
+        launch_wide<MULTI>((hipStream_t) s, fmt, a, 1);
+        note_launch();
+        return 0;
+    }
     int L, rpi;
     bool shfl;
     if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MULTI_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;

@@ -459,6 +459,50 @@ def test_mv_multi_equals_separate_matvecs(fmt, T):
         assert np.array_equal(a.view(np.uint32), b.view(np.uint32)) and not np.array_equal(a, ya[j].to_array(np.float32, (T, R))), j
 
 
+@pytest.mark.parametrize("fmt", [packs.MF_Q4, packs.MF_Q8, packs.MF_BF16])
+@pytest.mark.parametrize("T", [1, 3, 8])
+def test_mv_multi_affine_and_bf16_equal_separate_matvecs(fmt, T):
+    """kc_mv_multi over BF16 / Q8 / Q4 matrices (the q / k / v projections of the mixed-format layer): one launch, a wave a
+    row over the rows of all matrices, bit-equal to one kc_mv each (ragged row counts, one job accumulating into y);
+    refused - nothing launched - with an input norm or more than 8 tokens."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(57 + T + fmt)
+    K, Rs, adds = 704, [130, 9, 500], [0, 1, 0]
+    x = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, K)).astype(np.float32)))
+    keep, ws = [], (backend.WSlice * 3)()
+    for j, R in enumerate(Rs):
+        if fmt == packs.MF_BF16:
+            bufs = [moe.DevBuf.from_array(packs.f32_to_bf16_bits((rng.standard_normal((R, K)) * 0.05).astype(np.float32)))]
+            ws[j].p[0] = bufs[0].ptr.value
+        else:
+            pk = packs.affine(rng, 1, R, K, bits=4 if fmt == packs.MF_Q4 else 8, group=64)
+            bufs = [moe.DevBuf.from_array(pk[k][0]) for k in ("words", "scales", "biases")]
+            ws[j].p[0], ws[j].p[1], ws[j].p[2], ws[j].gs = bufs[0].ptr.value, bufs[1].ptr.value, bufs[2].ptr.value, 6
+        keep += bufs
+    y0 = [packs.round_bf16(rng.standard_normal((T, R)).astype(np.float32)) for R in Rs]
+    ya, yb = [moe.DevBuf.from_array(v) for v in y0], [moe.DevBuf.from_array(v) for v in y0]
+    for j, R in enumerate(Rs):
+        L.kc_mv(None, fmt, ws[j], K, R, x.ptr, K, ya[j].ptr, R, T, adds[j], None)
+    Ra, ysa, ada = (C.c_int * 3)(*Rs), (C.c_int * 3)(*Rs), (C.c_int * 3)(*adds)
+    yp = (C.c_void_p * 3)(*[b.ptr.value for b in yb])
+    L.kc_mv_multi.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(backend.WSlice), C.POINTER(C.c_int), C.POINTER(C.c_void_p), C.POINTER(C.c_int),
+                              C.POINTER(C.c_int), C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_float]
+    assert L.kc_mv_multi(None, fmt, 3, ws, Ra, yp, ysa, ada, K, x.ptr, K, T, None, 0.0) == 0
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    for j, R in enumerate(Rs):
+        a, b = ya[j].to_array(np.float32, (T, R)), yb[j].to_array(np.float32, (T, R))
+        assert np.abs(a).max() > 0 and not np.array_equal(a, y0[j]) and np.array_equal(a.view(np.uint32), b.view(np.uint32)), j
+    nw = moe.DevBuf.from_array(np.zeros(K, dtype=np.float32))
+    assert L.kc_mv_multi(None, fmt, 3, ws, Ra, yp, ysa, ada, K, x.ptr, K, T, nw.ptr, 1e-6) == -1
+    assert L.kc_mv_multi(None, fmt, 3, ws, Ra, yp, ysa, ada, K, x.ptr, K, 9, None, 0.0) == -1
+    for b in keep + ya + yb + [x, nw]:
+        b.free()
+
+
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
 @pytest.mark.parametrize("K,R", [(768, 300), (2048, 96), (256, 1000)])
 @pytest.mark.parametrize("T", [5, 16, 23, 64])
