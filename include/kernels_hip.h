@@ -273,7 +273,7 @@ int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice
  * shape, pair top_k of every token with weight 1.  res or NULL: out = bf16(res + bf16(sum)), res may be out.  A and D then
  * hold T * (top_k + 1) rows.  norm_w (f32 [d], d <= 4096) or NULL: x is normalised first, as kq4_norm1p(x, d, d, norm_w, norm_eps)
  * would have stored it (res stays the raw stream).  Same results as the separate launches: sum = f32 sum_j wt_j bf16(y_j) +
- * bf16(y_shared).  With a shared expert the expert-sharing form of the kernel is used from 6 tokens on (every token brings a
+ * bf16(y_shared).  With a shared expert the expert-sharing form of the kernel is used from 5 tokens on (every token brings a
  * pair on that expert); the rows are the same bits either way. */
 int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,

@@ -78,7 +78,7 @@ struct FusedArgs {
 #define BAR_GROUPS 32
 #define FUSED_ERR_WORD (32 * (2 * BAR_GROUPS + 1))
 #define FG_MAXT 24      // rows of the grouped kernel
-#define FG_MINT_SHARED 6   // with an always-on expert (every row a pair on the same expert) it also takes 6 to 8 rows
+#define FG_MINT_SHARED 5   // with an always-on expert (every row a pair on the same expert) it also takes 5 to 8 rows
 #define FUSED_LOGIT_WORDS (32 * (2 * BAR_GROUPS + 2))   // FG_MAXT x 1024 router logits, 64 bits each: value | generation << 32
 #define FUSED_IND_WORDS (FUSED_LOGIT_WORDS + 2 * FG_MAXT * 1024)   // FG_MAXT x 32 published selections, tagged the same way
 #define FUSED_TILES 256   // most items a pair in a pass of the per-pair kernel
@@ -1082,7 +1082,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         // GEMMs of the separate launches (C2, 16 rows: 199 against 268 us; 20 rows: 242 against 295; 24 rows: 278 against 305;
         // 28 rows: 335 against 327, so the limit is 24); with four to a decode (402 against 338 us at 32 rows) and where the gate+up row sums go through LDS (C3's 45 chunks a row: 1129 against 753 us) the GEMMs
         // win, so those shapes are left to them.  With an always-on expert every row brings a pair on the same expert, and
-        // the grouped kernel is already ahead of the per-pair one at 6 rows (whole model, 8 rows: 5.37 against 5.70 ms); without
+        // the grouped kernel is already ahead of the per-pair one at 5 rows (whole model, 5 rows: 4.05 against 4.18 ms, 8 rows:
+        // 5.37 against 5.70; 4 rows: 3.85 against 3.68); without
         // one the two are level at 8 rows (130 us) and the per-pair kernel is ahead below.
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
