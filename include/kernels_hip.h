@@ -239,7 +239,8 @@ void kc_kv_f32(kc_stream_t s, int fmt, const uint8_t* codes, const uint8_t* scal
 /* ---- additions for a host that runs a whole synthetic model (no counterpart in the reference's header) -------------------- */
 /* x = bf16(x + bf16(a + b)) (b may be NULL): the residual stream takes a block's branch outputs, BF16 at the boundary */
 void kc_residual_add(kc_stream_t s, float* x, const float* a, const float* b, size_t n);
-/* ri[t].pos += 1 for t < T: positions live on the device so that a captured decode step replays */
+/* ri[t].pos += 1 for t < T: positions live on the device so that a captured decode step replays.  ri[t].pad[0] > 0 is the
+ * length of the row's cache slot: the position saturates at pad[0] - 1 (0: no bound, the reference's RowInfo leaves it 0) */
 void kc_rows_advance(kc_stream_t s, RowInfo* ri, int T);
 /* reproducible pseudo-random fills for synthetic packs: bytes (any bytes are valid seed records; nbytes rounded down to 8),
  * and BF16 values uniform in [-scale, scale] */

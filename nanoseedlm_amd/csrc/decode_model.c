@@ -30,6 +30,7 @@ struct NslmModel {
     float *x, *xn, *q, *cl, *kr, *qr, *ql, *olat, *o, *part, *mo, *as, *gs, *us, *sh, *logits;
     uint16_t *px, *pa;                 /* BF16 views of activations for the GEMM path */
     int final;
+    int next_pos;                      /* the largest position the next step writes (host-side bound; -1 before nslm_model_start) */
     int branches;                      /* independent launches of a layer on side streams (parallel graph branches) */
     nh_stream_t side[2];
     nh_event_t ev[4];
@@ -84,6 +85,7 @@ NslmModel* nslm_model_open(const NslmModelCfg* c, char* err, int errlen) {
         return NULL;
     }
     NslmModel* m = (NslmModel*) calloc(1, sizeof *m);
+    if (m) m->next_pos = -1;
     m->c = *c;
     if (m->c.n_splits <= 0) m->c.n_splits = 32;
     NslmMoeCfg mc = {c->n_layer, c->n_exp, c->top_k, c->d, c->ff, MF_SEED4P4, NSLM_ROUTE_SOFTMAX, c->max_rows, 0, 1.0f};
@@ -229,13 +231,17 @@ int nslm_model_fill_random(NslmModel* m, uint64_t seed, int eb) {
 int nslm_model_start(NslmModel* m, int T, const int32_t* ids, const int32_t* pos) {
     if (T < 1 || T > m->c.max_rows) return -1;
     RowInfo ri[64];
+    int hi = 0;
     if (T > 64) return -1;
     memset(ri, 0, sizeof ri);
     for (int t = 0; t < T; ++t) {
         if (pos[t] < 0 || pos[t] >= m->c.max_ctx || ids[t] < 0 || ids[t] >= m->c.vocab) return -1;
         ri[t].pos = pos[t];
         ri[t].kv0 = t * m->c.max_ctx;
+        ri[t].pad[0] = m->c.max_ctx;   /* kc_rows_advance never moves a row past its slot's last position */
+        if (pos[t] > hi) hi = pos[t];
     }
+    m->next_pos = hi;
     int bad = nh_device_sync();
     bad |= nh_memcpy_h2d(m->ri, ri, sizeof(RowInfo) * (size_t) T);
     bad |= nh_memcpy_h2d(m->ids, ids, 4 * (size_t) T);
@@ -276,6 +282,9 @@ static void dense(const NslmModel* m, kc_stream_t s, const Dense* dn, const floa
 int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
     const NslmModelCfg* c = &m->c;
     if (!m->final || T < 1 || T > c->max_rows) return -1;
+    /* a step writes the cache at each row's position: refused once a sequence slot is full (the positions advance on the
+       device, so the host keeps the bound: nslm_model_start's largest position + the steps issued since) */
+    if (m->next_pos < 0 || m->next_pos >= c->max_ctx) return -1;
     const int d = c->d, H = c->n_head, hd = c->head_dim, r = c->r, rope = c->rope, QD = qd(c), ffs = c->ff_shared;
     const int big = T > MV_MAXT, bigd = T > DENSE_MV_ROWS;   /* rows above which the experts / the dense projections take the GEMMs */
     const size_t rows = cache_rows(c), e = kv_elem(c);
@@ -395,12 +404,23 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
     }
     kc_argmax(s, m->logits, m->ids, c->vocab, T);
     kc_rows_advance(s, m->ri, T);
+    m->next_pos += 1;
     return kc_last_error() ? -1 : 0;
 }
 
-int nslm_model_ids(NslmModel* m, int T, int32_t* ids) { return nh_device_sync() || nh_memcpy_d2h(ids, m->ids, 4 * (size_t) T) ? -1 : 0; }
+int nslm_model_steps_left(const NslmModel* m) { return m->next_pos < 0 ? 0 : m->c.max_ctx - m->next_pos; }
+int nslm_model_account(NslmModel* m, int steps) {
+    if (m->next_pos < 0 || m->next_pos + steps > m->c.max_ctx || m->next_pos + steps < 0) return -1;
+    m->next_pos += steps;
+    return 0;
+}
+
+/* (both synchronise, and report -1 when a wait inside the persistent expert kernel gave up since open: its results are void) */
+int nslm_model_ids(NslmModel* m, int T, int32_t* ids) {
+    return nh_device_sync() || nh_memcpy_d2h(ids, m->ids, 4 * (size_t) T) || nslm_moe_fused_error(m->moe) ? -1 : 0;
+}
 int nslm_model_logits(NslmModel* m, int T, float* logits) {
-    return nh_device_sync() || nh_memcpy_d2h(logits, m->logits, 4 * (size_t) T * m->c.vocab) ? -1 : 0;
+    return nh_device_sync() || nh_memcpy_d2h(logits, m->logits, 4 * (size_t) T * m->c.vocab) || nslm_moe_fused_error(m->moe) ? -1 : 0;
 }
 uint64_t nslm_model_step_bytes(const NslmModel* m) {
     const NslmModelCfg* c = &m->c;

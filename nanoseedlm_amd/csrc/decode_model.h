@@ -59,8 +59,16 @@ int nslm_model_fill_cache(NslmModel* m, int T, int upto, uint64_t seed);
  * expert beside the routed ones - the reference runs that one on a second stream, engine/qwen4_cuda.c:1026-1032) go to
  * two side streams joined by events, which a captured step turns into parallel graph branches.  Steps of up to 8 rows. */
 int nslm_model_set_branches(NslmModel* m, int on);
+/* -1 (nothing launched) when a sequence slot is full: a step writes the cache at every row's position, and the positions
+ * advance on the device, so the host keeps the bound - the largest position given to nslm_model_start plus the steps issued
+ * since.  A step captured into a graph counts once when captured; replays are accounted with nslm_model_account(m, n)
+ * before they are launched (-1: they would run past max_ctx; n < 0 takes steps back, e.g. the capture call itself, which
+ * launches nothing).  On the device the positions saturate at max_ctx - 1, so even an unaccounted replay stays inside the cache. */
 int nslm_model_step(NslmModel* m, kc_stream_t s, int T);
-/* synchronising reads for tests: the current ids, the last step's logits [T][vocab], the last step's final hidden rows */
+int nslm_model_steps_left(const NslmModel* m);
+int nslm_model_account(NslmModel* m, int steps);
+/* synchronising reads: the current ids, the last step's logits [T][vocab]; -1 also when a wait inside the persistent expert
+ * kernel gave up since open (the results are void then) */
 int nslm_model_ids(NslmModel* m, int T, int32_t* ids);
 int nslm_model_logits(NslmModel* m, int T, float* logits);
 /* compressed weight bytes one decode step of one token reads: experts selected + shared expert + dense + maps + LM head */

@@ -13,8 +13,8 @@
 // Data that one workgroup writes and another reads inside the launch (logits, A, D) moves with agent-scope relaxed
 // atomic stores and loads: on this GPU every XCD has its own L2, and those accesses go through to the coherent level, so
 // no device-scope fence (an L2 write-back / invalidate per workgroup, which costs far more than the step) is needed;
-// ordering against the counters and tagged words is a workgroup-scope release / acquire, i.e. a wait for outstanding
-// memory operations.
+// ordering against the counters and tagged words: every wave waits for its own stores to be acknowledged (an explicit
+// s_waitcnt vmcnt(0), see wg_release) before the workgroup barrier that precedes the flag store.
 //
 // Waiting: the grid is sized to the number of workgroups the device can hold at once (occupancy query), because
 // workgroups wait for each other's data; every wait is a bounded poll, and a workgroup that gives up sets an error word
@@ -67,9 +67,9 @@ struct FusedArgs {
 //   [FUSED_DFLAG_WORDS ..] a word per down item, set to the generation + 1 when its rows are stored; the down item of a
 //                        token's last expert polls the words of the other experts' items of its row tile and sums (a
 //                        ticket per (token, row tile) cost an atomic's round trip more before the sum)
-//   [FUSED_SYNC_WORDS ..] the grouped kernel's words: one ticket per (token, down row tile); behind them (at T (d + 1))
-//                        three words per group, each on its own line: finished gate+up items (atomics only), the group's
-//                        ready flag (what waiters poll), finished down items; then the rows' scales
+//   [FUSED_SYNC_WORDS ..] the grouped kernel's words: FG_RN_WORDS for the rows' published scales; three words per group
+//                        (FG_MAXP groups at most), each on its own line: finished gate+up items (atomics only), the group's
+//                        ready flag (what waiters poll), finished down items; then one ticket per (token, down row tile)
 // Hundreds of device-scope atomics on ONE address serialise at tens of nanoseconds each, so arrivals go to 32 group
 // counters and only each group's last arrival touches the shared one.  Earlier versions of these kernels separated their
 // phases by grid barriers on the same words (arrive, then poll the group's generation word): 3.3 us behind the last
@@ -93,8 +93,17 @@ __device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store
 __device__ __forceinline__ void st_agent(uint32_t* p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ unsigned long long ld_agent(const unsigned long long* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_agent(unsigned long long* p, unsigned long long v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-// this workgroup's earlier memory operations have completed / later ones start after this point
-__device__ __forceinline__ void wg_release() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+// Release: every store this wave has issued is acknowledged before the wave goes on to the barrier behind which the
+// workgroup's flag (or counter) is written.  The data stores are agent-scope atomics, which write through to the level all
+// XCDs share, so "acknowledged" means "readable by an agent-scope load of any workgroup"; the wait for the vector-memory
+// counter is spelled out because a workgroup-scope fence alone need not contain one on this target (waves of one workgroup
+// share a CU and its cache, so the compiler may leave it out).  The fence keeps the compiler from moving memory operations
+// across this point.  Acquire: the readers' loads are agent-scope atomics issued after the poll's value has been used, so
+// nothing has to be invalidated; the fence again only pins the compiler's order.
+__device__ __forceinline__ void wg_release() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 __device__ __forceinline__ void wg_acquire() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
 // The generation moves on once per launch: every workgroup arrives (nobody waits), the last arrival writes the next number
@@ -641,9 +650,11 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     const uint32_t G = (uint32_t) a.grid;
     const int P_ = a.T * a.kk, NE = a.E + a.ns;
     const int xsg = a.Lg * XPAD, xsd = a.Ld * XPAD;   // LDS floats between two rows of activations
-    uint32_t* tick = a.sync + FUSED_SYNC_WORDS;
-    uint32_t* grpc = a.sync + FUSED_SYNC_WORDS + (size_t) a.T * (size_t) (a.d + 1);   // [group][3][32]: arrivals, ready, done
-    float* rnpub = (float*) (grpc + (size_t) a.T * 33 * 96);
+    // (fixed places, whatever the launch's rows and widths: launches of different sizes share the area, and every word
+    // but the scales is back at zero when a launch ends)
+    float* rnpub = (float*) (a.sync + FUSED_SYNC_WORDS);
+    uint32_t* grpc = a.sync + FUSED_SYNC_WORDS + FG_RN_WORDS;                     // [group][3][32]: arrivals, ready, done
+    uint32_t* tick = grpc + (size_t) FG_MAXP * 96;                                // [token][down row tile]
     // the generation (all sense words are equal); the workgroup arrives, without waiting, further down
     const uint32_t my_gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
     const uint32_t tag = my_gen + 1u;
@@ -1049,7 +1060,7 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
 
 extern "C" {
 
-size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + (size_t) T * (size_t) (d + 1) + (size_t) T * 33 * 96 + FG_RN_WORDS; }
+size_t kc_moe_decode_sync_words(int T, int d) { return FUSED_SYNC_WORDS + FG_RN_WORDS + (size_t) FG_MAXP * 96 + (size_t) T * (size_t) (d + 1); }
 int kc_moe_decode_max_rows(void) { return FG_MAXT; }
 int kc_moe_decode_error_word(void) { return FUSED_ERR_WORD; }
 

@@ -140,7 +140,10 @@ __global__ void __launch_bounds__(256) k_residual_add(float* x, const float* a, 
 }
 __global__ void k_rows_advance(RowInfo* ri, int T) {
     const int t = (int) (blockIdx.x * blockDim.x + threadIdx.x);
-    if (t < T) ri[t].pos += 1;
+    if (t < T) {   // pad[0] > 0: the sequence slot's length; a row on its last position stays there (the cache write stays inside the slot)
+        const int lim = ri[t].pad[0], nxt = ri[t].pos + 1;
+        ri[t].pos = lim > 0 && nxt >= lim ? lim - 1 : nxt;
+    }
 }
 // splitmix64 of the word index: reproducible pseudo-random bytes for synthetic packs (any bytes are valid seed records)
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {

@@ -575,9 +575,16 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         note_launch();
         return;
     }
-    a.nt = T;
-    if (T <= MV_MAXT && wide_ok(fmt, K, x, xs, T)) launch_wide<DENSE>(st, fmt, a, 1);
-    else hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, a);
+    // Every other shape: the kernels' token loops hold MV_MAXT tokens, so more rows go in runs of MV_MAXT (a token's result does
+    // not depend on the run it is in).
+    for (int t0 = 0; t0 < T; t0 += MV_MAXT) {
+        MvArgs b = a;
+        b.x = x + (size_t) t0 * xs;
+        b.y = y + (size_t) t0 * ys;
+        b.nt = T - t0 < MV_MAXT ? T - t0 : MV_MAXT;
+        if (wide_ok(fmt, K, b.x, xs, b.nt)) launch_wide<DENSE>(st, fmt, b, 1);
+        else hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, b);
+    }
     note_launch();
 }
 

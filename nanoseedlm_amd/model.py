@@ -87,12 +87,18 @@ class DecodeModel:
         backend.check(self.L.nslm_graph_begin(stream), "nslm_graph_begin")
         self.step(stream, T)
         g = C.c_void_p(self.L.nslm_graph_end(stream))
+        backend.check(self.L.nslm_model_account(self.h, -1), "nslm_model_account")   # the capture call launched nothing
         if not g:
             raise RuntimeError("graph capture failed")
         return g
 
     def launch(self, g, stream):
+        """One replay of a captured step; refused (RuntimeError) when a sequence slot is full."""
+        backend.check(self.L.nslm_model_account(self.h, 1), "nslm_model_account: the cache slot is full")
         backend.check(self.L.nslm_graph_launch(g, stream), "nslm_graph_launch")
+
+    def steps_left(self):
+        return int(self.L.nslm_model_steps_left(self.h))
 
     def ids(self, T):
         out = np.zeros(T, dtype=np.int32)

@@ -211,6 +211,22 @@ def test_mv_empty_and_ragged(be, oracle):
     assert close_bf(be.kt_mv(p, x), packs.round_bf16(ref.astype(np.float32)).astype(np.float64), F32B * mag).all()
 
 
+@pytest.mark.parametrize("fmt,K", [(packs.MF_SEED4P4, 72), (packs.MF_SEED4P4, 8256), (packs.MF_SEED4, 136), (packs.MF_BF16, 72),
+                                   (packs.MF_Q4, 128), (packs.MF_Q8, 192)])
+def test_mv_more_rows_than_a_pass_on_the_general_path(be, oracle, fmt, K):
+    """Shapes outside the seed fast path (K % 64 != 0, K > 8192) and the other formats with more than MV_MAXT = 8 rows: every
+    row is written (the launcher goes in runs of 8), and a row does not depend on the run it is in."""
+    rng = np.random.default_rng(K + 31 * fmt)
+    R, T = 19, 12
+    p = make_pack(rng, fmt, 1, R, K)
+    x = packs.round_bf16(rng.uniform(-1, 1, (T, K)).astype(np.float32))
+    y = be.kt_mv(p, x, y0=np.full((T, R), 777.0, dtype=np.float32))
+    ref, mag = ref_mv(oracle, p, 0, x)
+    assert close_bf(y, packs.round_bf16(ref.astype(np.float32)).astype(np.float64), F32B * mag).all(), (NAMES[fmt], K)
+    y1 = be.kt_mv(p, x[9:10])
+    assert np.array_equal(y[9].view(np.uint32), y1[0].view(np.uint32))
+
+
 # ---- GEMM -----------------------------------------------------------------------------------------------------------------------
 
 def ref_mm(orc, p, s, x, exact):

@@ -169,3 +169,34 @@ def test_graph_replay_equals_eager_steps(T):
     assert len(seen) == 6                                            # the steps differ from one another (positions advance)
     for m in ms:
         m.close()
+
+
+def test_a_full_cache_slot_refuses_the_next_step():
+    """A step writes the cache at every row's position and the positions advance on the device: the host refuses the step
+    (and the replay of a captured step) that would write past a sequence slot, and the device-side position saturates."""
+    from nanoseedlm_amd import backend, model, moe
+    backend.require_gpu()
+    T = 2
+    cfg = dict(n_layer=2, d=128, n_head=2, head_dim=64, r=64, rope=64, n_exp=8, top_k=2, ff=64, ff_shared=64, vocab=96, max_ctx=8,
+               max_rows=T, kv_fmt=backend.KV_BF16, n_splits=2, eps=1e-6, rope_theta=10000.0)
+    m = model.DecodeModel(**cfg)
+    m.fill_random(seed=3, eb=-13)
+    with pytest.raises(RuntimeError):
+        m.step(None, T)                                              # no start yet
+    m.start(np.array([5, 9], dtype=np.int32), np.array([2, cfg["max_ctx"] - 1], dtype=np.int32))
+    assert m.steps_left() == 1
+    m.step(None, T)                                                  # row 1 writes its slot's last position
+    assert np.isfinite(m.logits(T)).all() and m.steps_left() == 0
+    with pytest.raises(RuntimeError):
+        m.step(None, T)
+    m.start(np.array([5, 9], dtype=np.int32), np.array([0, cfg["max_ctx"] - 3], dtype=np.int32))
+    stream = moe.new_stream()
+    g = m.graph_of_step(stream, T)
+    assert m.steps_left() == 3                                       # the capture itself launched nothing
+    for _ in range(3):
+        m.launch(g, stream)
+    moe.device_sync()
+    assert np.isfinite(m.logits(T)).all()
+    with pytest.raises(RuntimeError):
+        m.launch(g, stream)
+    m.close()
