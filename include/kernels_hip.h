@@ -280,6 +280,23 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                         int32_t* ind, float* wt, float* A, float* D, uint32_t* sync, const WSlice* shared, const float* res, const float* norm_w,
                         float norm_eps);
+/* kc_moe_decode without a workspace argument.  No counterpart in the reference: it is for callers that cannot allocate device
+ * memory or carry a workspace around - code under stream capture, tight serving loops, harnesses that forbid hipMalloc.  What
+ * kc_moe_decode's caller owns as scratch (logits, A, D, the sync words) lives in one array inside the library's code object
+ * (4.9 MB of device memory on every GPU the library runs on, held until the process ends); the call allocates and frees nothing.
+ * ind / wt [T][top_k] (the routing) and out stay the caller's.  Results: kc_moe_decode's, bit for bit.
+ * status (device, 4 bytes) or NULL: receives the error word after the step (non-zero: a wait between workgroups gave up, the
+ * results are void) - one more one-thread launch.  clear != 0: the sync words are zeroed first (a fill kernel on s); needed
+ * only after such an error.
+ * Limits: T <= kc_moe_decode_max_rows(); T * n_exp + T * top_k * (ff + d) floats (each part rounded up to 64) <= 2^20;
+ * T * ceil(d / (256 / (ff / 64))) <= 24576.  Returns 0; -1 as kc_moe_decode (no fused kernel for the shape, nothing launched);
+ * -2 the shape is beyond the limits above (nothing launched, kc_last_error() reports an invalid value); -3 the array's address
+ * could not be obtained on the current device.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads) race - serialise them.
+ * The first call on a device looks the address up (hipGetSymbolAddress): make it outside a capture. */
+int kc_moe_decode_static(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
+                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, int32_t* ind, float* wt,
+                         uint32_t* status, int clear);
 /* last launch-configuration error of this library on the calling thread's device: 0 none, else a hipError_t value */
 int kc_last_error(void);
 

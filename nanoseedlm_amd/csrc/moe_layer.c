@@ -299,6 +299,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 
 void nslm_moe_set_fused(NslmMoe* m, int on) { m->fused = on; }
 void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }
+const uint16_t* nslm_moe_router_w(const NslmMoe* m, int layer) { return m->rw + (size_t) layer * m->c.n_exp * m->c.d; }
 int nslm_moe_fused_error(NslmMoe* m) {
     uint32_t w = 0;
     if (nh_device_sync() || nh_memcpy_d2h(&w, m->sync + kc_moe_decode_error_word(), 4)) return -1;

@@ -59,6 +59,8 @@ int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
 /* the device slice table [n_exp] of a layer's tensor (0 gate, 1 up, 2 down): what kc_mv_gu / kc_mv_sel take */
 const WSlice* nslm_moe_tab(const NslmMoe* m, int layer, int tensor);
+/* the device address of a layer's BF16 router weight [n_exp][d] */
+const uint16_t* nslm_moe_router_w(const NslmMoe* m, int layer);
 uint64_t nslm_moe_unit_bytes(const NslmMoe* m);
 /* compressed bytes one expert's three matrices occupy (without alignment padding) */
 uint64_t nslm_moe_expert_bytes(const NslmMoe* m);

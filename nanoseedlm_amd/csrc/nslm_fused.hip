@@ -1056,6 +1056,38 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
     return 0;
 }
 
+// ---- the step without a workspace argument -------------------------------------------------------------------------------
+// kc_moe_decode_static keeps what kc_moe_decode's caller brings along (logits, A, D, the sync words) in one array in device
+// memory that the library's code object itself holds, so the call allocates nothing: for callers that cannot call
+// hipMalloc (stream capture, tight serving loops, harnesses that forbid it).  Every GPU has its own copy of the array at
+// its own address; host code may not use the array's name as an address (that name is a host-side stand-in), so the address
+// on the current device is asked for once per device with hipGetSymbolAddress and kept.
+// Layout (uint32 words): [0, NA_SYNC_WORDS) the sync words, laid out as kc_moe_decode's with the ticket area sized
+// NA_TICK_WORDS - zero when the code object is loaded, and kept consistent by the kernels from launch to launch;
+// [NA_SYNC_WORDS, + NA_DATA_WORDS) logits [T][n_exp], A [T kk][ff], D [T kk][d], each starting on a 256-byte boundary,
+// overwritten by every call before it is read.
+#define NA_TICK_WORDS (FG_MAXT * 1024)
+#define NA_SYNC_WORDS (((FUSED_SYNC_WORDS + FG_RN_WORDS + FG_MAXP * 96 + NA_TICK_WORDS) + 63) & ~63)
+#define NA_DATA_WORDS (1 << 20)   // 4 MiB
+#define NA_MAX_DEVICES 64
+static __device__ __align__(256) uint32_t scratch[NA_SYNC_WORDS + NA_DATA_WORDS];
+
+uint32_t* scratch_on_this_device() {
+    static uint32_t* at[NA_MAX_DEVICES] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NA_MAX_DEVICES) return nullptr;
+    if (!at[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+        at[dev] = (uint32_t*) p;   // (two threads racing here store the same address)
+    }
+    return at[dev];
+}
+__global__ void __launch_bounds__(256) k_words_zero(uint32_t* p, size_t n) {
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) gridDim.x * 256) p[i] = 0u;
+}
+__global__ void k_word_copy(uint32_t* dst, const uint32_t* src) { *dst = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
 }   // namespace
 
 extern "C" {
@@ -1102,6 +1134,41 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
+}
+
+int kc_moe_decode_static(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
+                         int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, int32_t* ind, float* wt,
+                         uint32_t* status, int clear) {
+    if (T < 1 || T > FG_MAXT || n_exp < 1 || n_exp > 1024 || top_k < 1 || top_k > 32 || d < 8 || ff < 8) return -1;
+    // what the call needs of the array: the ticket words of the grouped kernel (rows x down iterations at most) and the data
+    int Ld, rpid;
+    bool sd;
+    if (!shape_of(ff, false, &Ld, &rpid, &sd)) return -1;
+    const size_t it_d = ((size_t) d + rpid - 1) / rpid, pairs = (size_t) T * top_k;
+    const size_t wl = ((size_t) T * n_exp + 63) & ~(size_t) 63, wa = (pairs * ff + 63) & ~(size_t) 63, wd = (pairs * d + 63) & ~(size_t) 63;
+    if ((size_t) T * it_d > NA_TICK_WORDS || wl + wa + wd > NA_DATA_WORDS) {
+        host_note_unsupported();
+        return -2;
+    }
+    uint32_t* base = scratch_on_this_device();
+    if (!base) {
+        host_note_unsupported();
+        return -3;
+    }
+    if (clear) {   // by a kernel, not a memset node: callers may be capturing
+        hipLaunchKernelGGL(k_words_zero, dim3(64), dim3(256), 0, (hipStream_t) s, base, (size_t) NA_SYNC_WORDS);
+        host_note_launch();
+    }
+    float* logits = (float*) (base + NA_SYNC_WORDS);
+    float* A = logits + wl;
+    float* D = A + wa;
+    const int rc = kc_moe_decode_layer(s, fmt, router_w, gate, up, down, n_exp, top_k, d, ff, x, xs, T, out, os, logits, ind, wt, A, D, base, NULL, NULL, NULL,
+                                       0.0f);
+    if (rc == 0 && status) {
+        hipLaunchKernelGGL(k_word_copy, dim3(1), dim3(1), 0, (hipStream_t) s, status, (const uint32_t*) base + FUSED_ERR_WORD);
+        host_note_launch();
+    }
+    return rc;
 }
 
 }   // extern "C"
