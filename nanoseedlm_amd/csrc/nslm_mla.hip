@@ -8,7 +8,7 @@
 // latent): 660 bytes at r = 512, rope 128, FP8 - so the attention of a 4096-token context moves 2.7 MB per row, and what
 // it costs is the 2 x (r + rope) multiply-adds per (key, head).  Latent 512 + RoPE 64 runs them on the matrix cores
 // (k_mla_attn_mfma: exact BF16 products, f32 sums, P as BF16 hi + lo, which holds the reference tests' bound of one BF16
-// ulp + 2e-6 of a double-precision softmax); other shapes stay in f32 on the vector ALUs (k_mla_attn).
+// ulp + 2e-6 of a double-precision softmax); other shapes stay in f32 on the vector ALUs (k_mla_attn_any).
 #include "nslm_mv_dev.h"
 
 using namespace nslm;
@@ -122,50 +122,71 @@ __global__ void __launch_bounds__(256) k_heads_mv(HmvArgs a, int fmt, WSlice W, 
 }
 
 // ---- RoPE of the query RoPE parts (in place) and of the RoPE key into the cache; the latent into the cache -------------
-// Thread i: latent dim i (i < r) and the pair (i % half, + half) of head i / half (head n_head: the key), half = rope / 2.
-// One wave's share (i = 64 consecutive values of one row t); QPART false leaves the query heads to the caller.
-template <bool QPART>
-__device__ __forceinline__ void rope_cache_wave(const MlaArgs& a, int rope, float* qr, const float* kr, const float* c, const KvView& kv,
-                                                const RowInfo* ri, const float* inv, int i, int t) {
-    const int pos = ri[t].pos, half = rope / 2;
+// The work of a row is cut into jobs of one wave each: job 0 rotates the RoPE key and writes it, job 1 + j writes latent
+// dims [64 j, 64 j + 64).  An FP8 block is 32 consecutive values, so it always sits in 32 consecutive lanes of one job and
+// its maximum is five shuffles.  (The reference gives thread i latent dim i and, at once, rotation pair i % half of head
+// i / half, engine/kernels_moe.cu:1177-1208; here the query heads are a loop of their own over a table of the row's
+// sines and cosines, computed once instead of once per head.)
+__device__ __forceinline__ void rotate(float x0, float x1, float cs, float sn, float* y0, float* y1) {
+    *y0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));   // spelled out: the same bits wherever it is inlined
+    *y1 = __fadd_rn(__fmul_rn(x1, cs), __fmul_rn(x0, sn));
+}
+__device__ __forceinline__ void cache_job(int job, const MlaArgs& a, int rope, const float* kr, const float* c, const KvView& kv, const RowInfo* ri,
+                                          const float* inv, int t) {
+    const int lane = threadIdx.x & 63, pos = ri[t].pos, half = rope / 2;
     int row;
     const KvSeg sg = kv_seg(kv, ri[t].kv0 + pos, &row);
-    const int head = i / half, p = i % half;
-    const bool lat = i < a.r, key = head == a.n_head;
-    float y0 = 0.0f, y1 = 0.0f;
-    if (QPART ? head <= a.n_head : key) {
-        float sn, cs;
-        sincosf((float) pos * inv[p], &sn, &cs);
-        float* qh = qr + ((size_t) t * a.n_head + (key ? 0 : head)) * rope;
-        const float* xh = key ? kr + (size_t) t * rope : qh;
-        const float x0 = xh[p], x1 = xh[p + half];
-        y0 = x0 * cs - x1 * sn;
-        y1 = x1 * cs + x0 * sn;
-        if (!key) { qh[p] = bfr(y0); qh[p + half] = bfr(y1); }
-    }
-    if (kv.fmt == KV_BF16) {
-        if (lat) ((uint16_t*) sg.v)[(size_t) row * a.r + i] = (uint16_t) tobf(c[(size_t) t * a.r + i]);
-        if (key) {
-            uint16_t* kc = (uint16_t*) sg.k + (size_t) row * rope;
-            kc[p] = (uint16_t) tobf(y0);
-            kc[p + half] = (uint16_t) tobf(y1);
+    if (job == 0) {   // the key: lane p < half holds the pair (p, p + half)
+        const bool on = lane < half;
+        float y0 = 0.0f, y1 = 0.0f;
+        if (on) {
+            float sn, cs;
+            sincosf((float) pos * inv[lane], &sn, &cs);
+            rotate(kr[(size_t) t * rope + lane], kr[(size_t) t * rope + lane + half], cs, sn, &y0, &y1);
+        }
+        if (kv.fmt == KV_BF16) {
+            if (on) {
+                uint16_t* kc = (uint16_t*) sg.k + (size_t) row * rope;
+                kc[lane] = (uint16_t) tobf(y0);
+                kc[lane + half] = (uint16_t) tobf(y1);
+            }
+        } else {   // every lane runs the shuffles
+            fp8_put(on, bfr(y0), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, on ? lane : 0);
+            fp8_put(on, bfr(y1), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, on ? lane + half : 0);
         }
         return;
     }
-    // FP8 (uniform over the grid): every lane runs the shuffles; 32 consecutive lanes are one block
-    fp8_put(lat, lat ? bfr(c[(size_t) t * a.r + i]) : 0.0f, (uint8_t*) sg.v, (uint8_t*) sg.vs, (size_t) row, a.r, lat ? i : 0);
-    fp8_put(key, bfr(y0), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, p);
-    fp8_put(key, bfr(y1), (uint8_t*) sg.k, (uint8_t*) sg.ks, (size_t) row, rope, p + half);
+    const int i = (job - 1) * 64 + lane;
+    const bool on = i < a.r;
+    const float v = on ? c[(size_t) t * a.r + i] : 0.0f;
+    if (kv.fmt == KV_BF16) {
+        if (on) ((uint16_t*) sg.v)[(size_t) row * a.r + i] = (uint16_t) tobf(v);
+    } else {
+        fp8_put(on, bfr(v), (uint8_t*) sg.v, (uint8_t*) sg.vs, (size_t) row, a.r, on ? i : 0);
+    }
 }
-__global__ void __launch_bounds__(64) k_mla_rope(MlaArgs a, int rope, float* qr, const float* kr, const float* c, KvView kv,
-                                                 const RowInfo* ri, const float* inv) {
-    rope_cache_wave<true>(a, rope, qr, kr, c, kv, ri, inv, (int) blockIdx.x * 64 + threadIdx.x, (int) blockIdx.y);
+// one workgroup a row: the cache jobs dealt to the four waves, then every query head's pairs
+__global__ void __launch_bounds__(256) k_mla_rope(MlaArgs a, int rope, float* qr, const float* kr, const float* c, KvView kv,
+                                                  const RowInfo* ri, const float* inv) {
+    __shared__ float cs_s[ATT_HD / 2], sn_s[ATT_HD / 2];
+    const int t = (int) blockIdx.x, tid = threadIdx.x, half = rope / 2;
+    if (tid < half) sincosf((float) ri[t].pos * inv[tid], &sn_s[tid], &cs_s[tid]);
+    for (int job = tid >> 6; job < 1 + (a.r + 63) / 64; job += 4) cache_job(job, a, rope, kr, c, kv, ri, inv, t);
+    __syncthreads();
+    for (int i = tid; i < a.n_head * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        float* qh = qr + ((size_t) t * a.n_head + h) * rope;
+        float y0, y1;
+        rotate(qh[p], qh[p + half], cs_s[p], sn_s[p], &y0, &y1);
+        qh[p] = bfr(y0);
+        qh[p + half] = bfr(y1);
+    }
 }
 
 // ---- the two maps of the query, its RoPE, and the cache write as ONE launch -----------------------------------------------
-// Grid (1 + r / 64 | cache blocks, n_head + 1, rows).  Head h < n_head: block 0 computes the `rope` rows of the RoPE mix
+// Grid (1 + r / 64, n_head + 1, rows).  Head h < n_head: block 0 computes the `rope` rows of the RoPE mix
 // (k_heads_mv's arithmetic), rotates them (k_mla_rope's) and stores them; block b > 0 computes latent-query rows
-// [64 (b - 1), 64 b).  "Head" n_head: the blocks write the rotated key and the latent into the cache (rope_cache_wave).
+// [64 (b - 1), 64 b).  "Head" n_head: the blocks' waves take the cache jobs (the rotated key, the latent).
 // The same bits as kc_heads_mv x 2 + kc_mla_rope.
 __global__ void __launch_bounds__(256) k_qmaps_rope(MlaArgs a, int rope, HmvArgs hq, HmvArgs hl, int fmt, WSlice Wq, WSlice Wl, const float* q,
                                                    float* qr, float* ql, const float* kr, const float* c, KvView kv, const RowInfo* ri,
@@ -173,10 +194,9 @@ __global__ void __launch_bounds__(256) k_qmaps_rope(MlaArgs a, int rope, HmvArgs
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float qs[ATT_HD];
     const int tid = threadIdx.x, h = (int) blockIdx.y, t = (int) blockIdx.z, b = (int) blockIdx.x;
-    if (h == a.n_head) {   // uniform over the block
-        const int nx = (a.n_head + 1) * (rope / 2) > a.r ? (a.n_head + 1) * (rope / 2) : a.r;
-        const int i0 = (b * 4 + (tid >> 6)) * 64;
-        if (i0 < nx) rope_cache_wave<false>(a, rope, qr, kr, c, kv, ri, inv, i0 + (tid & 63), t);
+    if (h == a.n_head) {   // uniform over the block: cache jobs 4 b .. 4 b + 3
+        const int job = b * 4 + (tid >> 6);
+        if (job < 1 + (a.r + 63) / 64) cache_job(job, a, rope, kr, c, kv, ri, inv, t);
         return;
     }
     if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
@@ -216,96 +236,103 @@ __global__ void __launch_bounds__(256) k_qmaps_rope(MlaArgs a, int rope, HmvArgs
     if (tid < half) {
         float sn, cs;
         sincosf((float) ri[t].pos * inv[tid], &sn, &cs);
-        const float x0 = qs[tid], x1 = qs[tid + half];
+        float y0, y1;
+        rotate(qs[tid], qs[tid + half], cs, sn, &y0, &y1);
         float* qh = qr + ((size_t) t * a.n_head + h) * rope;
-        qh[tid] = bfr(x0 * cs - x1 * sn);
-        qh[tid + half] = bfr(x1 * cs + x0 * sn);
+        qh[tid] = bfr(y0);
+        qh[tid + half] = bfr(y1);
     }
 }
 
-// ---- latent attention -----------------------------------------------------------------------------------------------------
-// Workgroup (split, head group, row) of HG waves, one query head a wave; lane l holds latent dims l, l + 64, .. (up to
-// MAXL) and RoPE dims l (, l + 64).  Each step stages KU keys (latent, then RoPE key) decoded to f32 in LDS once for the
-// workgroup's heads.  Score = scale (ql . c + qr . k), online softmax, f32 sums.  n_splits > 1: partials
-// [row][head][split] = (m, l, acc[r]) for k_mla_reduce; n_splits == 1: olat[row][head] = bf16(acc / l).
-#define MLA_KU 8
+// ---- latent attention, any shape (f32 on the vector ALUs) ---------------------------------------------------------------------
+// Workgroup (split, group of GA_HW heads, row), one query head a wave.  A tile of GA_KT keys (latent, then RoPE key) is decoded
+// to f32 in LDS once for the workgroup's heads.
+//   scores   lane (key u = lane / 4, quarter q = lane % 4) forms the part of s_u = q . k_u that falls into its quarter of the
+//            r + rope dims - sequential reads of the key's LDS row and of the wave's staged query - and two quad shuffles add
+//            the quarters: GA_KT scores a wave are ready at once (no wave-wide reduction per key);
+//   softmax  the tile's maximum and its sum of exp over the 16 quads: four shuffles each, once a tile;
+//   P c      lane l owns latent dims l, l + 64, ...; exp(s_u - m) reaches it as the broadcast of lane 4 u.
+// n_splits > 1: partials [row][head][split] = (m, l, acc[r]) for the reduce; n_splits == 1: olat[row][head] = bf16(acc / l).
+#define GA_KT 16
+#define GA_HW 4
 #define MLA_MAXL 16    // latent dims a lane (r <= 1024)
 #define MLA_SPLITS_SHORT 32
 __device__ __forceinline__ int mla_row_splits(const MlaArgs& a, int pos) {
     (void) pos;
     return a.pad[2] > 0 && a.n_splits > MLA_SPLITS_SHORT ? MLA_SPLITS_SHORT : a.n_splits;
 }
-template <int HG>
-__global__ void __launch_bounds__(64 * HG) k_mla_attn(MlaArgs a, int rope, const float* ql, const float* qr, KvView kv, const RowInfo* ri,
-                                                     float* out) {
-    __shared__ __attribute__((aligned(16))) float sh[MLA_KU * (64 * MLA_MAXL + ATT_HD)];
-    const int lane = threadIdx.x & 63, tid = threadIdx.x, ntg = 64 * HG;
-    const int split = (int) blockIdx.x, t = (int) blockIdx.z, r = a.r, nl = (r + 63) / 64, kw = r + rope;
-    const int h = (int) blockIdx.y * HG + (tid >> 6);
-    const int pos = ri[t].pos, ns = mla_row_splits(a, pos);
-    const int nsr = min(ns, (pos + a.chunk) / a.chunk);
-    const int chunk = (pos + nsr) / nsr;
-    const int p0 = split * chunk, p1 = split < nsr ? min(pos + 1, p0 + chunk) : p0;
+// the keys [p0, p1) of split `split` of a row at position pos: the row's own 0..pos in equal runs, as few as `chunk` keys a run allow
+__device__ __forceinline__ void split_range(const MlaArgs& a, int pos, int split, int* p0, int* p1) {
+    const int ns = mla_row_splits(a, pos), want = (pos + a.chunk) / a.chunk, used = ns < want ? ns : want, run = (pos + used) / used;
+    *p0 = split * run;
+    *p1 = split < used ? min(pos + 1, *p0 + run) : *p0;
+}
+__global__ void __launch_bounds__(64 * GA_HW) k_mla_attn_any(MlaArgs a, int rope, const float* ql, const float* qr, KvView kv, const RowInfo* ri,
+                                                            float* out) {
+    extern __shared__ __attribute__((aligned(16))) float sm[];   // [GA_KT keys][ld] then [GA_HW queries][ld]
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, u = lane >> 2, qt = lane & 3;
+    const int split = (int) blockIdx.x, t = (int) blockIdx.z, r = a.r, kw = r + rope, ld = kw + 4, nl = (r + 63) / 64;
+    const int h = (int) blockIdx.y * GA_HW + wv;
     const bool live = h < a.n_head;
-    float q[MLA_MAXL], acc[MLA_MAXL], qp[2];
-    const float* qlh = ql + ((size_t) t * a.n_head + (live ? h : 0)) * r;
-    const float* qrh = qr + ((size_t) t * a.n_head + (live ? h : 0)) * rope;
-#pragma unroll
-    for (int j = 0; j < MLA_MAXL; ++j) {
-        q[j] = j < nl && lane + 64 * j < r ? qlh[lane + 64 * j] * a.scale : 0.0f;
-        acc[j] = 0.0f;
+    float* keys = sm;
+    float* qs = sm + GA_KT * ld + wv * ld;
+    for (int i = lane; i < kw; i += 64) {   // the wave's query, scaled (its own rows of LDS: no barrier needed before the wave reads them)
+        const int hh = live ? h : 0;
+        qs[i] = a.scale * (i < r ? ql[((size_t) t * a.n_head + hh) * r + i] : qr[((size_t) t * a.n_head + hh) * rope + (i - r)]);
     }
+    int p0, p1;
+    split_range(a, ri[t].pos, split, &p0, &p1);
+    const int q0 = qt * (kw / 4), q1 = q0 + kw / 4;   // kw % 8 == 0: whole pairs
+    float acc[MLA_MAXL];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) qp[j] = lane + 64 * j < rope ? qrh[lane + 64 * j] * a.scale : 0.0f;
+    for (int j = 0; j < MLA_MAXL; ++j) acc[j] = 0.0f;
     float m = -INFINITY, l = 0.0f;
-    for (int p = p0; p < p1; p += MLA_KU) {
-        const int nk = min(MLA_KU, p1 - p);
+    for (int p = p0; p < p1; p += GA_KT) {
+        const int nk = min(GA_KT, p1 - p);
         __syncthreads();
-        for (int e = tid; e < nk * (kw / 8); e += ntg) {   // 8 dims at a time (r and rope: multiples of 8)
-            const int u = e / (kw / 8), d = (e - u * (kw / 8)) * 8;
+        for (int e = tid; e < nk * (kw / 8); e += 64 * GA_HW) {   // 8 dims a thread (r and rope are multiples of 8)
+            const int ku = e / (kw / 8), d = (e - ku * (kw / 8)) * 8;
             int row;
-            const KvSeg sg = kv_seg(kv, ri[t].kv0 + p + u, &row);
+            const KvSeg sg = kv_seg(kv, ri[t].kv0 + p + ku, &row);
             float v[8];
             if (d < r) cache_get8(kv.fmt, sg.v, sg.vs, (size_t) row, r, d, v);
             else cache_get8(kv.fmt, sg.k, sg.ks, (size_t) row, rope, d - r, v);
-            float* dst = sh + u * kw + d;
+            float* dst = keys + ku * ld + d;
             *(float4*) dst = make_float4(v[0], v[1], v[2], v[3]);
             *(float4*) (dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
         }
         __syncthreads();
-        float s[MLA_KU];
-        float mx = m;
-#pragma unroll
-        for (int u = 0; u < MLA_KU; ++u) {
-            float d = 0.0f;
-            if (u < nk) {
-                const float* kk = sh + u * kw;
-#pragma unroll
-                for (int j = 0; j < MLA_MAXL; ++j)
-                    if (j < nl && lane + 64 * j < r) d = fmaf(q[j], kk[lane + 64 * j], d);
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (lane + 64 * j < rope) d = fmaf(qp[j], kk[r + lane + 64 * j], d);
+        float sc = 0.0f;
+        if (u < nk) {
+            const float* kr_ = keys + u * ld;
+            for (int i = q0; i < q1; i += 2) {
+                const float2 kk = *(const float2*) (kr_ + i), qq = *(const float2*) (qs + i);
+                sc = fmaf(qq.x, kk.x, sc);
+                sc = fmaf(qq.y, kk.y, sc);
             }
-            for (int o = 32; o > 0; o >>= 1) d += __shfl_xor(d, o);
-            s[u] = u < nk ? d : -INFINITY;
-            mx = fmaxf(mx, s[u]);
         }
-        const float cor = expf(m - mx);
-        l *= cor;
+        sc += __shfl_xor(sc, 1);
+        sc += __shfl_xor(sc, 2);
+        if (u >= nk) sc = -INFINITY;
+        float mx = sc;
+        for (int o = 4; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+        mx = fmaxf(mx, m);
+        const float cor = expf(m - mx), e = expf(sc - mx);   // exp(-inf) = 0: keys past the run, and the first tile's m
+        float es = e;
+        for (int o = 4; o < 64; o <<= 1) es += __shfl_xor(es, o);
+        l = fmaf(l, cor, es);
+        m = mx;
 #pragma unroll
         for (int j = 0; j < MLA_MAXL; ++j) acc[j] *= cor;
 #pragma unroll
-        for (int u = 0; u < MLA_KU; ++u) {
-            if (u >= nk) break;
-            const float e = expf(s[u] - mx);
-            l += e;
-            const float* kk = sh + u * kw;
+        for (int ku = 0; ku < GA_KT; ++ku) {
+            const float ek = __shfl(e, 4 * ku);
+            if (ku >= nk) break;   // uniform
+            const float* kr_ = keys + ku * ld;
 #pragma unroll
             for (int j = 0; j < MLA_MAXL; ++j)
-                if (j < nl && lane + 64 * j < r) acc[j] = fmaf(e, kk[lane + 64 * j], acc[j]);
+                if (j < nl && lane + 64 * j < r) acc[j] = fmaf(ek, kr_[lane + 64 * j], acc[j]);
         }
-        m = mx;
     }
     if (!live) return;
     if (a.n_splits == 1) {
@@ -364,10 +391,9 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
     f32x4* Sx = (f32x4*) (Vt + R * MA_KB);   // [wave][lane]: the waves' partial score tiles
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const int split = (int) blockIdx.x, t = (int) blockIdx.z, h = (int) blockIdx.y * 16 + c;
-    const int pos = ri[t].pos, kv0 = ri[t].kv0, ns = mla_row_splits(a, pos);
-    const int nsr = min(ns, (pos + a.chunk) / a.chunk);
-    const int chunk = (pos + nsr) / nsr;
-    const int p0 = split * chunk, p1 = split < nsr ? min(pos + 1, p0 + chunk) : p0;
+    const int pos = ri[t].pos, kv0 = ri[t].kv0;
+    int p0, p1;
+    split_range(a, pos, split, &p0, &p1);
     const bool live = h < a.n_head;
 #ifdef NSLM_MLA_DEV   // development builds only: a.pad[1] switches parts of the tile loop off (1 loads, 2 decode, 4 scores, 8 P c)
     const int abl = a.pad[1];
@@ -808,8 +834,7 @@ void kc_mla_rope(kc_stream_t s, MlaArgs a, float* qr, const float* kr, const flo
                  int T) {
     const int rope = rope_of(a);
     if (T < 1 || (kv.fmt != KV_BF16 && kv.fmt != KV_FP8) || (rope != 64 && rope != 128) || a.r % 32) { host_note_unsupported(); return; }
-    const int nx = (a.n_head + 1) * (rope / 2) > a.r ? (a.n_head + 1) * (rope / 2) : a.r;
-    hipLaunchKernelGGL(k_mla_rope, dim3((unsigned) (nx + 63) / 64, (unsigned) T), dim3(64), 0, (hipStream_t) s, a, rope, qr, kr, c, kv, ri, inv);
+    hipLaunchKernelGGL(k_mla_rope, dim3((unsigned) T), dim3(256), 0, (hipStream_t) s, a, rope, qr, kr, c, kv, ri, inv);
     host_note_launch();
 }
 int kc_mla_qmaps_rope(kc_stream_t s, MlaArgs a, HmvArgs hq, HmvArgs hl, int fmt, WSlice Wq, WSlice Wl, const float* q, float* qr, float* ql,
@@ -820,8 +845,7 @@ int kc_mla_qmaps_rope(kc_stream_t s, MlaArgs a, HmvArgs hq, HmvArgs hl, int fmt,
     if (T < 1 || (kv.fmt != KV_BF16 && kv.fmt != KV_FP8) || (rope != 64 && rope != 128) || a.r % 64 || hq.O != rope || hl.O != a.r || hq.I != hl.I ||
         hq.I % 8 || hq.I / 8 > 64 || lpr != hq.I / 8 || hq.H != a.n_head || hl.H != a.n_head || hq.gate || hl.gate || hq.xs != hl.xs || hq.hs != hl.hs)
         return -1;
-    const int nx = (a.n_head + 1) * (rope / 2) > a.r ? (a.n_head + 1) * (rope / 2) : a.r;
-    const int bx = 1 + a.r / 64 > (nx + 255) / 256 ? 1 + a.r / 64 : (nx + 255) / 256;
+    const int bx = 1 + a.r / 64;   // >= the cache jobs' blocks: (1 + r / 64 + 3) / 4
     hipLaunchKernelGGL(k_qmaps_rope, dim3((unsigned) bx, (unsigned) a.n_head + 1, (unsigned) T), dim3(256), 0, (hipStream_t) s, a, rope, hq, hl, fmt,
                        Wq, Wl, q, qr, ql, kr, c, kv, ri, inv, lpr);
     host_note_launch();
@@ -846,11 +870,14 @@ static bool mla_attn_launch(kc_stream_t s, MlaArgs a, const float* ql, const flo
         const dim3 grid((unsigned) a.n_splits, (unsigned) (a.n_head + 15) / 16, (unsigned) T);
         if (kv.fmt == KV_FP8) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_FP8>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
         else hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_BF16>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
-    } else if (a.n_head > 8)
-        hipLaunchKernelGGL(k_mla_attn<16>, dim3((unsigned) a.n_splits, (unsigned) (a.n_head + 15) / 16, (unsigned) T), dim3(1024), 0, (hipStream_t) s,
-                           a, rope, ql, qr, kv, ri, o);
-    else
-        hipLaunchKernelGGL(k_mla_attn<8>, dim3((unsigned) a.n_splits, 1, (unsigned) T), dim3(512), 0, (hipStream_t) s, a, rope, ql, qr, kv, ri, o);
+    } else {
+        const size_t lds = sizeof(float) * (size_t) (GA_KT + GA_HW) * (size_t) (a.r + rope + 4);
+        static const hipError_t once = hipFuncSetAttribute((const void*) k_mla_attn_any, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                           (int) (sizeof(float) * (GA_KT + GA_HW) * (64 * MLA_MAXL + ATT_HD + 4)));
+        (void) once;
+        hipLaunchKernelGGL(k_mla_attn_any, dim3((unsigned) a.n_splits, (unsigned) (a.n_head + GA_HW - 1) / GA_HW, (unsigned) T), dim3(64 * GA_HW), lds,
+                           (hipStream_t) s, a, rope, ql, qr, kv, ri, o);
+    }
     if (a.n_splits > 1 && reduce)
         hipLaunchKernelGGL(k_mla_reduce, dim3((unsigned) a.n_head, (unsigned) T, (unsigned) (a.r + 127) / 128), dim3(128), 0, (hipStream_t) s, a, ri,
                            part, olat);
