@@ -1,5 +1,6 @@
-"""ctypes bindings of the gfx950 library: libnslm_hip.so (kc_* / kq4_* kernels and the nh_* runtime layer) and
-libnslm_kt.so (the C99 kernel-test backend, kt_*).  There is no CPU fallback: a missing library or GPU raises."""
+"""ctypes bindings of the gfx950 libraries: libnslm_hip.so (kc_* / kq4_* kernels and the nh_* runtime layer), libnslm_host.so
+(the C99 host side: nslm_moe_*, nslm_model_*, nsf_*) and, for tests, tests/kt/libnslm_kt.so (the kernel-test binding, kt_*).
+There is no CPU fallback: a missing library or GPU raises."""
 import ctypes as C
 import os
 import subprocess
@@ -11,7 +12,8 @@ from . import packs
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 HIP_SO = os.path.join(HERE, "libnslm_hip.so")
-KT_SO = os.path.join(HERE, "libnslm_kt.so")
+HOST_SO = os.path.join(HERE, "libnslm_host.so")
+KT_SO = os.path.join(os.path.dirname(HERE), "tests", "kt", "libnslm_kt.so")
 
 
 class WSlice(C.Structure):
@@ -81,6 +83,7 @@ def build(force=False):
 
 _hip = None
 _kt = None
+_host = None
 
 
 def hip():
@@ -96,8 +99,20 @@ def hip():
     return _hip
 
 
+def host():
+    """libnslm_host.so, the C99 host side (MoE layer, model step, model folder; links libnslm_hip.so); raises when missing."""
+    global _host
+    if _host is None:
+        hip()
+        if not os.path.exists(HOST_SO):
+            raise RuntimeError(f"{HOST_SO} is missing: build it with nanoseedlm_amd.backend.build()")
+        _host = C.CDLL(HOST_SO)
+    return _host
+
+
 def kt():
-    """libnslm_kt.so (links libnslm_hip.so); raises when missing."""
+    """tests/kt/libnslm_kt.so, the kernel-test binding (kt_*: host arrays in, one kc_* call, host arrays out; links
+    libnslm_hip.so).  Test infrastructure, not part of the product libraries; raises when missing."""
     global _kt
     if _kt is None:
         hip()

@@ -414,9 +414,6 @@ struct MmRec2 {
 #define MM_STAMP(t, step, slot) do { } while (0)
 #define MM_WG_STAMP(t, slot) do { } while (0)
 #endif
-#ifndef NSLM_MM_ABLATE   // development builds only: 1 no activation loads, 2 no decode, 4 no MFMA
-#define NSLM_MM_ABLATE 0
-#endif
 template <int CT, int NCW, int XCH, int FMT>
 __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice wd, const WSlice* ws, const uint16_t* X, float* Y,
                                                    const int32_t* perm, const MmTile* tiles, const int32_t* ntiles) {
@@ -504,10 +501,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         auto produce = [&](int s, const MmRec2& r, const Look& k) {
             float f[2][8];   // rows past R decode their zeroed records: harmless, their outputs are never stored
             {
-                if (NSLM_MM_ABLATE & 2) {
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) f[0][c] = f[1][c] = __uint_as_float(r.u);
-                } else if (seedf) {
+                if (seedf) {
                     const uint32_t up[2] = {r.u << 16, r.u}, word[2] = {r.v & 0xFFFFu, r.v >> 16};
                     int is[2][8];
                     if (FMT == MF_SEED4P4) isum2_p4(up, k.g, k.qa, k.qb, is);
@@ -600,7 +594,6 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     }
     uint16_t* ring = Xs + wv * (XCH * XCHUNK);
     auto fetch = [&](int sf, int mf, int slot) {   // chunk (sf, mf) -> ring slot (past the end: a harmless reload of the last step)
-        if (NSLM_MM_ABLATE & 1) return;
         const char* src = (const char*) X + (size_t) min(sf, nsteps - 1) * WK * 2;
         uint16_t* dst = ring + slot * XCHUNK;
 #pragma unroll
@@ -635,7 +628,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
             for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
                 for (int n = 0; n < 2; ++n)
-                    if (!(NSLM_MM_ABLATE & 4)) acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(((m & 1) ? fb : fa)[kk], bq[kk][n], acc[m][n], 0, 0, 0);
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(((m & 1) ? fb : fa)[kk], bq[kk][n], acc[m][n], 0, 0, 0);
             MM_STAMP(0, s, 2 + m);
         }
     };

@@ -27,7 +27,7 @@ class Tensor(C.Structure):
 
 
 def _lib():
-    L = backend.kt()
+    L = backend.host()
     L.nsf_open.restype = C.c_void_p
     L.nsf_at.restype = C.POINTER(Tensor)
     L.nsf_find.restype = C.POINTER(Tensor)

@@ -1,5 +1,5 @@
 """Host mirror of csrc/decode_model.h: a whole synthetic seeded-MoE model's greedy decode on the gfx950 kernels
-(the benchmark's full-model configuration).  ctypes only; every launch goes through libnslm_kt.so / libnslm_hip.so."""
+(the benchmark's full-model configuration).  ctypes only; every launch goes through libnslm_host.so / libnslm_hip.so."""
 import ctypes as C
 
 import numpy as np
@@ -22,7 +22,7 @@ def _p(a):
 
 class DecodeModel:
     def __init__(self, **kw):
-        self.L = backend.kt()
+        self.L = backend.host()
         self.cfg = ModelCfg(**kw)
         err = C.create_string_buffer(256)
         self.L.nslm_model_open.restype = C.c_void_p

@@ -15,7 +15,7 @@ class NslmMoeCfg(C.Structure):
 
 
 def _lib():
-    L = backend.kt()
+    L = backend.host()
     L.nslm_moe_open.restype = C.c_void_p
     L.nslm_graph_end.restype = C.c_void_p
     L.nslm_moe_tab.restype = C.c_void_p

@@ -17,7 +17,7 @@ def declared(header):
 @pytest.fixture(scope="module")
 def libs():
     from nanoseedlm_amd import backend
-    if not os.path.exists(backend.HIP_SO) or not os.path.exists(backend.KT_SO):
+    if not os.path.exists(backend.HIP_SO) or not os.path.exists(backend.KT_SO) or not os.path.exists(backend.HOST_SO):
         backend.build()
     return backend
 
@@ -40,12 +40,15 @@ def test_struct_layouts_match_the_reference_abi(libs):
 
 def test_kt_backend_exports(libs):
     K = libs.kt()
-    txt = open(os.path.join(ROOT, "nanoseedlm_amd", "csrc", "kernel_backend.h")).read()
+    txt = open(os.path.join(ROOT, "tests", "kt", "kernel_backend.h")).read()
     txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
     for n in set(re.findall(r"\b(kt_\w+)\s*\(", txt)):
         assert hasattr(K, n), n
     assert K.kt_name() == b"HIP gfx950" and K.kt_mm_tile() == 128
-    for h in ("moe_layer.h", "decode_model.h"):                        # the layer and whole-model hosts live in the same library
+    assert not hasattr(K, "nslm_moe_open")                             # the test binding holds no product code ...
+    K = libs.host()
+    assert not hasattr(K, "kt_mv")                                     # ... and the host library no test binding
+    for h in ("moe_layer.h", "decode_model.h"):                        # the layer and whole-model hosts
         txt = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "nanoseedlm_amd", "csrc", h)).read(), flags=re.S)
         names = set(re.findall(r"\b(nslm_\w+)\s*\(", txt))
         assert len(names) > 8

@@ -85,7 +85,7 @@ def test_upload_of_a_stream_longer_than_the_staging_buffers(tmp_path):
     mf = folder.ModelFolder(tmp_path)
     t = mf.find("big.weight")
     assert t.s[0].len == big.nbytes
-    K = backend.kt()
+    K = backend.host()
     K.nsf_upload.argtypes = [C.c_void_p, C.POINTER(folder.Stream), C.c_uint64, C.c_uint64]
     raw = big.view(np.uint8).reshape(-1)
     for skip, n in ((0, big.nbytes), (12345, 17 * 1024 * 1024 + 77), (big.nbytes - 5, 5)):

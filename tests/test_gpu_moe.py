@@ -120,7 +120,7 @@ def test_whole_expert_block_in_one_launch(T):
     import ctypes as C
     from nanoseedlm_amd import backend, moe
     backend.require_gpu()
-    L, K = backend.hip(), backend.kt()
+    L, K = backend.hip(), backend.host()
     rng = np.random.default_rng(77 + T)
     E, k, d, ff = 16, 4, 256, 128
     st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=32)

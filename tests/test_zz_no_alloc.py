@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 def test_static_scratch_step_equals_workspace_step():
     from nanoseedlm_amd import backend, moe
     backend.require_gpu()
-    L, K = backend.hip(), backend.kt()
+    L, K = backend.hip(), backend.host()
     rng = np.random.default_rng(321)
     E, k, d, ff = 16, 4, 256, 128
     st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=32)
