@@ -33,13 +33,31 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def traffic_of(workload):
-    """HBM bytes per launch of the workload's dominant kernel, from the committed rocprofv3 --pmc summary (or None)."""
+COUNTERS = "profiles/traffic.json"
+
+
+def counters_of(workload):
+    """What the committed rocprofv3 --pmc summaries hold for the workload's dominant kernel: HBM bytes per launch and the share
+    of the kernel's time its vector ALUs were busy.  Constants of an earlier profiled run of the same command, not measurements
+    of this run: the JSON line says so (traffic_source)."""
     try:
-        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")) as f:
-            return json.load(f).get(workload, {}).get("hbm_bytes_per_launch")
+        with open(os.path.join(ROOT, COUNTERS)) as f:
+            e = json.load(f).get(workload, {})
     except OSError:
-        return None
+        e = {}
+    return dict(traffic=e.get("hbm_bytes_per_launch"), traffic_source=COUNTERS if e.get("hbm_bytes_per_launch") else None,
+                valu_busy=e.get("valu_busy_pct") / 100.0 if e.get("valu_busy_pct") is not None else None,
+                valu_busy_source=COUNTERS if e.get("valu_busy_pct") is not None else None)
+
+
+def fail_on_kernel_error(st=None):
+    """A launch error, or a wait inside the persistent MoE kernel that gave up (its results are void): no throughput is printed."""
+    from nanoseedlm_amd import backend
+    err = backend.hip().kc_last_error()
+    if err:
+        sys.exit(f"bench.py: a kernel launch failed ({err}); no result")
+    if st is not None and st.fused_error():
+        sys.exit("bench.py: a wait between workgroups of the persistent MoE kernel gave up (error word set); no result")
 
 
 class Q4Projections:
@@ -166,6 +184,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     moe.device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms = e1.ms_since(e0) / steps
+    fail_on_kernel_error(st)
 
     # bytes: unique selected experts x expert bytes + the BF16 router weight; at batch 1 every pair is unique
     uniq = []
@@ -174,6 +193,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         st.step(stream, l, xs[xi].ptr, T, out.ptr)
         ind, _ = st.last_routing(T)
         uniq.append(len(set(ind.reshape(-1).tolist())))
+    fail_on_kernel_error(st)
     eb = st.expert_bytes()
     bytes_step = float(np.mean(uniq)) * eb + E * d * 2 + (q4.bytes_per_layer if q4 else 0)
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T,
@@ -210,18 +230,18 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         # Its launch duration is the step's event time: HIP events over the timed region on the launch stream (launches are
         # queued back to back, so there is no gap between them unless the step is wrapped in a graph).
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=traffic_of(name), kernel="k_moe_decode (one launch per step)",
-                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part)
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_moe_decode (one launch per step)",
+                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part, **counters_of(name))
         ind.free(); A.free()
     else:
         # Batched steps: 9 to 24 rows of C2 are one launch of the grouped persistent kernel; beyond that (and for C3) three
         # grouped GEMM launches over tiles of a few pairs each dominate, and what they spend is the records' expansion, not
         # matrix flops: priced against HBM on the records the step has to read.
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=None,
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
                                kernel=("k_moe_decode_grouped (one launch per step)" if T <= 24 and name[:2] == "c2" else
                                        "k_mm_stream<1, 4, 3> grouped (three launches of the step, with its glue kernels)"),
-                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
+                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, **counters_of(name))
     desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",
             "c3": "C3 mixed-format layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880 Q4-g64 projections (q, k, v, o, shared gate / up / down)"}[name[:2]]
     res["config"] = {"workload": f"{desc}, batch {T}", "layers_rotated": n_layers, "inputs_rotated": NX,
@@ -272,7 +292,8 @@ def model_workload(name, steps, warmup, no_graph, branches=False, splits=32):
     moe.device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms = e1.ms_since(e0) / steps
-    ids, logits = m.ids(T), m.logits(T)
+    ids, logits = m.ids(T), m.logits(T)           # (both raise when the persistent MoE kernel's error word is set)
+    fail_on_kernel_error()
     if not np.isfinite(logits).all():
         raise RuntimeError("the synthetic model's logits are not finite")
     # bytes a step has to read: weight records (top-k experts per row; rows of a batch share some, counted once from the
@@ -290,7 +311,7 @@ def model_workload(name, steps, warmup, no_graph, branches=False, splits=32):
     flops = 2.0 * T * (m.step_bytes() - 2 * cfg["vocab"] * cfg["d"]) / 4.5 * 8 + 2.0 * T * cfg["vocab"] * cfg["d"]
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
     res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s", frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
-                           traffic=None, kernel="whole decode step (k_moe_decode x 24 is the largest share)" if T <= 8 else
+                           traffic=None, traffic_source=None, kernel="whole decode step (k_moe_decode x 24 is the largest share)" if T <= 8 else
                            "whole decode step (grouped k_mm_stream launches are the largest share)",
                            launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
     res["config"] = {"workload": f"C4 full synthetic model greedy decode: 24 layers, hidden 2048, MLA 16 heads (latent 512 + rope 64, FP8 cache), "
@@ -355,16 +376,16 @@ def dense_workload(name, steps, warmup):
     moe.device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms = e1.ms_since(e0) / steps
-    backend.check(L.kc_last_error(), "kernel launch")
+    fail_on_kernel_error()
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
     if bound == "hbm":
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, traffic=None, kernel="k_mv_seed<dense>",
-                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_mv_seed<dense>",
+                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, **counters_of(name))
     else:
         res["roofline"] = dict(bound="mfma", achieved=flops / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                               frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, traffic=traffic_of(name), kernel="k_mm_stream<2, 8> (BF16 activations, 512-token tile)",
-                               launch_us=ms * 1e3, algorithmic_flops=flops)
+                               frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, kernel="k_mm_stream<2, 8> (BF16 activations, 512-token tile)",
+                               launch_us=ms * 1e3, algorithmic_flops=flops, **counters_of(name))
     res["config"] = {"workload": desc, "launch": "stream"}
     res["cpu_sample"] = sample
     return res

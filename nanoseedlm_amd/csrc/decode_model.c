@@ -422,6 +422,11 @@ int nslm_model_ids(NslmModel* m, int T, int32_t* ids) {
 int nslm_model_logits(NslmModel* m, int T, float* logits) {
     return nh_device_sync() || nh_memcpy_d2h(logits, m->logits, 4 * (size_t) T * m->c.vocab) || nslm_moe_fused_error(m->moe) ? -1 : 0;
 }
+int nslm_model_hidden(NslmModel* m, int T, float* h) { return nh_device_sync() || nh_memcpy_d2h(h, m->xn, 4 * (size_t) T * m->c.d) ? -1 : 0; }
+int nslm_model_get_embed(NslmModel* m, int first, int rows, uint16_t* w) {
+    if (first < 0 || rows < 0 || first + rows > m->c.vocab) return -1;
+    return nh_device_sync() || nh_memcpy_d2h(w, m->embed + (size_t) first * m->c.d, 2 * (size_t) rows * m->c.d) ? -1 : 0;
+}
 uint64_t nslm_model_step_bytes(const NslmModel* m) {
     const NslmModelCfg* c = &m->c;
     uint64_t b = 0;

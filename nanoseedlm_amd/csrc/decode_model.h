@@ -71,6 +71,10 @@ int nslm_model_account(NslmModel* m, int steps);
  * kernel gave up since open (the results are void then) */
 int nslm_model_ids(NslmModel* m, int T, int32_t* ids);
 int nslm_model_logits(NslmModel* m, int T, float* logits);
+/* for tests (both synchronise): the last step's final hidden rows [T][d] after the closing norm - what the LM head multiplies -
+ * and rows [first, first + rows) of the BF16 embedding / LM-head matrix */
+int nslm_model_hidden(NslmModel* m, int T, float* h);
+int nslm_model_get_embed(NslmModel* m, int first, int rows, uint16_t* w);
 /* compressed weight bytes one decode step of one token reads: experts selected + shared expert + dense + maps + LM head */
 uint64_t nslm_model_step_bytes(const NslmModel* m);
 

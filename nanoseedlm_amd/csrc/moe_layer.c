@@ -310,6 +310,10 @@ int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {
     if (nh_device_sync()) return -1;
     return (nh_memcpy_d2h(ind, m->ind, 4 * (size_t) T * m->c.top_k) | nh_memcpy_d2h(wt, m->wt, 4 * (size_t) T * m->c.top_k)) ? -1 : 0;
 }
+int nslm_moe_last_pairs(NslmMoe* m, int pairs, float* A, float* D) {
+    if (nh_device_sync()) return -1;
+    return (nh_memcpy_d2h(A, m->A, 4 * (size_t) pairs * m->c.ff) | nh_memcpy_d2h(D, m->D, 4 * (size_t) pairs * m->c.d)) ? -1 : 0;
+}
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses) {
     uint32_t st[2] = {0, 0};
     if (nh_device_sync() || nh_memcpy_d2h(st, m->pool.stats, 8)) return -1;

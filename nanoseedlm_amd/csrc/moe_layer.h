@@ -55,6 +55,10 @@ void nslm_moe_set_fused(NslmMoe* m, int on);
 int nslm_moe_fused_error(NslmMoe* m);
 /* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
+/* the last step's intermediates per (token, expert) pair, copied to the host (synchronises): A [pairs][ff] = the SwiGLU outputs
+ * the down projections read, D [pairs][d] = the experts' outputs the combine sums.  Pair t * top_k + j of nslm_moe_step (the
+ * batched path's A is the packed BF16 view: read it as uint16 [pairs][ff] in the first half of the buffer). */
+int nslm_moe_last_pairs(NslmMoe* m, int pairs, float* A, float* D);
 /* the slot table's counters and state (synchronises): hits, misses since open */
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
 /* the device slice table [n_exp] of a layer's tensor (0 gate, 1 up, 2 down): what kc_mv_gu / kc_mv_sel take */

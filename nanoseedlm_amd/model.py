@@ -110,5 +110,15 @@ class DecodeModel:
         backend.check(self.L.nslm_model_logits(self.h, T, _p(out)), "nslm_model_logits")
         return out
 
+    def hidden(self, T):
+        out = np.zeros((T, self.cfg.d), dtype=np.float32)
+        backend.check(self.L.nslm_model_hidden(self.h, T, _p(out)), "nslm_model_hidden")
+        return out
+
+    def embed_rows(self, first, rows):
+        out = np.zeros((rows, self.cfg.d), dtype=np.uint16)
+        backend.check(self.L.nslm_model_get_embed(self.h, first, rows, _p(out)), "nslm_model_get_embed")
+        return out
+
     def step_bytes(self):
         return int(self.L.nslm_model_step_bytes(self.h))

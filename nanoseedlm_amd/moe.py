@@ -123,6 +123,15 @@ class MoeStack:
             raise RuntimeError("nslm_moe_last_routing failed")
         return ind, wt
 
+    def last_pairs(self, pairs):
+        """The last step's per-pair intermediates: A [pairs][ff] (SwiGLU outputs; uint16 BF16 bits in the batched path's packed
+        layout are returned as the raw f32 buffer - see moe_layer.h) and D [pairs][d] (expert outputs)."""
+        A = np.zeros((pairs, self.cfg.ff), dtype=np.float32)
+        D = np.zeros((pairs, self.cfg.d), dtype=np.float32)
+        if self.L.nslm_moe_last_pairs(self.h, pairs, A.ctypes.data_as(C.c_void_p), D.ctypes.data_as(C.c_void_p)):
+            raise RuntimeError("nslm_moe_last_pairs failed")
+        return A, D
+
     def cache_stats(self):
         h, m = C.c_uint32(0), C.c_uint32(0)
         if self.L.nslm_moe_cache_stats(self.h, C.byref(h), C.byref(m)):
