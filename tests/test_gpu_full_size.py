@@ -102,6 +102,9 @@ def test_c2_layer_step_128_experts(oracle, T):
         want = (wt[t].astype(np.float64)[:, None] * ys).sum(0)
         tol = 2e-2 * np.abs(wt[t].astype(np.float64)[:, None] * ys).sum(0) + 1e-6
         assert np.all(np.abs(out[t] - want) <= tol)
+        assert np.max(np.abs(out[t] - want)) / np.max(np.abs(want)) < 2e-3
+    A, D = st.last_pairs(T * k)
+    check_stages(oracle, gate, up, down, xn, ind, wt, A, D, out, sorted({0, T - 1}), gemm=False)
     # the same step through the five separate launchers: the same bits
     st.set_fused(0)
     dio2 = moe.DevBuf(4 * T * d)
@@ -144,7 +147,7 @@ def end_to_end(oracle, gate, up, down, xn, ind, wt, out, tokens, gemm):
         terms = wt[t].astype(np.float64)[:, None] * ys
         want = terms.sum(0)
         assert np.all(np.abs(out[t] - want) <= 2e-2 * np.abs(terms).sum(0) + 1e-6), t
-        assert np.max(np.abs(out[t] - want)) / np.max(np.abs(want)) < 2e-3, t       # the stated bar, as a max-rel-err
+        assert np.max(np.abs(out[t] - want)) / np.max(np.abs(want)) < (1e-2 if gemm else 2e-3), t   # the stated bars (BF16 MFMA / fp32), as a max-rel-err
 
 
 def test_c2_layer_step_32_tokens_bucket_and_grouped_gemm(oracle):

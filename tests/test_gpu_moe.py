@@ -103,7 +103,11 @@ def test_moe_step(oracle, router, T, slots):
                         s = (s + r((ys[j] * float(r(wt[t, j]))).astype(np.float32))).astype(np.float32)
                     want = r(x0[t] + r(r(s) + 0.0)).astype(np.float64)
                     tol = 2e-2 * (np.abs(x0[t]) + np.abs(ys).sum(0) * np.abs(wt[t]).max()) + 1e-6
+                # Elementwise the bound is 2e-2 of the summed magnitudes: G, U, A, D are rounded to BF16 at the reference's rounding
+                # points, and a sum next to a rounding boundary may round the other way on the GPU (one BF16 ulp = 2^-8 of the
+                # value).  As a max-rel-err (the form of the stated 2e-3 bar) such flips average out over the down projection.
                 assert np.all(np.abs(out[t] - want) <= tol), (rep, l, t, np.max(np.abs(out[t] - want) / tol))
+                assert np.max(np.abs(out[t] - want)) / np.max(np.abs(want)) < (1e-2 if gemm else 2e-3), (rep, l, t)   # MFMA / fp32 bar
     hits, misses = st.cache_stats()
     if slots == 0:
         assert (hits, misses) == (0, 0)          # all resident: the table is never consulted
