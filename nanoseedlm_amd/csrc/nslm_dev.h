@@ -103,6 +103,34 @@ __device__ __forceinline__ void load_tables(uint32_t* tab) {
     for (int i = threadIdx.x; i < 512; i += blockDim.x) tab[i] = kBasis.v[i];
     for (int i = threadIdx.x; i < 256; i += blockDim.x) tab[512 + i] = kPairs.v[i];
 }
+// The same for a workgroup of exactly NTHR threads (256, 512 or 1024), in two halves: a thread's loads are requested in
+// tables_fetch() (put it beside the kernel's other first loads), and tables_store() writes them to LDS once they are needed -
+// the loop above waits for every load in turn, one memory round trip each.
+template <int NTHR>
+struct TableWords {
+    uint32_t w[(NSLM_TAB_WORDS + NTHR - 1) / NTHR];
+};
+template <int NTHR>
+__device__ __forceinline__ TableWords<NTHR> tables_fetch() {
+    TableWords<NTHR> t;
+#pragma unroll
+    for (int j = 0; j < (NSLM_TAB_WORDS + NTHR - 1) / NTHR; ++j) {
+        const int i = min((int) threadIdx.x + NTHR * j, NSLM_TAB_WORDS - 1);   // clamped: the loads stay unconditional
+        t.w[j] = i < 512 ? kBasis.v[i] : kPairs.v[i - 512];
+    }
+    return t;
+}
+template <int NTHR>
+__device__ __forceinline__ void tables_store(uint32_t* tab, const TableWords<NTHR>& t) {
+#pragma unroll
+    for (int j = 0; j < (NSLM_TAB_WORDS + NTHR - 1) / NTHR; ++j) {
+        const int i = (int) threadIdx.x + NTHR * j;
+        if (i < NSLM_TAB_WORDS) tab[i] = t.w[j];
+    }
+}
+// keeps the loads written above this line above it: left alone, the compiler moves a load down to its first use, and a load
+// whose use sits in a conditional block becomes a load, a wait and a branch - one round trip per load instead of one for all
+__device__ __forceinline__ void loads_issued() { asm volatile("" ::: "memory"); }
 __device__ __forceinline__ uint32_t stream_of(const uint32_t* tab, uint32_t seed16) {
     return tab[seed16 & 0xFFu] ^ tab[256 + (seed16 >> 8)];
 }

@@ -45,19 +45,35 @@ struct MvArgs {
                           // added in the middle cost them a second round of argument loads, 0.3 us a launch)
 };
 #define MV_MAXJ 4
+#define MV_YBUF 1024   // virtual rows a workgroup takes at most (rpi <= 256 of them an iteration)
 
 enum { DENSE = 0, GATHER = 1, GATEUP = 2, MULTI = 3 };
 
+#ifdef NSLM_MV_STAMPS   // development builds only: wall-clock stamps of every workgroup
+__device__ unsigned long long g_mvstamp[8192 * 16];
+#define MV_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 8192) { g_mvstamp[blockIdx.x * 16 + (i)] = wall_clock64(); g_mvstamp[blockIdx.x * 16 + 8 + (i)] = clock64(); } } while (0)
+#else
+#define MV_STAMP(i) do { } while (0)
+#endif
 // SHFL: L is a power of two <= 64 (<= 32 for GATEUP): row sums by wave shuffles, no barrier.  Otherwise through LDS.
-template <int P, int MODE, int NT, bool SHFL>
-__global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
-    extern __shared__ float xl[];                  // NT > 1: activations [token][chunk][XPAD]
+// NTHR: threads a workgroup (256; 512 or 1024 for one-token SHFL launches whose rows fill more than four waves a CU - the
+// row and the tables are then fetched once per CU instead of once per four waves).
+template <int P, int MODE, int NT, bool SHFL, int NTHR = 256>
+__global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
+    static_assert(NTHR == 256 || (SHFL && NT == 1), "the LDS row sums and the staged multi-token passes are written for 256 threads");
+    extern __shared__ float xl[];                  // activations [token][chunk][XPAD]
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[SHFL ? 1 : 2][SHFL ? 1 : NT][SHFL ? 1 : 256];
     __shared__ float nred[4];
+    // The workgroup's results wait here until the loop is over and leave as coalesced stores.  A store inside the loop costs a
+    // memory round trip per iteration: the wait for the next records at the end of an iteration is a wait for every
+    // outstanding vector memory operation, the store of a moment ago included (C0: 3.5 us for the first of two
+    // iterations, 2.35 us - the arithmetic - for the second, which ends the kernel and waits for nothing).
+    __shared__ float ybuf[NT][MV_YBUF];
     const int tid = threadIdx.x, L = a.L, rpi = a.rpi;
     const int lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
+    MV_STAMP(0);
     constexpr bool DN = MODE == DENSE || MODE == MULTI;   // all tokens against one matrix
     const int pair = DN ? 0 : (int) blockIdx.y;
     int job = 0, wg = (int) blockIdx.x;
@@ -74,17 +90,32 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
     float* const yb = (MODE == MULTI ? a.yj[job] : a.y) + (size_t) tg0 * (MODE == MULTI ? a.ysj[job] : a.ys);
     const int V = MODE == GATEUP ? 2 * R : R;   // virtual rows: gate row r = 2r, up row r = 2r + 1
     const int v0 = wg * a.rows_per_wg, v1 = min(v0 + a.rows_per_wg, V);
+    const float* xrow = a.x + (size_t) (DN ? 0 : pair / a.xdiv) * a.xs;
+    // Request order = return order (a wave's loads come back in the order they went out): the tables and the row, which sit in
+    // L2 and are needed first, go out before the records, which come from HBM behind everybody else's.
+    const TableWords<NTHR> tw = tables_fetch<NTHR>();
+    const bool prenorm = MODE == MULTI && a.nw != nullptr;   // uniform; the other modes compile without it
+    float xreg[NT == 1 ? 64 : 1];
+    constexpr int NXQ = 2048 / NTHR;   // K <= 8192: at most 2048 16-byte pieces of a row
+    float4 xq[NT == 1 ? NXQ : 1], wq[NT == 1 ? NXQ : 1];
+    if (NT == 1) {   // clamped, so that the loads stay unconditional
+#pragma unroll
+        for (int j = 0; j < NXQ; ++j) {
+            const int i = min(tid + NTHR * j, a.K / 4 - 1);
+            xq[j] = ((const float4*) xrow)[i];
+            if (MODE == MULTI && prenorm) wq[j] = ((const float4*) a.nw)[i];
+        }
+    }
+    loads_issued();
     WSlice wA = MODE == MULTI ? a.wj[job] : a.wd, wB = wA;
     if (!DN) {
         const int sl = a.sel[pair];
         wA = a.ws[sl];
         if (MODE == GATEUP) wB = a.wu[sl];
     }
-    const float* xrow = a.x + (size_t) (DN ? 0 : pair / a.xdiv) * a.xs;
+    const bool al = true;
 
-    const bool al = streams_aligned(P, wA) && (MODE != GATEUP || streams_aligned(P, wB));
-
-    // first records in flight before anything else
+    // first records in flight before the first wait
     int v = v0 + lr;
     auto fetch = [&](int vv) {
         const bool ok = active && vv < v1;
@@ -93,40 +124,32 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
         return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
     };
     Chunk cur = fetch(v);
-
-    load_tables(tab);
-    const bool prenorm = MODE == MULTI && a.nw != nullptr;   // uniform; the other modes compile without it
-    float xreg[NT == 1 ? 64 : 1];
+    loads_issued();
+    MV_STAMP(5);
     if (NT == 1) {
-        // The row's scale first, while few registers are live (its 16 loads then go out back to back; issued beside the
-        // 128 registers of row and weight data the allocator serialised them), then the row and the norm weights together.
+        // The row goes through LDS once per workgroup and from there into each thread's registers (the 256 / L threads that
+        // share a chunk do not each fetch it).  Every load of the prologue - tables, row, records - is requested before the
+        // first wait, so the kernel starts after one memory round trip.
+        const int K4 = a.K / 4;
+        // (with a norm: the row's scale, bit for bit as the norm kernel forms it - a second pass over the row, from L2)
         const float rn = (MODE == MULTI && prenorm) ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
-        if (active) {
-            const float4* xp = (const float4*) (xrow + (size_t) ch * 64);
-            float4 wq[MODE == MULTI ? 16 : 1];
-            if (MODE == MULTI && prenorm) {
-                const float4* wp = (const float4*) (a.nw + (size_t) ch * 64);
+        tables_store<NTHR>(tab, tw);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) wq[i] = wp[i];
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float4 q = xp[i];
-                xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
-            }
-            if (MODE == MULTI && prenorm) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    xreg[4 * i] = xreg[4 * i] * rn * (1.0f + wq[i].x);
-                    xreg[4 * i + 1] = xreg[4 * i + 1] * rn * (1.0f + wq[i].y);
-                    xreg[4 * i + 2] = xreg[4 * i + 2] * rn * (1.0f + wq[i].z);
-                    xreg[4 * i + 3] = xreg[4 * i + 3] * rn * (1.0f + wq[i].w);
+        for (int j = 0; j < NXQ; ++j) {
+            const int i = tid + NTHR * j;
+            if (i < K4) {
+                float4 v4 = xq[j];
+                if (MODE == MULTI && prenorm) {
+                    v4.x = v4.x * rn * (1.0f + wq[j].x); v4.y = v4.y * rn * (1.0f + wq[j].y);
+                    v4.z = v4.z * rn * (1.0f + wq[j].z); v4.w = v4.w * rn * (1.0f + wq[j].w);
                 }
+                *(float4*) &xl[(i >> 4) * XPAD + (i & 15) * 4] = v4;
             }
         }
     } else {
         // Stage nt rows of K floats: 8 loads in flight a thread before the first store (a loop of load-then-store over a
         // run-time count waits for every load in turn).
+        tables_store<NTHR>(tab, tw);
         __shared__ float rn_s[NT];
         if (prenorm) {
             for (int t = 0; t < nt_; ++t) {
@@ -159,6 +182,14 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
         }
     }
     __syncthreads();
+    if (NT == 1 && active) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float4 q = *(const float4*) &xl[ch * XPAD + 4 * i];
+            xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
+        }
+    }
+    MV_STAMP(1);
 
     const int eA = wA.eb, eB = wB.eb;
     int par = 0;
@@ -183,11 +214,10 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                     const float other = __shfl_xor(s, L);   // rows 2r and 2r+1 sit side by side in the wave
                     if (active && ch == 0 && !(v & 1) && v < v1) {
                         const float gs = s * NSLM_R32, us = other * NSLM_R32;
-                        float* yo = yb + (size_t) pair * ys + (v >> 1);
-                        *yo = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
+                        ybuf[t][(v - v0) >> 1] = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                     }
                 } else if (active && ch == 0 && v < v1) {
-                    store_y(yb + (size_t) (DN ? t : pair) * ys + v, s * NSLM_R32, add, a.f32out);
+                    ybuf[t][v - v0] = s * NSLM_R32;
                 }
             }
         } else {
@@ -202,21 +232,33 @@ __global__ void __launch_bounds__(256) k_mv_seed(MvArgs a) {
                     for (int j = 0; j < L; ++j) us += part[par][0][(2 * tid + 1) * L + j];
                     gs *= NSLM_R32;
                     us *= NSLM_R32;
-                    float* yo = yb + (size_t) pair * ys + ((vb >> 1) + tid);
-                    *yo = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
+                    ybuf[0][((vb - v0) >> 1) + tid] = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                 }
             } else {
                 for (int w = tid; w < nrow * (NT > 1 ? nt_ : 1); w += 256) {   // (token, row) sums: more than 256 with many tokens of short rows
                     const int t = w / nrow, r = w - t * nrow;
                     float s = 0.0f;
                     for (int j = 0; j < L; ++j) s += part[par][t][r * L + j];
-                    store_y(yb + (size_t) (DN ? t : pair) * ys + (vb + r), s * NSLM_R32, add, a.f32out);
+                    ybuf[t][vb - v0 + r] = s * NSLM_R32;
                 }
             }
         }
         cur = nxt;
+        MV_STAMP(2 + min((vb - v0) / rpi, 4));
     }
+    __syncthreads();
+    const int nout = MODE == GATEUP ? (v1 - v0) >> 1 : v1 - v0, o0 = MODE == GATEUP ? v0 >> 1 : v0;
+    for (int w = tid; w < nout * (NT > 1 ? nt_ : 1); w += NTHR) {
+        const int t = w / nout, r = w - t * nout;
+        float* yo = yb + (size_t) (DN ? t : pair) * ys + (o0 + r);
+        if (MODE == GATEUP) *yo = ybuf[t][r];
+        else store_y(yo, ybuf[t][r], add, a.f32out);
+    }
+    MV_STAMP(7);
 }
+#ifdef NSLM_MV_STAMPS
+extern "C" int kc_mv_stamps(unsigned long long* host) { return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_mvstamp), sizeof(unsigned long long) * 8192 * 16); }
+#endif
 
 // ---- generic path: every format, one wave per row --------------------------------------------------------------------
 template <int MODE>
@@ -457,14 +499,25 @@ int cu_count() {
     return n;
 }
 
-// virtual rows per workgroup: a multiple of rpi, sized so the grid has about 3 workgroups per CU when the work allows
-int pick_rows_per_wg(int V, int rpi, int ny) {
+// virtual rows per workgroup: a multiple of rpi, sized so the grid has about 3 workgroups of 256 threads per CU (2 of 512, 1 of
+// 1024) when the work allows
+int pick_rows_per_wg(int V, int rpi, int ny, int nthr = 256) {
     const int iters = (V + rpi - 1) / rpi;
-    const int want = 3 * cu_count();
+    const int want = (nthr >= 1024 ? 1 : nthr >= 512 ? 2 : 3) * cu_count();
     int per = (iters * ny + want - 1) / want;
     if (per < 1) per = 1;
     if (per > 64) per = 64;
+    while (per > 1 && per * rpi > MV_YBUF) --per;   // a workgroup's results wait in LDS until its last iteration
     return per * rpi;
+}
+// Threads a workgroup for a one-token dense pass over V rows of L chunks: every workgroup fetches the activation row (K floats)
+// and the decode tables, and at the start of a launch those fills compete with the first records for the same path into the
+// CUs (C0: 512 workgroups of 256 threads brought in 8 MB of row copies beside 9.4 MB of records).  So a CU's share of the rows
+// goes to ONE workgroup when it is more than four waves' worth: 512 or 1024 threads.
+int pick_threads(int V, int L, bool shfl) {
+    if (!shfl || L > 64) return 256;
+    const long waves = ((long) V * L + 63) / 64, per_cu = (waves + cu_count() - 1) / cu_count();
+    return per_cu > 8 ? 1024 : per_cu > 4 ? 512 : 256;
 }
 
 // kernels that stage activations may need more dynamic LDS than the default limit: raise it once per kernel
@@ -474,8 +527,12 @@ void allow_big_lds(Kern k) {
     (void) once;
 }
 template <int P, int MODE, int NT>
-void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t lds) {
+void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256) {
     if (shfl) {
+        if constexpr (NT == 1 && (MODE == DENSE || MODE == MULTI)) {
+            if (nthr == 1024) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 1024>), grid, dim3(1024), lds, st, a); return; }
+            if (nthr == 512) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 512>), grid, dim3(512), lds, st, a); return; }
+        }
         if (lds > 48 * 1024) allow_big_lds(k_mv_seed<P, MODE, NT, true>);
         hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true>), grid, dim3(256), lds, st, a);
     } else {
@@ -484,9 +541,9 @@ void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t l
     }
 }
 template <int MODE, int NT>
-void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds) {
-    if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds);
-    else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds);
+void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256) {
+    if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds, nthr);
+    else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds, nthr);
 }
 
 // the wide path: BF16 / Q8 / Q4, whole blocks, 16-byte aligned activations and weights, staged activations within LDS
@@ -556,6 +613,11 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(R, rpi, 1);
         const dim3 grid((unsigned) ((R + a.rows_per_wg - 1) / a.rows_per_wg), 1);
+        const int nthr = pick_threads(R, L, shfl);   // the one-token launches below
+        MvArgs a1 = a;
+        a1.rpi = nthr / L;
+        a1.rows_per_wg = pick_rows_per_wg(R, a1.rpi, 1, nthr);
+        const dim3 grid1((unsigned) ((R + a1.rows_per_wg - 1) / a1.rows_per_wg), 1);
         // Several tokens: their activations staged in LDS, MV_TG tokens a workgroup, the runs of MV_TG tokens dealt to grid.y
         // (a token's arithmetic does not depend on the run it is in).  One workgroup for all of 16 tokens needed 139 KB of
         // LDS, i.e. one workgroup a CU: 2048 x 2048 at 16 tokens 21.5 us, in runs of four 14.1 us (8 tokens: 12.6 -> 9.9).
@@ -565,11 +627,11 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
             launch_seed_fmt<DENSE, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG), (size_t) MV_TG * L * XPAD * sizeof(float));
         } else {
             for (int t0 = 0; t0 < T; ++t0) {
-                MvArgs b = a;
+                MvArgs b = a1;
                 b.x = x + (size_t) t0 * xs;
                 b.y = y + (size_t) t0 * ys;
                 b.nt = 1;
-                launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid, 0);
+                launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid1, (size_t) L * XPAD * sizeof(float), nthr);
             }
         }
         note_launch();
@@ -621,7 +683,7 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     if (T == 1) {
         a.nt = 1;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
-        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, 0);
+        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
     } else {   // runs of MV_TG tokens over grid.y, as kc_mv's
         a.ttot = T;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
@@ -645,7 +707,7 @@ void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const flo
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(R, rpi, P);
         const dim3 grid((unsigned) ((R + a.rows_per_wg - 1) / a.rows_per_wg), (unsigned) P);
-        launch_seed_fmt<GATHER, 1>(st, fmt, a, shfl, grid, 0);
+        launch_seed_fmt<GATHER, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
         note_launch();
         return;
     }
@@ -668,7 +730,7 @@ void kc_mv_gu(kc_stream_t s, int fmt, const WSlice* wg, const WSlice* wu, int K,
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(2 * R, rpi, P);
         const dim3 grid((unsigned) ((2 * R + a.rows_per_wg - 1) / a.rows_per_wg), (unsigned) P);
-        launch_seed_fmt<GATEUP, 1>(st, fmt, a, shfl, grid, 0);
+        launch_seed_fmt<GATEUP, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
         note_launch();
         return;
     }

@@ -10,30 +10,25 @@ struct Chunk {
     uint32_t codes;
 };
 
-// al: the slice's streams are 16-byte (codes: 4-byte) aligned; otherwise the same records by 2-byte and 1-byte loads
+// A chunk's records: 16 bytes of seeds, 16 of coefficient (nibble) words, 4 of exponent codes.  The streams of a slice may start
+// at any 2-byte (codes: 1-byte) boundary - the loads are typed with that alignment, and the target reads a misaligned
+// 16-byte unit in one instruction all the same - so there is one code path, no branch on the alignment and no join for the
+// compiler to put a wait at.  `al` is kept in the signature for the callers and not used.
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u32_a1 __attribute__((aligned(1)));
 template <int P>
 __device__ __forceinline__ Chunk load_chunk(const WSlice& w, uint32_t unit, bool ok, bool al) {
+    (void) al;
     Chunk c;
     c.sd = make_uint4(0, 0, 0, 0);
     c.cw = c.sd;
     c.codes = 0;
     if (!ok) return c;
-    if (al) {
-        c.sd = ldg16(gp<uint4>(w.p[0]) + unit);
-        c.cw = ldg16(gp<uint4>(w.p[1]) + unit);
-        if (P == 4) c.codes = gp<uint32_t>(w.p[3])[unit];
-    } else {
-        const NSLM_GLOBAL uint16_t* sp = gp<uint16_t>(w.p[0]) + (size_t) unit * 8;
-        const NSLM_GLOBAL uint16_t* cp = gp<uint16_t>(w.p[1]) + (size_t) unit * 8;
-        c.sd = make_uint4(sp[0] | (uint32_t) sp[1] << 16, sp[2] | (uint32_t) sp[3] << 16, sp[4] | (uint32_t) sp[5] << 16,
-                          sp[6] | (uint32_t) sp[7] << 16);
-        c.cw = make_uint4(cp[0] | (uint32_t) cp[1] << 16, cp[2] | (uint32_t) cp[3] << 16, cp[4] | (uint32_t) cp[5] << 16,
-                          cp[6] | (uint32_t) cp[7] << 16);
-        if (P == 4) {
-            const NSLM_GLOBAL uint8_t* ep = gp<uint8_t>(w.p[3]) + (size_t) unit * 4;
-            c.codes = ep[0] | (uint32_t) ep[1] << 8 | (uint32_t) ep[2] << 16 | (uint32_t) ep[3] << 24;
-        }
-    }
+    const u32x4_a2 s4 = *(const NSLM_GLOBAL u32x4_a2*) (gp<uint8_t>(w.p[0]) + (size_t) unit * 16);
+    const u32x4_a2 c4 = *(const NSLM_GLOBAL u32x4_a2*) (gp<uint8_t>(w.p[1]) + (size_t) unit * 16);
+    c.sd = make_uint4(s4.x, s4.y, s4.z, s4.w);
+    c.cw = make_uint4(c4.x, c4.y, c4.z, c4.w);
+    if (P == 4) c.codes = *(const NSLM_GLOBAL u32_a1*) (gp<uint8_t>(w.p[3]) + (size_t) unit * 4);
     return c;
 }
 __device__ __forceinline__ bool streams_aligned(int P, const WSlice& w) {
