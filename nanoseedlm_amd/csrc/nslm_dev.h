@@ -190,6 +190,51 @@ __device__ __forceinline__ void isum_p3(uint32_t up, uint32_t g, uint32_t q01, u
     }
 }
 
+// ---- P = 4 by nibble columns (the matvec's form) -----------------------------------------------------------------------------
+// What a VALU instruction costs on this target was measured (issue slots of a SIMD with two or more waves resident): and / or /
+// xor / shift right / add / mov / f32 mul, fma / int -> f32 convert ~2.5 cycles; everything with three sources or sub-word
+// operands - v_alignbit, v_perm, v_bfe, shift left, the v_dot*, v_mad_* - ~4.3.  The exact decode above spends 47 of the
+// expensive ones a block (15 windows, 16 pairings, 16 dot2).  A matvec does not need the eight sums themselves, only
+// sum_c x_c isum_c, and that can be regrouped so that eleven v_dot8_i32_i4 do the 32 multiply-adds:
+//   state_(4c+1+p) = sum_n 16^n N_p(c + n),  N_p(m) = the nibble at bits [4m+1+p, 4m+5+p) of the 48-bit stream S (m = 0..10);
+//   sum_c x_c isum_c = sum_m Z(m) X(m) - 32768 Q SX,   Z(m) = sum_p q_p N_p(m),  X(m) = sum_n 16^n x_(m-n),  Q = sum_p q_p,  SX = sum_c x_c;
+//   with signed nibbles N' = N - 8 (one xor):  = sum_m Z'(m) X(m) + Q CX,  Z'(m) = sum_p q_p N'_p(m),  CX = (8 * 4369 - 32768) SX = 2184 SX.
+// N_p(m) is nibble m of V_p = S >> (1 + p), so byte j of V_0..V_3, gathered into one register (a 4 x 6 byte transpose: 12 v_perm),
+// holds the columns m = 2j and 2j + 1, and v_dot8_i32_i4 against the coefficient nibbles spread to the even (odd) nibble
+// positions gives Z'(2j) (Z'(2j + 1)).  Z' and Q are exact small integers; X and CX depend on the activations only and are
+// formed once per activation row (xform_block in nslm_mv_dev.h).  The weights are never materialised: kernels that need
+// them (the GEMM's decoder, kc_slice_deq) keep the exact sums above.
+__device__ __forceinline__ int dot8z(uint32_t a, uint32_t b) {
+    int d;
+    asm("v_dot8_i32_i4 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+// the coefficient nibbles q0..q3 of block `odd` (0 / 1) of a packed pair of coefficient words, one to a byte: the even-column operand
+__device__ __forceinline__ uint32_t coef_bytes(uint32_t cc, int odd) {
+    const uint32_t t = cc & 0x0F0F0F0Fu, u = (cc >> 4) & 0x0F0F0F0Fu;   // (q0, q2 | q0', q2'), (q1, q3 | q1', q3')
+    return __builtin_amdgcn_perm(u, t, odd ? 0x07030602u : 0x05010400u);
+}
+// sl: stream bits 0..31 (the seed below 16 bits of g), g: bits 16..47.  G[j] = byte j of V_0..V_3 with the nibbles made signed:
+// columns 2j (low nibbles) and 2j + 1 (high nibbles).
+__device__ __forceinline__ void col_bytes_p4(uint32_t sl, uint32_t g, uint32_t (&G)[6]) {
+    const uint32_t sh = g >> 16;
+    uint32_t vl[4], vh[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        vl[p] = __builtin_amdgcn_alignbit(sh, sl, 1 + p);
+        vh[p] = sh >> (1 + p);
+    }
+    const uint32_t a01 = __builtin_amdgcn_perm(vl[1], vl[0], 0x05010400u), b01 = __builtin_amdgcn_perm(vl[1], vl[0], 0x07030602u);
+    const uint32_t a23 = __builtin_amdgcn_perm(vl[3], vl[2], 0x05010400u), b23 = __builtin_amdgcn_perm(vl[3], vl[2], 0x07030602u);
+    const uint32_t h01 = __builtin_amdgcn_perm(vh[1], vh[0], 0x05010400u), h23 = __builtin_amdgcn_perm(vh[3], vh[2], 0x05010400u);
+    G[0] = __builtin_amdgcn_perm(a23, a01, 0x05040100u) ^ 0x88888888u;
+    G[1] = __builtin_amdgcn_perm(a23, a01, 0x07060302u) ^ 0x88888888u;
+    G[2] = __builtin_amdgcn_perm(b23, b01, 0x05040100u) ^ 0x88888888u;
+    G[3] = __builtin_amdgcn_perm(b23, b01, 0x07060302u) ^ 0x88888888u;
+    G[4] = __builtin_amdgcn_perm(h23, h01, 0x05040100u) ^ 0x88888888u;
+    G[5] = __builtin_amdgcn_perm(h23, h01, 0x07060302u) ^ 0x88888888u;
+}
+
 // Two blocks at once, written in phases (all windows, then all sign flips, all pairings, all products) with the
 // scheduler held to that order: a VALU result is not available to the next instruction slots, and a wave that has a SIMD's
 // vector issue to itself (the GEMM's decoder waves) loses those slots unless dependent instructions sit far apart.  In

@@ -159,7 +159,7 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
         const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
         // (two blocks at a time in phase order where three workgroups a CU compute at once; the down pass, whose waves mostly
         // run alone behind their pair's readiness, keeps the compiler's order)
-        if (active && v < v1) chunk_dot<P, 1, GATEUP>(cur, eb, tab, xl + ch * XPAD, 0, 1, acc);
+        if (active && v < v1) chunk_dot<P, 1, GATEUP>(cur, eb, tab, xl + ch * xpad<P>(), 0, 1, acc);
         if (SHFL) {
             float s = acc[0];
             for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -189,40 +189,53 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
     if (!SHFL) __syncthreads();   // part may be reused by the next pass
 }
 
-// n floats of a row staged chunk-padded into LDS by the whole workgroup; coherent: agent-scope loads (the row was
-// written by other workgroups of this launch).  Eight loads a thread are requested before the first is used (clamped
-// indices, so they are unconditional): one load and one LDS store a round is one memory round trip a round.
+// n floats of a row staged into LDS in the form the format's matvec reads (store_block: chunk-padded, P = 4 as its 12 column
+// values a block) by the whole workgroup; coherent: agent-scope loads (the row was written by other workgroups of this
+// launch).  A thread takes whole blocks, four a round, and requests their 32 words before the first is used (clamped
+// indices, so the loads are unconditional): one load and one LDS store a round is one memory round trip a round.
+template <int P>
 __device__ __forceinline__ void stage_row(const float* src, int n, float* xl, bool coherent) {
-    for (int i0 = threadIdx.x; i0 < n; i0 += 256 * 8) {
-        float v[8];
+    const int nb = n / 8;
+    for (int b0 = threadIdx.x; b0 < nb; b0 += 256 * 4) {
+        float v[4][8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int i = min(i0 + 256 * u, n - 1);
-            v[u] = coherent ? ld_agent(src + i) : src[i];
+        for (int u = 0; u < 4; ++u) {
+            const float* p = src + (size_t) min(b0 + 256 * u, nb - 1) * 8;
+            if (coherent) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[u][c] = ld_agent(p + c);
+            } else {
+                const float4 q0 = *(const float4*) p, q1 = *(const float4*) (p + 4);
+                v[u][0] = q0.x; v[u][1] = q0.y; v[u][2] = q0.z; v[u][3] = q0.w; v[u][4] = q1.x; v[u][5] = q1.y; v[u][6] = q1.z; v[u][7] = q1.w;
+            }
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int i = i0 + 256 * u;
-            if (i < n) xl[(i >> 6) * XPAD + (i & 63)] = v[u];
-        }
+        for (int u = 0; u < 4; ++u)
+            if (b0 + 256 * u < nb) store_block<P>(xl, b0 + 256 * u, v[u]);
     }
 }
 // an input row, normalised on the way when nw is given: the values kq4_norm1p would have stored
+template <int P>
 __device__ __forceinline__ void stage_input(const float* src, int n, float* xl, const float* nw, float rn) {
-    if (!nw) { stage_row(src, n, xl, false); return; }
-    for (int i0 = threadIdx.x; i0 < n; i0 += 256 * 8) {
-        float v[8], w[8];
+    if (!nw) { stage_row<P>(src, n, xl, false); return; }
+    const int nb = n / 8;
+    for (int b0 = threadIdx.x; b0 < nb; b0 += 256 * 4) {
+        float v[4][8], w[4][8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int i = min(i0 + 256 * u, n - 1);
-            v[u] = src[i];
-            w[u] = nw[i];
+        for (int u = 0; u < 4; ++u) {
+            const size_t o = (size_t) min(b0 + 256 * u, nb - 1) * 8;
+            const float4 q0 = *(const float4*) (src + o), q1 = *(const float4*) (src + o + 4);
+            const float4 w0 = *(const float4*) (nw + o), w1 = *(const float4*) (nw + o + 4);
+            v[u][0] = q0.x; v[u][1] = q0.y; v[u][2] = q0.z; v[u][3] = q0.w; v[u][4] = q1.x; v[u][5] = q1.y; v[u][6] = q1.z; v[u][7] = q1.w;
+            w[u][0] = w0.x; w[u][1] = w0.y; w[u][2] = w0.z; w[u][3] = w0.w; w[u][4] = w1.x; w[u][5] = w1.y; w[u][6] = w1.z; w[u][7] = w1.w;
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int i = i0 + 256 * u;
-            if (i < n) xl[(i >> 6) * XPAD + (i & 63)] = v[u] * rn * (1.0f + w[u]);
-        }
+        for (int u = 0; u < 4; ++u)
+            if (b0 + 256 * u < nb) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c) v[u][c] = v[u][c] * rn * (1.0f + w[u][c]);
+                store_block<P>(xl, b0 + 256 * u, v[u]);
+            }
     }
 }
 
@@ -373,7 +386,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     // the first gate+up item's activations are an input of the launch: staged while the other workgroups' logits arrive
     if ((int) blockIdx.x < items_g) {
         staged = ((int) blockIdx.x / a.ntile_g) / a.kk;
-        stage_input(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
+        stage_input<P>(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
     }
     STAMP(1);
     // No grid barrier: what the other workgroups produce here are the logits, and those say themselves when they are there.
@@ -466,7 +479,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         route_weights(t);
         if (staged != t) {
             __syncthreads();
-            stage_input(a.x + (size_t) t * a.xs, a.d, xl, a.nw, a.nw ? rn_s[t] : 1.0f);
+            stage_input<P>(a.x + (size_t) t * a.xs, a.d, xl, a.nw, a.nw ? rn_s[t] : 1.0f);
             staged = t;
             __syncthreads();
         }
@@ -521,7 +534,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         __syncthreads();
         wg_acquire();
         if (item == (int) blockIdx.x) STAMP(4);   // the first down item's pair is ready
-        stage_row(a.A + (size_t) p * a.ff, a.ff, xl, true);
+        stage_row<P>(a.A + (size_t) p * a.ff, a.ff, xl, true);
         staged = -1;
         __syncthreads();
         if (item == (int) blockIdx.x) DSTAMP(16);
@@ -571,6 +584,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 // slots >= k are the always-on experts (expert ids E, E + 1, ...).
 #define FG_MAXP 512    // pairs a launch: T * kk
 #define FG_RN_WORDS 64   // the rows' RMSNorm scales behind the pairs' words of the sync area
+#define FG_PRE_BYTES (1024 * 4 + FG_MAXP * 2 + 2 * (1024 + 32) * 2)   // dynamic LDS the phases before the passes use
 
 template <int P, bool GATEUP, bool SHFL, int NT, typename Emit>
 __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1,
@@ -592,7 +606,7 @@ __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const W
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
         const int eb = (GATEUP && (v & 1)) ? wB.eb : wA.eb;
-        if (active && v < v1) chunk_dot<P, NT, true>(cur, eb, tab, xl + ch * XPAD, xstride, nt, acc);
+        if (active && v < v1) chunk_dot<P, NT, true>(cur, eb, tab, xl + ch * xpad<P>(), xstride, nt, acc);
         if (SHFL) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -634,22 +648,27 @@ __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const W
 
 template <int P, int NT, bool SHFL_G, bool SHFL_D>
 __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
-    extern __shared__ float xl[];   // NT rows of max(d, ff) activations, chunk-padded, side by side
+    extern __shared__ __attribute__((aligned(16))) float xl[];   // NT rows of max(d, ff) activations, chunk-padded, side by side
+    // What only the routing and the building of the groups need lives in the same area, which the passes overwrite (the launch
+    // asks for FG_PRE_BYTES at least): a kilobyte of static LDS less is a resident workgroup more at some widths.
+    float* const rv = xl;                                          // [1024] a token's logits
+    uint16_t* const gof = (uint16_t*) (xl + 1024);                 // [FG_MAXP] a pair's position among its expert's pairs
+    uint16_t* const cnt_s = gof + FG_MAXP;                         // [1024 + 32] per expert: pairs
+    uint16_t* const base_s = cnt_s + 1024 + 32;                    // [1024 + 32] per expert: first group
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[2 * NT * 256];
-    __shared__ __attribute__((aligned(16))) float rv[1024];
     __shared__ float rw_s[33];
     __shared__ int ri_s[33];
     __shared__ WSlice sl_s[3];
     __shared__ int s_flag, s_ng;
     __shared__ float rn_s[FG_MAXT], nred[4];
     __shared__ __attribute__((aligned(16))) uint16_t pe[FG_MAXP + 8];   // a pair's expert
-    __shared__ uint16_t gof[FG_MAXP], gm[FG_MAXP * NT], cnt_s[1024 + 32], base_s[1024 + 32];   // position; members; per expert: pairs, first group
+    __shared__ uint16_t gm[FG_MAXP * NT];   // a group's members
     __shared__ uint8_t gn[FG_MAXP];   // a group's number of members
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t G = (uint32_t) a.grid;
     const int P_ = a.T * a.kk, NE = a.E + a.ns;
-    const int xsg = a.Lg * XPAD, xsd = a.Ld * XPAD;   // LDS floats between two rows of activations
+    const int xsg = a.Lg * xpad<P>(), xsd = a.Ld * xpad<P>();   // LDS floats between two rows of activations
     // (fixed places, whatever the launch's rows and widths: launches of different sizes share the area, and every word
     // but the scales is back at zero when a launch ends)
     float* rnpub = (float*) (a.sync + FUSED_SYNC_WORDS);
@@ -854,7 +873,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         if (staged_g != g) {
             for (int m = 0; m < nt; ++m) {
                 const int t = gm[g * NT + m] / a.kk;
-                stage_input(a.x + (size_t) t * a.xs, a.d, xl + m * xsg, a.nw, a.nw ? rn_s[t] : 1.0f);
+                stage_input<P>(a.x + (size_t) t * a.xs, a.d, xl + m * xsg, a.nw, a.nw ? rn_s[t] : 1.0f);
             }
             staged_g = g;
             __syncthreads();
@@ -894,7 +913,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         }
         __syncthreads();
         wg_acquire();
-        for (int m = 0; m < nt; ++m) stage_row(a.A + (size_t) gm[g * NT + m] * a.ff, a.ff, xl + m * xsd, true);
+        for (int m = 0; m < nt; ++m) stage_row<P>(a.A + (size_t) gm[g * NT + m] * a.ff, a.ff, xl + m * xsd, true);
         staged_g = -1;
         __syncthreads();
         auto put_d = [&](int m, int r, float sm, float) { st_agent(a.D + (size_t) gm[g * NT + m] * a.d + r, bfr(sm)); };
@@ -1024,7 +1043,8 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
     void (*kern)(FusedArgs) = sg ? (sd ? k_moe_decode_grouped<P, NT, true, true> : k_moe_decode_grouped<P, NT, true, false>)
                                  : (sd ? k_moe_decode_grouped<P, NT, false, true> : k_moe_decode_grouped<P, NT, false, false>);
     const int lmax = a.Lg > a.Ld ? a.Lg : a.Ld;
-    const size_t lds = (size_t) NT * lmax * XPAD * sizeof(float);
+    size_t lds = (size_t) NT * lmax * xpad<P>() * sizeof(float);
+    if (lds < FG_PRE_BYTES) lds = FG_PRE_BYTES;
     static int cached[2][2] = {{0, 0}, {0, 0}};   // resident workgroups per CU, by kernel variant, for the largest request seen
     static size_t cached_lds[2][2] = {{0, 0}, {0, 0}};
     int& per_cu = cached[sg][sd];
@@ -1132,7 +1152,7 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
     const int kmax = d > ff ? d : ff;
-    size_t lds = (size_t) (kmax / 64) * XPAD * sizeof(float);
+    size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
 }
 

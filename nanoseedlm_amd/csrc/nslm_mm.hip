@@ -346,10 +346,11 @@ __global__ void __launch_bounds__(512) k_mm(int fmt, MmArgs a, WSlice wd, const 
             }
 }
 
-// a kernel that asks for more dynamic LDS than the default limit has the limit raised to what it needs, once
-template <typename Kern>
-void allow_big_lds(Kern k, size_t bytes) {
-    static const hipError_t once = bytes > 48 * 1024 ? hipFuncSetAttribute((const void*) k, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes)
+// a kernel that asks for more dynamic LDS than the default limit has the limit raised to what it needs, once (the kernel is a
+// template argument so that every kernel has its own "once": kernels of one signature share a pointer type)
+template <auto K>
+void allow_big_lds(size_t bytes) {
+    static const hipError_t once = bytes > 48 * 1024 ? hipFuncSetAttribute((const void*) K, hipFuncAttributeMaxDynamicSharedMemorySize, (int) bytes)
                                                      : hipSuccess;
     (void) once;
 }
@@ -362,11 +363,11 @@ void launch_mm(hipStream_t st, int fmt, const MmArgs& a, WSlice wd, const WSlice
     const bool exact = g_seed_exact && (fmt == MF_SEED4 || fmt == MF_SEED4P4);
     if (exact) {
         const size_t lds = mm_lds<MT, 3>();
-        allow_big_lds(k_mm<MT, 3, PACKED>, lds);
+        allow_big_lds<k_mm<MT, 3, PACKED>>(lds);
         hipLaunchKernelGGL((k_mm<MT, 3, PACKED>), grid, dim3(512), lds, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
     } else {
         const size_t lds = mm_lds<MT, 1>();
-        allow_big_lds(k_mm<MT, 1, PACKED>, lds);
+        allow_big_lds<k_mm<MT, 1, PACKED>>(lds);
         hipLaunchKernelGGL((k_mm<MT, 1, PACKED>), grid, dim3(512), lds, st, fmt, a, wd, ws, X, Y, perm, tiles, ntiles);
     }
     host_note_launch();
@@ -680,9 +681,8 @@ template <int CT, int NCW, int XCH, int FMT>
 void launch_mm_stream_f(hipStream_t st, const MmArgs& a, WSlice wd, const WSlice* ws, const void* X, float* Y, const int32_t* perm,
                         const MmTile* tiles, const int32_t* ntiles, dim3 grid) {
     const size_t lds = mm_stream_lds<NCW, XCH>();
-    auto kern = k_mm_stream<CT, NCW, XCH, FMT>;
-    allow_big_lds(kern, lds);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * (NCW + 4)), lds, st, a, wd, ws, (const uint16_t*) X, Y, perm, tiles, ntiles);
+    allow_big_lds<k_mm_stream<CT, NCW, XCH, FMT>>(lds);
+    hipLaunchKernelGGL((k_mm_stream<CT, NCW, XCH, FMT>), grid, dim3(64 * (NCW + 4)), lds, st, a, wd, ws, (const uint16_t*) X, Y, perm, tiles, ntiles);
     host_note_launch();
 }
 template <int CT, int NCW, int XCH>

@@ -58,10 +58,12 @@ __device__ unsigned long long g_mvstamp[8192 * 16];
 // SHFL: L is a power of two <= 64 (<= 32 for GATEUP): row sums by wave shuffles, no barrier.  Otherwise through LDS.
 // NTHR: threads a workgroup (256; 512 or 1024 for one-token SHFL launches whose rows fill more than four waves a CU - the
 // row and the tables are then fetched once per CU instead of once per four waves).
-template <int P, int MODE, int NT, bool SHFL, int NTHR = 256>
+// COLS: P = 4 blocks in the column form (one- and two-token passes, and every pass of a launch of up to MV_MAXT tokens, whose
+// tokens get the bits of a one-token call); false: the weights' form (launches of more tokens, four to a pass).
+template <int P, int MODE, int NT, bool SHFL, int NTHR = 256, bool COLS = (P == 4)>
 __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
     static_assert(NTHR == 256 || (SHFL && NT == 1), "the LDS row sums and the staged multi-token passes are written for 256 threads");
-    extern __shared__ float xl[];                  // activations [token][chunk][XPAD]
+    extern __shared__ float xl[];                  // activations as the format reads them (xform_block): [token][chunk][xpad<P>()]
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[SHFL ? 1 : 2][SHFL ? 1 : NT][SHFL ? 1 : 256];
     __shared__ float nred[4];
@@ -95,15 +97,22 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
     // L2 and are needed first, go out before the records, which come from HBM behind everybody else's.
     const TableWords<NTHR> tw = tables_fetch<NTHR>();
     const bool prenorm = MODE == MULTI && a.nw != nullptr;   // uniform; the other modes compile without it
-    float xreg[NT == 1 ? 64 : 1];
-    constexpr int NXQ = 2048 / NTHR;   // K <= 8192: at most 2048 16-byte pieces of a row
-    float4 xq[NT == 1 ? NXQ : 1], wq[NT == 1 ? NXQ : 1];
+    constexpr int XW = xw<P, COLS>(), XP = xpad<P, COLS>();
+    constexpr bool XREG = NT == 1 && !COLS;   // P = 3 keeps the thread's 64 activations in registers; the 96 column values of
+                                               // P = 4 stay in LDS (three 16-byte reads a block), which leaves the registers for eight waves a SIMD
+    float xreg[XREG ? 8 * XW : 1];
+    constexpr int NXQ = 1024 / NTHR;   // K <= 8192: at most 1024 blocks of a row, a thread takes whole blocks (two 16-byte pieces)
+    float4 xq[NT == 1 ? NXQ : 1][2], wq[NT == 1 ? NXQ : 1][2];
     if (NT == 1) {   // clamped, so that the loads stay unconditional
 #pragma unroll
         for (int j = 0; j < NXQ; ++j) {
-            const int i = min(tid + NTHR * j, a.K / 4 - 1);
-            xq[j] = ((const float4*) xrow)[i];
-            if (MODE == MULTI && prenorm) wq[j] = ((const float4*) a.nw)[i];
+            const int i = min(tid + NTHR * j, a.K / 8 - 1);
+            xq[j][0] = ((const float4*) xrow)[2 * i];
+            xq[j][1] = ((const float4*) xrow)[2 * i + 1];
+            if (MODE == MULTI && prenorm) {
+                wq[j][0] = ((const float4*) a.nw)[2 * i];
+                wq[j][1] = ((const float4*) a.nw)[2 * i + 1];
+            }
         }
     }
     loads_issued();
@@ -130,20 +139,20 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         // The row goes through LDS once per workgroup and from there into each thread's registers (the 256 / L threads that
         // share a chunk do not each fetch it).  Every load of the prologue - tables, row, records - is requested before the
         // first wait, so the kernel starts after one memory round trip.
-        const int K4 = a.K / 4;
         // (with a norm: the row's scale, bit for bit as the norm kernel forms it - a second pass over the row, from L2)
         const float rn = (MODE == MULTI && prenorm) ? row_rnorm(xrow, a.K, a.neps, nred) : 1.0f;
         tables_store<NTHR>(tab, tw);
 #pragma unroll
         for (int j = 0; j < NXQ; ++j) {
             const int i = tid + NTHR * j;
-            if (i < K4) {
-                float4 v4 = xq[j];
+            if (i < a.K / 8) {
+                float x8[8] = {xq[j][0].x, xq[j][0].y, xq[j][0].z, xq[j][0].w, xq[j][1].x, xq[j][1].y, xq[j][1].z, xq[j][1].w};
                 if (MODE == MULTI && prenorm) {
-                    v4.x = v4.x * rn * (1.0f + wq[j].x); v4.y = v4.y * rn * (1.0f + wq[j].y);
-                    v4.z = v4.z * rn * (1.0f + wq[j].z); v4.w = v4.w * rn * (1.0f + wq[j].w);
+                    const float w8[8] = {wq[j][0].x, wq[j][0].y, wq[j][0].z, wq[j][0].w, wq[j][1].x, wq[j][1].y, wq[j][1].z, wq[j][1].w};
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) x8[c] = x8[c] * rn * (1.0f + w8[c]);
                 }
-                *(float4*) &xl[(i >> 4) * XPAD + (i & 15) * 4] = v4;
+                store_block<P, COLS>(xl, i, x8);
             }
         }
     } else {
@@ -158,34 +167,37 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
             }
             __syncthreads();
         }
-        const int K4 = a.K / 4, tot = nt_ * K4;
-        for (int base = tid; base < tot; base += 256 * 8) {
-            float4 q[8];
+        const int nb = a.K / 8, tot = nt_ * nb;   // whole blocks: four a thread and round, their eight loads in flight together
+        for (int base = tid; base < tot; base += 256 * 4) {
+            float4 q[4][2];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int idx = min(base + 256 * j, tot - 1), t = idx / K4, i = idx - t * K4;
-                q[j] = ((const float4*) (xbase + (size_t) t * a.xs))[i];
+            for (int j = 0; j < 4; ++j) {
+                const int idx = min(base + 256 * j, tot - 1), t = idx / nb, i = idx - t * nb;
+                q[j][0] = ((const float4*) (xbase + (size_t) t * a.xs))[2 * i];
+                q[j][1] = ((const float4*) (xbase + (size_t) t * a.xs))[2 * i + 1];
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 4; ++j) {
                 const int idx = base + 256 * j;
                 if (idx >= tot) break;
-                const int t = idx / K4, i = idx - t * K4;
-                float4 v = q[j];
+                const int t = idx / nb, i = idx - t * nb;
+                float x8[8] = {q[j][0].x, q[j][0].y, q[j][0].z, q[j][0].w, q[j][1].x, q[j][1].y, q[j][1].z, q[j][1].w};
                 if (prenorm) {
-                    const float4 w4 = ((const float4*) a.nw)[i];
+                    const float4 w0 = ((const float4*) a.nw)[2 * i], w1 = ((const float4*) a.nw)[2 * i + 1];
+                    const float w8[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
                     const float rn = rn_s[t];
-                    v.x = v.x * rn * (1.0f + w4.x); v.y = v.y * rn * (1.0f + w4.y); v.z = v.z * rn * (1.0f + w4.z); v.w = v.w * rn * (1.0f + w4.w);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) x8[c] = x8[c] * rn * (1.0f + w8[c]);
                 }
-                *(float4*) &xl[(t * L + (i >> 4)) * XPAD + (i & 15) * 4] = v;
+                store_block<P, COLS>(xl + (size_t) t * L * XP, i, x8);
             }
         }
     }
     __syncthreads();
-    if (NT == 1 && active) {
+    if (XREG && active) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float4 q = *(const float4*) &xl[ch * XPAD + 4 * i];
+        for (int i = 0; i < 2 * XW; ++i) {
+            const float4 q = *(const float4*) &xl[ch * XP + 4 * i];
             xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
         }
     }
@@ -201,8 +213,8 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
         const int eb = (MODE == GATEUP && (v & 1)) ? eB : eA;
         if (active && v < v1) {
-            if (NT == 1) chunk_dot<P, NT>(cur, eb, tab, xreg, 0, 1, acc);
-            else chunk_dot<P, NT>(cur, eb, tab, xl + ch * XPAD, L * XPAD, nt_, acc);
+            if (XREG) chunk_dot<P, NT, false, COLS>(cur, eb, tab, xreg, 0, 1, acc);
+            else chunk_dot<P, NT, false, COLS>(cur, eb, tab, xl + ch * XP, L * XP, nt_, acc);
         }
         if (SHFL) {
 #pragma unroll
@@ -488,6 +500,12 @@ bool fast_shape(int fmt, int K, int mode, int* L, int* rpi, bool* shfl) {
     return true;
 }
 
+// staged floats per 64-weight chunk; cols: the launch's P = 4 blocks go in the column form
+int xpad_of(int fmt, bool cols = true) { return fmt == MF_SEED4P4 ? (cols ? xpad<4, true>() : xpad<4, false>()) : xpad<3>(); }
+// launches of up to MV_MAXT tokens give every token the bits of a one-token call (the column form); longer ones trade that for
+// the weights' form, which reads a third less LDS a token
+bool cols_for(int T) { return T <= MV_MAXT; }
+
 int cu_count() {
     static int n = 0;
     if (!n) {
@@ -520,36 +538,46 @@ int pick_threads(int V, int L, bool shfl) {
     return per_cu > 8 ? 1024 : per_cu > 4 ? 512 : 256;
 }
 
-// kernels that stage activations may need more dynamic LDS than the default limit: raise it once per kernel
-template <typename Kern>
-void allow_big_lds(Kern k) {
-    static const hipError_t once = hipFuncSetAttribute((const void*) k, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+// kernels that stage activations may need more dynamic LDS than the default limit: raise it once per kernel, to what the
+// CU's 160 KB leave beside the kernels' static arrays (under 32 KB each)
+#define MV_LDS_MAX (128 * 1024)
+// (the kernel is a template argument so that every kernel has its own "once": kernels of one signature share a pointer type)
+template <auto K>
+void allow_big_lds() {
+    static const hipError_t once = hipFuncSetAttribute((const void*) K, hipFuncAttributeMaxDynamicSharedMemorySize, MV_LDS_MAX);
     (void) once;
 }
-template <int P, int MODE, int NT>
-void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256) {
+template <int P, int MODE, int NT, bool COLS>
+void launch_seed256(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t lds) {
     if (shfl) {
-        if constexpr (NT == 1 && (MODE == DENSE || MODE == MULTI)) {
-            if (nthr == 1024) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 1024>), grid, dim3(1024), lds, st, a); return; }
-            if (nthr == 512) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 512>), grid, dim3(512), lds, st, a); return; }
-        }
-        if (lds > 48 * 1024) allow_big_lds(k_mv_seed<P, MODE, NT, true>);
-        hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true>), grid, dim3(256), lds, st, a);
+        if (lds > 48 * 1024) allow_big_lds<k_mv_seed<P, MODE, NT, true, 256, COLS>>();
+        hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 256, COLS>), grid, dim3(256), lds, st, a);
     } else {
-        if (lds > 48 * 1024) allow_big_lds(k_mv_seed<P, MODE, NT, false>);
-        hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, false>), grid, dim3(256), lds, st, a);
+        if (lds > 48 * 1024) allow_big_lds<k_mv_seed<P, MODE, NT, false, 256, COLS>>();
+        hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, false, 256, COLS>), grid, dim3(256), lds, st, a);
     }
 }
+template <int P, int MODE, int NT>
+void launch_seed(hipStream_t st, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256, bool cols = true) {
+    if constexpr (NT == 1 && (MODE == DENSE || MODE == MULTI)) {
+        if (shfl && nthr == 1024) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 1024>), grid, dim3(1024), lds, st, a); return; }
+        if (shfl && nthr == 512) { hipLaunchKernelGGL((k_mv_seed<P, MODE, NT, true, 512>), grid, dim3(512), lds, st, a); return; }
+    }
+    if constexpr (P == 4 && NT > 2) {
+        if (!cols) { launch_seed256<P, MODE, NT, false>(st, a, shfl, grid, lds); return; }
+    }
+    launch_seed256<P, MODE, NT, P == 4>(st, a, shfl, grid, lds);
+}
 template <int MODE, int NT>
-void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256) {
-    if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds, nthr);
-    else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds, nthr);
+void launch_seed_fmt(hipStream_t st, int fmt, const MvArgs& a, bool shfl, dim3 grid, size_t lds, int nthr = 256, bool cols = true) {
+    if (fmt == MF_SEED4P4) launch_seed<4, MODE, NT>(st, a, shfl, grid, lds, nthr, cols);
+    else launch_seed<3, MODE, NT>(st, a, shfl, grid, lds, nthr, cols);
 }
 
 // the wide path: BF16 / Q8 / Q4, whole blocks, 16-byte aligned activations and weights, staged activations within LDS
 bool wide_ok(int fmt, int K, const void* x, int xs, int nt) {
     return (fmt == MF_BF16 || fmt == MF_Q8 || fmt == MF_Q4) && K % 8 == 0 && ((uintptr_t) x & 15u) == 0 && xs % 4 == 0 &&
-           (size_t) nt * K * sizeof(float) <= 128 * 1024;
+           (size_t) nt * K * sizeof(float) <= MV_LDS_MAX;
 }
 template <int MODE>
 void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
@@ -566,7 +594,7 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
     const dim3 grid((unsigned) gx, (unsigned) ny);
 #define NSLM_WIDE(F)                                                                         \
     do {                                                                                     \
-        if (lds > 48 * 1024) allow_big_lds(k_mv_wide<F, MODE>);                              \
+        if (lds > 48 * 1024) allow_big_lds<k_mv_wide<F, MODE>>();                              \
         hipLaunchKernelGGL((k_mv_wide<F, MODE>), grid, dim3(256), lds, st, a);               \
     } while (0)
     if (fmt == MF_BF16) NSLM_WIDE(MF_BF16);
@@ -622,16 +650,18 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         // (a token's arithmetic does not depend on the run it is in).  One workgroup for all of 16 tokens needed 139 KB of
         // LDS, i.e. one workgroup a CU: 2048 x 2048 at 16 tokens 21.5 us, in runs of four 14.1 us (8 tokens: 12.6 -> 9.9).
         // Rows too long for the staging take one launch per token with the activations in registers.
-        if (T > 1 && L <= 96) {
+        const bool cols = cols_for(T);
+        if (T > 1 && (size_t) MV_TG * L * xpad_of(fmt, cols) * sizeof(float) <= MV_LDS_MAX) {
             a.ttot = T;
-            launch_seed_fmt<DENSE, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG), (size_t) MV_TG * L * XPAD * sizeof(float));
+            launch_seed_fmt<DENSE, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG),
+                                          (size_t) MV_TG * L * xpad_of(fmt, cols) * sizeof(float), 256, cols);
         } else {
             for (int t0 = 0; t0 < T; ++t0) {
                 MvArgs b = a1;
                 b.x = x + (size_t) t0 * xs;
                 b.y = y + (size_t) t0 * ys;
                 b.nt = 1;
-                launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid1, (size_t) L * XPAD * sizeof(float), nthr);
+                launch_seed_fmt<DENSE, 1>(st, fmt, b, shfl, grid1, (size_t) L * xpad_of(fmt) * sizeof(float), nthr);
             }
         }
         note_launch();
@@ -666,7 +696,9 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     }
     int L, rpi;
     bool shfl;
-    if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MULTI_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 || L > 96) return -1;
+    if (n < 1 || n > MV_MAXJ || T < 1 || T > MV_MULTI_MAXT || !fast_shape(fmt, K, DENSE, &L, &rpi, &shfl) || !aligned16(x) || xs % 4 ||
+        (size_t) MV_TG * L * xpad_of(fmt, cols_for(T)) * sizeof(float) > MV_LDS_MAX)
+        return -1;
     if (norm_w && (K > 256 * 16 || !aligned16(norm_w))) return -1;
     MvArgs a = {};
     a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n; a.nw = norm_w; a.neps = norm_eps;
@@ -683,11 +715,12 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     if (T == 1) {
         a.nt = 1;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
-        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
+        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, (size_t) L * xpad_of(fmt) * sizeof(float));
     } else {   // runs of MV_TG tokens over grid.y, as kc_mv's
         a.ttot = T;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
-        launch_seed_fmt<MULTI, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG), (size_t) MV_TG * L * XPAD * sizeof(float));
+        launch_seed_fmt<MULTI, MV_TG>(st, fmt, a, shfl, dim3(grid.x, (unsigned) (T + MV_TG - 1) / MV_TG),
+                                      (size_t) MV_TG * L * xpad_of(fmt, cols_for(T)) * sizeof(float), 256, cols_for(T));
     }
     note_launch();
     return 0;
@@ -707,7 +740,7 @@ void kc_mv_sel(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const flo
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(R, rpi, P);
         const dim3 grid((unsigned) ((R + a.rows_per_wg - 1) / a.rows_per_wg), (unsigned) P);
-        launch_seed_fmt<GATHER, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
+        launch_seed_fmt<GATHER, 1>(st, fmt, a, shfl, grid, (size_t) L * xpad_of(fmt) * sizeof(float));
         note_launch();
         return;
     }
@@ -730,7 +763,7 @@ void kc_mv_gu(kc_stream_t s, int fmt, const WSlice* wg, const WSlice* wu, int K,
         a.L = L; a.rpi = rpi;
         a.rows_per_wg = pick_rows_per_wg(2 * R, rpi, P);
         const dim3 grid((unsigned) ((2 * R + a.rows_per_wg - 1) / a.rows_per_wg), (unsigned) P);
-        launch_seed_fmt<GATEUP, 1>(st, fmt, a, shfl, grid, (size_t) L * XPAD * sizeof(float));
+        launch_seed_fmt<GATEUP, 1>(st, fmt, a, shfl, grid, (size_t) L * xpad_of(fmt) * sizeof(float));
         note_launch();
         return;
     }

@@ -37,8 +37,47 @@ __device__ __forceinline__ bool streams_aligned(int P, const WSlice& w) {
 
 __device__ __forceinline__ uint32_t word_of(const uint4& v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 
-// One chunk (8 blocks) against NT tokens.  xr: this chunk's activations, token t at xr + t * xstride (registers when
-// NT == 1, LDS otherwise).  acc[t] accumulates 2^(e+0) * sum_c isum_c x_c per block (R32 is applied to the row sum).
+// ---- activations as the matvec reads them ----------------------------------------------------------------------------------
+// P = 3: a block's 8 activations as they are.  P = 4: the 12 values of the nibble-column form (cols_p4 in nslm_dev.h):
+// X(0..10), X(m) = x_m + 16 x_(m-1) + 256 x_(m-2) + 4096 x_(m-3) (terms outside 0..7 dropped), and CX = 2184 sum x.  One fixed
+// order of operations, so every kernel that stages a row forms the same bits.
+// COLS: the column form (P = 4 only; passes of more than two tokens read too much LDS with it - 48 bytes a token and block where
+// the weights' form reads 32 - and are given COLS = false: the block's activations as they are, like P = 3).
+template <int P, bool COLS = (P == 4)>
+constexpr int xw() { return COLS ? 12 : 8; }          // floats a block
+// LDS floats per 64-weight chunk (8 blocks + 4): 16-byte reads of 8 consecutive lanes land on 32 distinct banks (68 and 100 are 4 mod 32)
+template <int P, bool COLS = (P == 4)>
+constexpr int xpad() { return 8 * xw<P, COLS>() + 4; }
+template <int P, bool COLS = (P == 4)>
+__device__ __forceinline__ void xform_block(const float (&x)[8], float (&X)[xw<P, COLS>()]) {
+    static_assert(!COLS || P == 4, "the column form is the P = 4 block's");
+    if constexpr (COLS) {
+#pragma unroll
+        for (int m = 0; m < 11; ++m) {
+            float v = m < 8 ? x[m] : 0.0f;
+            if (m >= 1 && m <= 8) v = fmaf(16.0f, x[m - 1], v);
+            if (m >= 2 && m <= 9) v = fmaf(256.0f, x[m - 2], v);
+            if (m >= 3) v = fmaf(4096.0f, x[m - 3], v);
+            X[m] = v;
+        }
+        X[11] = 2184.0f * (((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7])));
+    } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) X[c] = x[c];
+    }
+}
+// block `blk` of a row into its place of a chunk-padded LDS row
+template <int P, bool COLS = (P == 4)>
+__device__ __forceinline__ void store_block(float* row, int blk, const float (&x)[8]) {
+    float X[xw<P, COLS>()];
+    xform_block<P, COLS>(x, X);
+    float* dst = row + (blk >> 3) * xpad<P, COLS>() + (blk & 7) * xw<P, COLS>();
+#pragma unroll
+    for (int i = 0; i < xw<P, COLS>(); i += 4) *(float4*) (dst + i) = make_float4(X[i], X[i + 1], X[i + 2], X[i + 3]);
+}
+
+// One chunk (8 blocks) against NT tokens.  xr: this chunk's staged activations, token t at xr + t * xstride (registers when
+// NT == 1 and the caller copied them, LDS otherwise).  acc[t] accumulates 2^e * (block . x) per block (R32 is applied to the row sum).
 template <int P, int NT>
 __device__ __forceinline__ void block_dot(const int (&is)[8], float e2, int b, const float* xr, int xstride, float (&acc)[NT]) {
     float w[8];
@@ -74,57 +113,78 @@ __device__ __forceinline__ void block_dot(const int (&is)[8], float e2, int b, c
         }
     }
 }
-// PAIRED: two blocks at a time in phase order (isum2_*), as the GEMM's decoder waves decode: measured 1 % faster in the
-// persistent MoE kernel (three waves a SIMD), 6 % slower in the stand-alone matvec, which keeps the compiler's own order.
-template <int P, int NT, bool PAIRED = false>
+// The column form of a P = 4 block against NT tokens' 12 staged values: every column's sum is converted and used as soon as it
+// is formed (eleven sums and their float images held at once cost the persistent kernels their five waves a SIMD).
+template <int NT>
+__device__ __forceinline__ void cols_dot(uint32_t sl, uint32_t g, uint32_t be, float e2, int b, const float* xr, int xstride, float (&acc)[NT]) {
+    float4 xa[NT][3];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const float* xb = xr + t * xstride + 12 * b;
+        xa[t][0] = *(const float4*) xb;
+        xa[t][1] = *(const float4*) (xb + 4);
+        xa[t][2] = *(const float4*) (xb + 8);
+    }
+    uint32_t G[6];
+    col_bytes_p4(sl, g, G);
+    const uint32_t bo = be << 4;
+    float d[NT];
+    auto xv = [&](int t, int m) { const float4& q = xa[t][m >> 2]; return (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w; };
+#pragma unroll
+    for (int m = 0; m < 12; ++m) {
+        const float z = (float) (m == 11 ? dot8z(be, 0x01010101u) : dot8z(G[m >> 1], (m & 1) ? bo : be));
+#pragma unroll
+        for (int t = 0; t < NT; ++t) d[t] = m == 0 ? z * xv(t, 0) : fmaf(z, xv(t, m), d[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = fmaf(d[t], e2, acc[t]);
+}
+// PAIRED (P = 3 only): two blocks at a time in phase order (isum2_p3), as the GEMM's decoder waves decode: measured 1 % faster
+// in the persistent MoE kernel (three waves a SIMD), 6 % slower in the stand-alone matvec, which keeps the compiler's own order.
+template <int P, int NT, bool PAIRED = false, bool COLS = (P == 4)>
 __device__ __forceinline__ void chunk_dot(const Chunk& ck, int eb, const uint32_t* tab, const float* xr, int xstride, int nt,
                                           float (&acc)[NT]) {
     (void) nt;
-    if constexpr (PAIRED) {
+    static_assert(!PAIRED || P == 3 || COLS, "blocks in pairs: P = 3 only (the column form has one order)");
+    if constexpr (COLS) {
 #pragma unroll
-    for (int b = 0; b < 8; b += 2) {   // blocks b and b + 1 share a word of seeds and a word of coefficients
-        const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
-        const uint32_t seed[2] = {ss & 0xFFFFu, ss >> 16}, word[2] = {cc & 0xFFFFu, cc >> 16};
-        const uint32_t g[2] = {stream_of(tab, seed[0]), stream_of(tab, seed[1])}, up[2] = {ss << 16, ss};
-        int is[2][8], code[2];
-        if (P == 4) {
-            const uint32_t q01[2] = {tab[512 + (word[0] & 0xFFu)], tab[512 + (word[1] & 0xFFu)]};
-            const uint32_t q23[2] = {tab[512 + (word[0] >> 8)], tab[512 + (word[1] >> 8)]};
-            isum2_p4(up, g, q01, q23, is);
-            code[0] = (int) ((ck.codes >> (4 * b)) & 15u);
-            code[1] = (int) ((ck.codes >> (4 * b + 4)) & 15u);
-        } else {
+        for (int b = 0; b < 8; ++b) {
+            const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
+            const uint32_t g = stream_of(tab, (b & 1) ? ss >> 16 : ss & 0xFFFFu);
+            const uint32_t sl = __builtin_amdgcn_perm(g, ss, (b & 1) ? 0x05040302u : 0x05040100u);   // seed | g << 16
+            cols_dot<NT>(sl, g, coef_bytes(cc, b & 1), pow2f(eb + (int) ((ck.codes >> (4 * b)) & 15u)), b, xr, xstride, acc);
+        }
+    } else if constexpr (PAIRED) {
+#pragma unroll
+        for (int b = 0; b < 8; b += 2) {   // blocks b and b + 1 share a word of seeds and a word of nibble words
+            const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
+            const uint32_t seed[2] = {ss & 0xFFFFu, ss >> 16}, word[2] = {cc & 0xFFFFu, cc >> 16};
+            const uint32_t g[2] = {stream_of(tab, seed[0]), stream_of(tab, seed[1])}, up[2] = {ss << 16, ss};
+            int is[2][8];
             const uint32_t q01[2] = {tab[512 + ((word[0] >> 4) & 0xFFu)], tab[512 + ((word[1] >> 4) & 0xFFu)]};
             const uint32_t q2[2] = {tab[512 + (word[0] >> 12)], tab[512 + (word[1] >> 12)]};
             isum2_p3(up, g, q01, q2, is);
-            code[0] = (int) (word[0] & 15u);
-            code[1] = (int) (word[1] & 15u);
+            block_dot<P, NT>(is[0], pow2f(eb + (int) (word[0] & 15u)), b, xr, xstride, acc);
+            block_dot<P, NT>(is[1], pow2f(eb + (int) (word[1] & 15u)), b + 1, xr, xstride, acc);
         }
-        block_dot<P, NT>(is[0], pow2f(eb + code[0]), b, xr, xstride, acc);
-        block_dot<P, NT>(is[1], pow2f(eb + code[1]), b + 1, xr, xstride, acc);
-    }
     } else {
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-        const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
-        const uint32_t seed16 = (b & 1) ? ss >> 16 : ss & 0xFFFFu, word16 = (b & 1) ? cc >> 16 : cc & 0xFFFFu;
-        const uint32_t g = stream_of(tab, seed16);
-        const uint32_t up = (b & 1) ? ss : ss << 16;   // only the upper 16 bits are read
-        int is[8];
-        int code;
-        if (P == 4) {
-            isum_p4(up, g, tab[512 + (word16 & 0xFFu)], tab[512 + (word16 >> 8)], is);
-            code = (int) ((ck.codes >> (4 * b)) & 15u);
-        } else {
-            isum_p3(up, g, tab[512 + ((word16 >> 4) & 0xFFu)], tab[512 + (word16 >> 12)], is);
-            code = (int) (word16 & 15u);
+        for (int b = 0; b < 8; ++b) {
+            const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
+            const uint32_t seed16 = (b & 1) ? ss >> 16 : ss & 0xFFFFu, word16 = (b & 1) ? cc >> 16 : cc & 0xFFFFu;
+            const uint32_t g = stream_of(tab, seed16);
+            const uint32_t up = (b & 1) ? ss : ss << 16;   // only the upper 16 bits are read
+            int is[8];
+            if constexpr (P == 4) {   // the weights' form of a P = 4 block
+                isum_p4(up, g, tab[512 + (word16 & 0xFFu)], tab[512 + (word16 >> 8)], is);
+                block_dot<P, NT>(is, pow2f(eb + (int) ((ck.codes >> (4 * b)) & 15u)), b, xr, xstride, acc);
+            } else {
+                isum_p3(up, g, tab[512 + ((word16 >> 4) & 0xFFu)], tab[512 + (word16 >> 12)], is);
+                block_dot<P, NT>(is, pow2f(eb + (int) (word16 & 15u)), b, xr, xstride, acc);
+            }
         }
-        block_dot<P, NT>(is, pow2f(eb + code), b, xr, xstride, acc);
-    }
     }
 }
-
-#define XPAD 68   // LDS floats per 64-float chunk: 16-byte reads of 8 consecutive lanes land on 32 distinct banks
 
 // The 8 weights of block j of row r as f32: seeds unscaled integers with *sc = 2^e R32; BF16 / Q8 as BF16 values; Q4 in
 // MLX's matvec form s * q + b unrounded (reference engine/kernels_moe.cu:91-107, 171-189).

@@ -523,9 +523,12 @@ def test_mv_multi_affine_and_bf16_equal_separate_matvecs(fmt, T):
 @pytest.mark.parametrize("K,R", [(768, 300), (2048, 96), (256, 1000)])
 @pytest.mark.parametrize("T", [5, 16, 23, 64])
 def test_mv_many_tokens_equal_single_token_calls(fmt, K, R, T):
-    """kc_mv over T tokens (runs of four tokens dealt to grid.y) gives every token the bits of a one-token call: batch
-    invariance beyond the reference's 8 tokens (engine/kernels_moe.cu:239-240).  K = 768: 12 chunks a row, row sums through
-    LDS with more (token, row) sums than threads at four tokens; add = 1 accumulates into y."""
+    """kc_mv over T tokens (runs of four tokens dealt to grid.y).  Up to 8 tokens every token gets the bits of a one-token call,
+    the reference's batch invariance (engine/kernels_moe.cu:239-240).  Launches of more tokens may use another order of
+    operations (P = 4: the weights' form instead of the column form) but stay invariant among themselves: a token's bits
+    depend neither on its place nor on the others, checked against 9-token calls over shifted windows; P = 3 has one form
+    and equals the one-token calls at any T.  K = 768: 12 chunks a row, row sums through LDS with more (token, row) sums
+    than threads at four tokens; add = 1 accumulates into y."""
     import ctypes as C
     from nanoseedlm_amd import backend, moe
     backend.require_gpu()
@@ -543,14 +546,30 @@ def test_mv_many_tokens_equal_single_token_calls(fmt, K, R, T):
     x = packs.round_bf16(rng.standard_normal((T, K)).astype(np.float32))
     y0 = packs.round_bf16(rng.standard_normal((T, R)).astype(np.float32))
     dx = moe.DevBuf.from_array(x)
+    win = 1 if T <= 8 or fmt == packs.MF_SEED4 else 9
     for add in (0, 1):
         ya, yb = moe.DevBuf.from_array(y0), moe.DevBuf.from_array(y0)
         L.kc_mv(None, fmt, w, K, R, dx.ptr, K, ya.ptr, R, T, add, None)
-        for t in range(T):
-            L.kc_mv(None, fmt, w, K, R, dx.at(4 * t * K), K, yb.at(4 * t * R), R, 1, add, None)
+        t0 = 0
+        while t0 < T:                                  # windows of `win` tokens; the last one is cut short, not shifted back:
+            n = min(win, T - t0)                       # (an overlap would accumulate twice with add = 1)
+            if win > 1 and n < win:                    # ... a short tail joins tokens of the start again, into scratch rows
+                xt = np.concatenate([x[t0:], x[:win - n]])
+                yt = np.concatenate([y0[t0:], y0[:win - n]])
+                dxt, dyt = moe.DevBuf.from_array(xt), moe.DevBuf.from_array(yt)
+                L.kc_mv(None, fmt, w, K, R, dxt.ptr, K, dyt.ptr, R, win, add, None)
+                moe.device_sync()
+                tail = dyt.to_array(np.float32, (win, R))[:n]
+                dxt.free(); dyt.free()
+            else:
+                L.kc_mv(None, fmt, w, K, R, dx.at(4 * t0 * K), K, yb.at(4 * t0 * R), R, n, add, None)
+                tail = None
+            t0 += n
         moe.device_sync()
         assert L.kc_last_error() == 0
         a, b = ya.to_array(np.float32, (T, R)), yb.to_array(np.float32, (T, R))
+        if tail is not None:
+            b[T - len(tail):] = tail
         bad = np.argwhere(a.view(np.uint32) != b.view(np.uint32))
         assert not np.array_equal(a, y0) and len(bad) == 0, (add, len(bad), bad[:6].tolist())
         ya.free(); yb.free()
