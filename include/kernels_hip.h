@@ -265,6 +265,9 @@ void kc_fill_fp8_codes(kc_stream_t s, void* p, size_t nbytes, uint64_t seed);   
 size_t kc_moe_decode_sync_words(int T, int d);
 int kc_moe_decode_max_rows(void);
 int kc_moe_decode_error_word(void);
+/* polls a wait between workgroups makes before it gives up (0: the default, 2^21 - seconds).  A host that shares the GPU
+ * between streams may want a shorter bound; tests set a tiny one to drive the error path while every kernel still exits. */
+void kc_moe_decode_spin_limit(unsigned polls);
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                   int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                   int32_t* ind, float* wt, float* A, float* D, uint32_t* sync);

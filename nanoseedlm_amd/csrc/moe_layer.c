@@ -23,7 +23,9 @@ struct NslmMoe {
     MmTile* tiles;
     int max_tiles;
     uint32_t* sync;             /* device: the fused decode kernel's barrier words */
-    int fused;                  /* 1: steps of the softmax composition up to kc_moe_decode_max_rows() rows take kc_moe_decode */
+    int fused;                  /* 1: steps of the softmax composition up to kc_moe_decode_max_rows() rows take kc_moe_decode;
+                                   2: the same, and every such step is checked and redone by the separate launchers if it failed */
+    int fallbacks;              /* checked steps that were redone */
 };
 
 static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
@@ -227,7 +229,8 @@ int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, i
     if (!m->final || T < 1 || T > c->max_rows || layer < 0 || layer >= c->n_layer) return -1;
     const int E = c->n_exp;
     const WSlice* tab = m->pool.tab + (size_t) layer * 3 * E;
-    if (!(m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows())) return 1;
+    /* (a checked stack composes the block from nslm_moe_step, which can redo its part: this launch updates out in place) */
+    if (!(m->fused == 1 && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows())) return 1;
     if (kc_moe_decode_layer(s, c->fmt, m->rw + (size_t) layer * E * c->d, tab, tab + E, tab + 2 * E, E, c->top_k, c->d, c->ff, xn, c->d, T, out,
                             c->d, m->logit, m->ind, m->wt, m->A, m->D, m->sync, shared, res, norm_w, norm_eps))
         return 1;
@@ -243,8 +246,19 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
     const WSlice* down = m->pool.tab + ((size_t) layer * 3 + 2) * E;
     if (m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows() &&
         !kc_moe_decode(s, c->fmt, m->rw + (size_t) layer * E * d, gate, up, down, E, k, d, ff, xn, d, T, io, d, m->logit, m->ind,
-                       m->wt, m->A, m->D, m->sync))
-        return kc_last_error() ? -1 : 0;   /* the whole step in one persistent kernel */
+                       m->wt, m->A, m->D, m->sync)) {   /* the whole step in one persistent kernel */
+        if (m->fused != 2) return kc_last_error() ? -1 : 0;
+        /* checked: the kernel's workgroups wait for each other, and a wait that gave up (the grid was not resident at once:
+           another stream's kernel held the CUs) has left void results and the sync words in no defined state.  Then the words
+           are zeroed, the stack goes back to the separate launchers (until nslm_moe_set_fused turns the kernel on again) and
+           the step is redone by them: xn is untouched and io only written. */
+        uint32_t w = 0;
+        if (kc_last_error() || nh_stream_sync((nh_stream_t) s) || nh_memcpy_d2h(&w, m->sync + kc_moe_decode_error_word(), 4)) return -1;
+        if (!w) return 0;
+        if (nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d))) return -1;
+        m->fused = 0;
+        m->fallbacks++;
+    }
     if (c->router == NSLM_ROUTE_SOFTMAX) {
         WSlice rw;
         memset(&rw, 0, sizeof rw);
@@ -298,6 +312,8 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 }
 
 void nslm_moe_set_fused(NslmMoe* m, int on) { m->fused = on; }
+int nslm_moe_fused_mode(const NslmMoe* m) { return m->fused; }
+int nslm_moe_fallbacks(const NslmMoe* m) { return m->fallbacks; }
 void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }
 const uint16_t* nslm_moe_router_w(const NslmMoe* m, int layer) { return m->rw + (size_t) layer * m->c.n_exp * m->c.d; }
 int nslm_moe_fused_error(NslmMoe* m) {

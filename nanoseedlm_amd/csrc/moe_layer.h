@@ -49,8 +49,16 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out,
                         const float* norm_w, float norm_eps);   /* norm_w: xn is the raw stream, normalised inside (kq4_norm1p's values) */
 /* 1 (default): decode steps of the softmax composition with every expert resident run as one persistent kernel
- * (kc_moe_decode); 0: always the separate launchers.  The results are the same bits either way. */
+ * (kc_moe_decode); 0: always the separate launchers.  The results are the same bits either way.
+ * 2: as 1, checked - for hosts that run other streams beside the steps (the reference engine copies experts on a second
+ * stream, engine/mova_cuda.c:136-146): the kernel's workgroups wait for each other, and if they cannot all be resident a
+ * bounded wait gives up and the results are void.  In this mode nslm_moe_step synchronises s after the kernel, reads its
+ * error word and, if set, zeroes the sync words, redoes the step through the separate launchers and leaves the stack at
+ * mode 0; nslm_moe_fallbacks() counts these.  Not capturable (it synchronises); nslm_moe_step_layer answers 1 (not
+ * available) so that the caller composes the block around nslm_moe_step. */
 void nslm_moe_set_fused(NslmMoe* m, int on);
+int nslm_moe_fused_mode(const NslmMoe* m);
+int nslm_moe_fallbacks(const NslmMoe* m);
 /* 0, or non-zero when a grid barrier of the fused kernel gave up since open (synchronises) */
 int nslm_moe_fused_error(NslmMoe* m);
 /* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */

@@ -46,6 +46,7 @@ struct FusedArgs {
     int Lg, rpig, it_g, ntile_g;        // gate+up pass: chunks per row, virtual rows per iteration, iterations and items per pair
     int Ld, rpid, it_d, ntile_d;        // down pass (item i of a pair owns iterations i it / ntile .. (i + 1) it / ntile)
     int grid;
+    uint32_t spin;                      // polls a bounded wait makes before it gives up and sets the error word
 };
 
 // Words of the sync area (uint32; every counter sits alone on a 128-byte line = 32 words):
@@ -85,7 +86,7 @@ struct FusedArgs {
 #define FUSED_PAIR_WORDS (FUSED_IND_WORDS + 2 * FG_MAXT * 32)        // per-pair kernel: [MV_MAXT * 33 pairs][64]: arrivals, ready word
 #define FUSED_DFLAG_WORDS (FUSED_PAIR_WORDS + MV_MAXT * 33 * 64)     // per-pair kernel: [MV_MAXT][FUSED_TILES][33] finished down items
 #define FUSED_SYNC_WORDS (FUSED_DFLAG_WORDS + MV_MAXT * FUSED_TILES * 33)
-#define SPIN_LIMIT (1u << 21)
+#define SPIN_LIMIT (1u << 21)   // the default of FusedArgs::spin
 
 __device__ __forceinline__ uint32_t ld_agent(const uint32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -414,7 +415,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
                 unsigned long long w = ld_agent(lg64 + (size_t) t * a.E + e);
                 for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(lg64 + (size_t) t * a.E + e)) {
                     __builtin_amdgcn_s_sleep(2);
-                    if (++spins > SPIN_LIMIT) {
+                    if (++spins > a.spin) {
                         atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                         break;
                     }
@@ -525,7 +526,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             uint32_t spins = 0;
             while (ld_agent(&pairw[p * 64 + 32]) != tag) {
                 __builtin_amdgcn_s_sleep(2);
-                if (++spins > SPIN_LIMIT) {
+                if (++spins > a.spin) {
                     atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                     break;
                 }
@@ -552,7 +553,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
                 uint32_t spins = 0;
                 while (ld_agent(&dflag[((size_t) t * FUSED_TILES + tile) * 33 + tid]) != tag) {
                     __builtin_amdgcn_s_sleep(2);
-                    if (++spins > SPIN_LIMIT) {
+                    if (++spins > a.spin) {
                         atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                         break;
                     }
@@ -756,7 +757,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
                 unsigned long long w = ld_agent(lg64 + (size_t) t * a.E + e);
                 for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(lg64 + (size_t) t * a.E + e)) {
                     __builtin_amdgcn_s_sleep(2);
-                    if (++spins > SPIN_LIMIT) {
+                    if (++spins > a.spin) {
                         atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                         break;
                     }
@@ -796,7 +797,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             unsigned long long w = ld_agent(ind64 + (size_t) t * 32 + j);
             for (uint32_t spins = 0; (uint32_t) (w >> 32) != tag; w = ld_agent(ind64 + (size_t) t * 32 + j)) {
                 __builtin_amdgcn_s_sleep(2);
-                if (++spins > SPIN_LIMIT) {
+                if (++spins > a.spin) {
                     atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                     w = 0;   // expert 0: the results are void, the indices stay in range
                     break;
@@ -905,7 +906,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             uint32_t spins = 0;
             while (ld_agent(&grpc[g * 96 + 32]) == 0u) {
                 __builtin_amdgcn_s_sleep(2);
-                if (++spins > SPIN_LIMIT) {
+                if (++spins > a.spin) {
                     atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
                     break;
                 }
@@ -947,6 +948,8 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         }
     }
 }
+
+uint32_t g_spin_limit = SPIN_LIMIT;
 
 int cu_count() {
     static int n = 0;
@@ -1006,8 +1009,14 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // One token is at most a few hundred items more than three workgroups a CU hold (C2: 784): that launch may use the
     // registers of four waves a SIMD instead of five (107 instead of 96, no spills: 35.0 -> 34.5 us).
     const bool few = a.T == 1;
-    void (*kern)(FusedArgs) = few ? (sg ? (sd ? k_moe_decode<P, true, true, 4> : k_moe_decode<P, true, false, 4>)
-                                        : (sd ? k_moe_decode<P, false, true, 4> : k_moe_decode<P, false, false, 4>))
+#ifndef NSLM_FEW_WAVES
+#define NSLM_FEW_WAVES 4
+#endif
+#ifndef NSLM_WG_CAP
+#define NSLM_WG_CAP 5
+#endif
+    void (*kern)(FusedArgs) = few ? (sg ? (sd ? k_moe_decode<P, true, true, NSLM_FEW_WAVES> : k_moe_decode<P, true, false, NSLM_FEW_WAVES>)
+                                        : (sd ? k_moe_decode<P, false, true, NSLM_FEW_WAVES> : k_moe_decode<P, false, false, NSLM_FEW_WAVES>))
                                   : (sg ? (sd ? k_moe_decode<P, true, true, 5> : k_moe_decode<P, true, false, 5>)
                                         : (sd ? k_moe_decode<P, false, true, 5> : k_moe_decode<P, false, false, 5>));
     static int cached[2][2][2] = {};   // resident workgroups per CU, by kernel variant (same LDS request every call)
@@ -1025,9 +1034,13 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // takes more, shorter items than one round holds (C2, items a pair -> us; 4 tokens: 24 -> 82.2, 40 -> 79.6, 64 -> 78.0;
     // 6 tokens: 24 -> 120.2, 32 -> 111.4, 48 -> 115.2; 8 tokens: 20 -> 135.4, 32 -> 131.2, 48 -> 138.9); where the row sums go
     // through LDS (C3) one round stayed ahead.
-    const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
+    const int gmax = (per_cu < NSLM_WG_CAP ? per_cu : NSLM_WG_CAP) * cu_count(), P_ = a.T * a.kk;
     a.ntile_g = few || !sg ? pick_one_round(P_, a.it_g, gmax, FUSED_TILES) : pick_by_cu_load(P_, a.it_g, cu_count(), FUSED_TILES);
     a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES);
+#ifdef NSLM_FUSED_TUNE   // development builds: item counts from the environment
+    if (getenv("NSLM_NG")) a.ntile_g = atoi(getenv("NSLM_NG"));
+    if (getenv("NSLM_ND")) a.ntile_d = atoi(getenv("NSLM_ND"));
+#endif
     const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     int grid = items < gmax ? (int) items : gmax;
     if (grid < 1) grid = 1;
@@ -1131,6 +1144,7 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     if (fmt != MF_SEED4P4 && fmt != MF_SEED4) return -1;
     if (host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u)) return -1;
     FusedArgs a = {};
+    a.spin = g_spin_limit;
     bool sg, sd;
     if (!shape_of(d, true, &a.Lg, &a.rpig, &sg) || !shape_of(ff, false, &a.Ld, &a.rpid, &sd)) return -1;
     a.rw = router_w; a.gate = gate; a.up = up; a.down = down; a.x = x; a.out = out; a.logits = logits; a.wt = wt; a.A = A;
@@ -1155,6 +1169,8 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);
 }
+
+void kc_moe_decode_spin_limit(unsigned polls) { g_spin_limit = polls ? polls : SPIN_LIMIT; }
 
 int kc_moe_decode_static(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                          int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, int32_t* ind, float* wt,

@@ -141,6 +141,12 @@ class MoeStack:
     def set_fused(self, on):
         self.L.nslm_moe_set_fused(self.h, int(on))
 
+    def fused_mode(self):
+        return self.L.nslm_moe_fused_mode(self.h)
+
+    def fallbacks(self):
+        return self.L.nslm_moe_fallbacks(self.h)
+
     def fused_error(self):
         return self.L.nslm_moe_fused_error(self.h)
 

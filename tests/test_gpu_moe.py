@@ -317,3 +317,120 @@ def test_steps_of_changing_size_share_the_barrier_words():
     assert np.array_equal(first[13][:1].view(np.uint32), first[1].view(np.uint32))
     dx.free(); dio.free()
     st.close()
+
+
+def _small_stack(rng, E=32, k=4, d=512, ff=256, nl=2):
+    from nanoseedlm_amd import moe
+    st = moe.MoeStack(nl, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=24)
+    for l in range(nl):
+        gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, ff, d, eb=-21), packs.seed4p4(rng, E, d, ff, eb=-20)
+        st.set_layer(l, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+    st.finalize()
+    return st
+
+
+def _quiet_results(st, dx, dio, d, cases, fused):
+    """the steps with nothing else on the GPU: through the separate launchers (fused = 0) or the persistent kernel (1).  Up to
+    8 rows the two give the same bits; above, the launchers take the grouped GEMMs on BF16-rounded weights."""
+    st.set_fused(fused)
+    want = {}
+    for l, T in cases:
+        st.step(None, l, dx.ptr, T, dio.ptr)
+        want[(l, T)] = dio.to_array(np.float32, (24, d))[:T].copy()
+        assert np.abs(want[(l, T)]).max() > 0 and st.fused_error() == 0
+    return want
+
+
+def _same(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def test_checked_step_beside_another_streams_kernels():
+    """The persistent kernel's workgroups wait for each other, so its grid must be resident at once - which another stream's
+    kernels can prevent for a while (the reference engine runs a copy stream beside compute, engine/mova_cuda.c:136-146).
+    Here a queue of large GEMMs occupies the GPU on a second stream while checked steps (nslm_moe_set_fused(2)) run: every
+    step must return the separate launchers' bits, whether the kernel got through or the step was redone; the other stream's
+    queue is finite, so every wait ends and every kernel exits by itself."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(777)
+    d = 512
+    st = _small_stack(rng, d=d)
+    xn = packs.round_bf16(rng.standard_normal((24, d)).astype(np.float32))
+    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf(4 * 24 * d)
+    cases = [(l, T) for T in (1, 4, 8, 16) for l in (0, 1)]
+    want, wantf = _quiet_results(st, dx, dio, d, cases, 0), _quiet_results(st, dx, dio, d, cases, 1)
+    assert all(_same(want[c], wantf[c]) == (c[1] <= 8) for c in cases)
+    # the other stream's work: a dense seed GEMM 4096 x 4096 x 512 on device-filled records, a hundred times over
+    R = K = 4096
+    seeds, coefs, codes = moe.DevBuf(R * K // 8 * 2), moe.DevBuf(R * K // 8 * 2), moe.DevBuf(R * K // 16 // 2 * 2)
+    for i, b in enumerate((seeds, coefs, codes)):
+        L.kc_fill_random(None, b.ptr, C.c_size_t(b.nbytes), C.c_uint64(5 + i))
+    w = backend.WSlice()
+    w.p[0], w.p[1], w.p[3], w.eb = seeds.ptr.value, coefs.ptr.value, codes.ptr.value, -30
+    gx = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((512, K)).astype(np.float32)))
+    gy = moe.DevBuf(4 * 512 * R)
+    sa, sb = moe.new_stream(), moe.new_stream()
+    moe.device_sync()
+    st.set_fused(2)
+    for rep in range(3):
+        for i in range(100):
+            L.kc_mm(sb, packs.MF_SEED4P4, w, K, R, gx.ptr, K, gy.ptr, R, 512, 0, None)
+        for l, T in cases:
+            if st.fused_mode() == 0:      # a step was redone: the stack went back to the launchers; turn the kernel on again
+                st.set_fused(2)
+            st.step(sa, l, dx.ptr, T, dio.ptr)
+            backend.check(L.nh_stream_sync(sa), "nh_stream_sync")
+            got = dio.to_array(np.float32, (24, d))[:T]
+            assert _same(got, wantf[(l, T)]) or (st.fused_mode() == 0 and _same(got, want[(l, T)])), (rep, l, T, st.fallbacks())
+        moe.device_sync()
+        assert L.kc_last_error() == 0
+    print("steps redone by the launchers:", st.fallbacks())
+    st.set_fused(1)
+    assert st.fused_error() == 0          # whatever happened, the sync words are in order again
+    for b in (dx, dio, seeds, coefs, codes, gx, gy):
+        b.free()
+    st.close()
+
+
+def test_checked_step_is_redone_when_a_wait_gives_up():
+    """The error path, driven from the host: with a spin limit of one poll the first workgroup that finds a logit not yet
+    there gives up (every kernel still runs to its end).  A plain step then reports the error word; a checked step notices
+    it, zeroes the sync words, redoes the step through the launchers - the same bits - and leaves the stack on the
+    launchers.  With the limit back at its default the kernel can be turned on again and works on the zeroed words."""
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(778)
+    d = 512
+    st = _small_stack(rng, d=d)
+    xn = packs.round_bf16(rng.standard_normal((24, d)).astype(np.float32))
+    dx, dio = moe.DevBuf.from_array(xn), moe.DevBuf(4 * 24 * d)
+    cases = [(0, 1), (1, 8), (0, 16)]     # the per-pair kernel and the grouped one
+    want, wantf = _quiet_results(st, dx, dio, d, cases, 0), _quiet_results(st, dx, dio, d, cases, 1)
+    try:
+        for n, (l, T) in enumerate(cases):
+            L.kc_moe_decode_spin_limit(1)
+            st.set_fused(2)
+            st.step(None, l, dx.ptr, T, dio.ptr)
+            moe.device_sync()
+            assert st.fallbacks() == n + 1 and st.fused_mode() == 0, (l, T)
+            got = dio.to_array(np.float32, (24, d))[:T]
+            assert _same(got, want[(l, T)]), (l, T)
+            L.kc_moe_decode_spin_limit(0)
+            st.set_fused(1)                # on again, on the zeroed words: no error, the kernel's bits
+            for l2, T2 in cases:
+                st.step(None, l2, dx.ptr, T2, dio.ptr)
+                assert st.fused_error() == 0
+                got = dio.to_array(np.float32, (24, d))[:T2]
+                assert _same(got, wantf[(l2, T2)]), (l, T, l2, T2)
+        # unchecked, the same failure is reported by the error word (and the caller zeroes the words)
+        L.kc_moe_decode_spin_limit(1)
+        st.step(None, 0, dx.ptr, 1, dio.ptr)
+        assert st.fused_error() != 0
+    finally:
+        L.kc_moe_decode_spin_limit(0)
+    dx.free(); dio.free()
+    st.close()
