@@ -25,8 +25,23 @@ int nh_memcpy_d2h(void* dst, const void* src, size_t n);      /* cudaMemcpy(Devi
 int nh_memcpy_d2d(void* dst, const void* src, size_t n);      /* cudaMemcpy(DeviceToDevice) */
 int nh_memcpy_h2d_async(void* dst, const void* src, size_t n, nh_stream_t s);   /* cudaMemcpyAsync */
 int nh_memcpy_d2h_async(void* dst, const void* src, size_t n, nh_stream_t s);
+int nh_memcpy_d2d_async(void* dst, const void* src, size_t n, nh_stream_t s);   /* cudaMemcpyAsync(DeviceToDevice) */
+int nh_memcpy_async(void* dst, const void* src, size_t n, nh_stream_t s);       /* cudaMemcpyAsync(cudaMemcpyDefault): direction from the pointers */
 int nh_memset(void* p, int v, size_t n);                      /* cudaMemset */
+/* cudaMemsetAsync (engine/mova_cuda.c:1160): a fill kernel on s, not a memset node, so the call may be captured into a graph */
+int nh_memset_async(void* p, int v, size_t n, nh_stream_t s);
+/* cudaHostAlloc(cudaHostAllocMapped) + cudaHostGetDevicePointer (engine/mova_cuda.c:352, engine/qwen4_cuda.c:186,397): pinned host memory and the
+ * address kernels use for it (results a kernel leaves where the host polls them; pass dev = NULL to skip the second call) */
+int nh_host_alloc_mapped(void** host, void** dev, size_t n);
+int nh_host_device_ptr(void** dev, void* host);               /* cudaHostGetDevicePointer, for memory from nh_host_alloc */
+int nh_get_device(int* dev);                                  /* cudaGetDevice */
 int nh_stream_create(nh_stream_t* s);                         /* cudaStreamCreateWithFlags(NonBlocking), default priority */
+/* cudaDeviceGetStreamPriorityRange / cudaStreamCreateWithPriority (engine/mova_cuda.c:892, the copy stream): this layer
+ * has one priority - the range is [0, 0] and the priority asked for is ignored - because streams of different priorities
+ * are not used on these GPUs; a host that orders work by priority still runs, its streams then share the GPU evenly */
+int nh_stream_priority_range(int* least, int* greatest);
+int nh_stream_create_prio(nh_stream_t* s, int priority);
+int nh_event_create_untimed(nh_event_t* e);                   /* cudaEventCreateWithFlags(cudaEventDisableTiming) */
 int nh_stream_destroy(nh_stream_t s);
 int nh_stream_sync(nh_stream_t s);                            /* cudaStreamSynchronize */
 int nh_device_sync(void);                                     /* cudaDeviceSynchronize */

@@ -255,7 +255,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         uint32_t w = 0;
         if (kc_last_error() || nh_stream_sync((nh_stream_t) s) || nh_memcpy_d2h(&w, m->sync + kc_moe_decode_error_word(), 4)) return -1;
         if (!w) return 0;
-        if (nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d))) return -1;
+        if (nh_memset_async(m->sync, 0, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d), (nh_stream_t) s)) return -1;   /* on s: ordered before the stack's next kernel there */
         m->fused = 0;
         m->fallbacks++;
     }

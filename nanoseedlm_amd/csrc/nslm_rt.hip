@@ -5,6 +5,20 @@
 
 #include "nslm_rt.h"
 
+namespace {
+// nh_memset_async's fill: a kernel, so that the call can be captured into a graph (memset nodes gave wrong results on replays
+// after the first on these GPUs).  Whole 16-byte pieces by 16-byte stores, the ragged ends by bytes.
+__global__ void __launch_bounds__(256) k_fill_bytes(unsigned char* p, unsigned char v, size_t n) {
+    const size_t i0 = (size_t) blockIdx.x * 256 + threadIdx.x, step = (size_t) gridDim.x * 256;
+    const size_t head = (16 - ((uintptr_t) p & 15u)) & 15u, h = head < n ? head : n, mid = (n - h) / 16;
+    const unsigned w = v * 0x01010101u;
+    uint4* q = (uint4*) (p + h);
+    for (size_t i = i0; i < mid; i += step) q[i] = make_uint4(w, w, w, w);
+    for (size_t i = i0; i < h; i += step) p[i] = v;
+    for (size_t i = h + mid * 16 + i0; i < n; i += step) p[i] = v;
+}
+}   // namespace
+
 extern "C" {
 
 int nh_device_count(int* n) { return (int) hipGetDeviceCount(n); }
@@ -22,8 +36,39 @@ int nh_memcpy_h2d_async(void* dst, const void* src, size_t n, nh_stream_t s) {
 int nh_memcpy_d2h_async(void* dst, const void* src, size_t n, nh_stream_t s) {
     return n ? (int) hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, (hipStream_t) s) : 0;
 }
+int nh_memcpy_d2d_async(void* dst, const void* src, size_t n, nh_stream_t s) {
+    return n ? (int) hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, (hipStream_t) s) : 0;
+}
+int nh_memcpy_async(void* dst, const void* src, size_t n, nh_stream_t s) {
+    return n ? (int) hipMemcpyAsync(dst, src, n, hipMemcpyDefault, (hipStream_t) s) : 0;
+}
 int nh_memset(void* p, int v, size_t n) { return n ? (int) hipMemset(p, v, n) : 0; }
+int nh_memset_async(void* p, int v, size_t n, nh_stream_t s) {
+    if (!n) return 0;
+    size_t wg = (n / 16 + 255) / 256;
+    if (wg < 1) wg = 1;
+    if (wg > 4096) wg = 4096;
+    hipLaunchKernelGGL(k_fill_bytes, dim3((unsigned) wg), dim3(256), 0, (hipStream_t) s, (unsigned char*) p, (unsigned char) v, n);
+    return (int) hipGetLastError();
+}
+int nh_host_alloc_mapped(void** host, void** dev, size_t n) {
+    const hipError_t e = hipHostMalloc(host, n ? n : 16, hipHostMallocMapped);
+    if (e != hipSuccess) return (int) e;
+    return dev ? (int) hipHostGetDevicePointer(dev, *host, 0) : 0;
+}
+int nh_host_device_ptr(void** dev, void* host) { return (int) hipHostGetDevicePointer(dev, host, 0); }
+int nh_get_device(int* dev) { return (int) hipGetDevice(dev); }
 int nh_stream_create(nh_stream_t* s) { return (int) hipStreamCreateWithFlags((hipStream_t*) s, hipStreamNonBlocking); }
+int nh_stream_priority_range(int* least, int* greatest) {   // one priority: every stream of this library is a default-priority stream
+    if (least) *least = 0;
+    if (greatest) *greatest = 0;
+    return 0;
+}
+int nh_stream_create_prio(nh_stream_t* s, int priority) {
+    (void) priority;
+    return nh_stream_create(s);
+}
+int nh_event_create_untimed(nh_event_t* e) { return (int) hipEventCreateWithFlags((hipEvent_t*) e, hipEventDisableTiming); }
 int nh_stream_destroy(nh_stream_t s) { return (int) hipStreamDestroy((hipStream_t) s); }
 int nh_stream_sync(nh_stream_t s) { return (int) hipStreamSynchronize((hipStream_t) s); }
 int nh_device_sync(void) { return (int) hipDeviceSynchronize(); }
