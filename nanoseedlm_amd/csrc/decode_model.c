@@ -88,7 +88,7 @@ NslmModel* nslm_model_open(const NslmModelCfg* c, char* err, int errlen) {
     if (m) m->next_pos = -1;
     m->c = *c;
     if (m->c.n_splits <= 0) m->c.n_splits = 32;
-    NslmMoeCfg mc = {c->n_layer, c->n_exp, c->top_k, c->d, c->ff, MF_SEED4P4, NSLM_ROUTE_SOFTMAX, c->max_rows, 0, 1.0f};
+    NslmMoeCfg mc = {c->n_layer, c->n_exp, c->top_k, c->d, c->ff, MF_SEED4P4, NSLM_ROUTE_SOFTMAX, c->max_rows, 0, 1.0f, 0, 0};
     m->moe = nslm_moe_open(&mc, err, errlen);
     if (!m->moe) { free(m); return NULL; }
     /* the dense seeded matrices of a layer, each stream at a 256-byte aligned offset of the layer's block */

@@ -13,7 +13,14 @@ struct NslmMoe {
     int units, resident, final;
     uint64_t unit_bytes, stream_len[3][4];
     CachePool pool;             /* device pointers inside */
-    uint8_t* arena;             /* device: every unit */
+    uint8_t* arena;             /* every unit: device memory, or (host_units) the device address of pinned host memory */
+    uint8_t* arena_host;        /* host_units: the same memory as the host sees it */
+    CachePool pool_pre;         /* prefetch: the pool with job lists and statistics of its own (two producers never share a list) */
+    nh_stream_t cst;            /* prefetch: the copy stream */
+    nh_event_t ev_admit, *ev_pred;   /* prefetch: admit done on the step's stream; layer l's predicted experts copied */
+    int pred_pending;           /* layer whose predicted experts are being copied, or -1 */
+    float *plogit, *pscore, *pwt;
+    int32_t* pind;
     uint8_t* unit_host;         /* staging for one unit */
     int32_t* eb;                /* host: [units][3] exponent biases */
     uint16_t *rw, *rb;          /* device: router weights [layer][n_exp][d], biases [layer][n_exp] */
@@ -66,7 +73,8 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     const int P = c->max_rows * (c->top_k + 1);   /* + 1: the shared expert's pair in nslm_moe_step_layer */
     m->max_tiles = P / MMT_BN + c->n_exp + 1;
     int bad = 0;
-    bad |= nh_malloc((void**) &m->arena, cur * (uint64_t) m->units);
+    if (c->host_units) bad |= nh_host_alloc_mapped((void**) &m->arena_host, (void**) &m->arena, cur * (uint64_t) m->units);
+    else bad |= nh_malloc((void**) &m->arena, cur * (uint64_t) m->units);
     if (m->resident) m->pool.vram = m->arena;
     else bad |= nh_malloc((void**) &m->pool.vram, cur * (uint64_t) m->pool.slots);
     m->pool.host = m->arena;
@@ -95,6 +103,22 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 3));
     bad |= nh_malloc((void**) &m->sync, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d));
     m->fused = 1;
+    m->pred_pending = -1;
+    if (c->prefetch && !m->resident && c->router == NSLM_ROUTE_SIGMOID) {
+        m->pool_pre = m->pool;   /* the table and the slots are shared; filled in again by nslm_moe_finalize */
+        bad |= nh_malloc((void**) &m->pool_pre.jobs, 8 * (size_t) c->n_exp);
+        bad |= nh_malloc((void**) &m->pool_pre.njobs, 16);
+        bad |= nh_malloc((void**) &m->pool_pre.stats, 16);
+        bad |= nh_malloc((void**) &m->plogit, 4 * (size_t) c->max_rows * c->n_exp);
+        bad |= nh_malloc((void**) &m->pscore, 4 * (size_t) c->max_rows * c->n_exp);
+        bad |= nh_malloc((void**) &m->pwt, 4 * (size_t) P);
+        bad |= nh_malloc((void**) &m->pind, 4 * (size_t) P);
+        bad |= nh_stream_create_prio(&m->cst, 0);
+        bad |= nh_event_create_untimed(&m->ev_admit);
+        m->ev_pred = (nh_event_t*) calloc((size_t) c->n_layer, sizeof(nh_event_t));
+        for (int l = 0; m->ev_pred && l < c->n_layer; ++l) bad |= nh_event_create_untimed(&m->ev_pred[l]);
+        if (!m->ev_pred) bad = 1;
+    }
     m->unit_host = (uint8_t*) calloc(1, cur);
     m->eb = (int32_t*) calloc((size_t) m->units * 3, 4);
     if (bad || !m->unit_host || !m->eb) {
@@ -110,6 +134,21 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
 
 void nslm_moe_close(NslmMoe* m) {
     if (!m) return;
+    if (m->cst) {
+        nh_stream_sync(m->cst);
+        nh_stream_destroy(m->cst);
+        nh_event_destroy(m->ev_admit);
+        for (int l = 0; m->ev_pred && l < m->c.n_layer; ++l)
+            if (m->ev_pred[l]) nh_event_destroy(m->ev_pred[l]);
+        free(m->ev_pred);
+        void* pd[] = {m->pool_pre.jobs, m->pool_pre.njobs, m->pool_pre.stats, m->plogit, m->pscore, m->pwt, m->pind};
+        for (size_t i = 0; i < sizeof pd / sizeof pd[0]; ++i)
+            if (pd[i]) nh_free(pd[i]);
+    }
+    if (m->arena_host) {
+        nh_host_free(m->arena_host);
+        m->arena = NULL;
+    }
     void* d[] = {m->arena, m->resident ? NULL : m->pool.vram, m->pool.unit_slot, m->pool.slot_unit, m->pool.slot_last, m->pool.tick,
                  m->pool.stats, m->pool.jobs, m->pool.njobs, m->pool.tab, m->rw, m->rb, m->logit, m->score, m->wt, m->ind, m->A,
                  m->G, m->U, m->D, m->zero, m->perm, m->tiles, m->ntiles, m->sync, m->px};
@@ -120,14 +159,21 @@ void nslm_moe_close(NslmMoe* m) {
     free(m);
 }
 
+/* host bytes into the arena: a copy to the device, or a plain copy where the arena is host memory */
+static int arena_write(NslmMoe* m, uint8_t* dst, const void* src, uint64_t n) {
+    if (!m->arena_host) return nh_memcpy_h2d(dst, src, n);
+    memcpy(m->arena_host + (dst - m->arena), src, n);
+    return 0;
+}
+
 int nslm_moe_set_expert(NslmMoe* m, int layer, int expert, int tensor, const uint16_t* seeds, const uint16_t* words,
                         const uint8_t* codes, int eb) {
     if (layer < 0 || layer >= m->c.n_layer || expert < 0 || expert >= m->c.n_exp || tensor < 0 || tensor > 2) return -1;
     const int u = layer * m->c.n_exp + expert;
     uint8_t* base = m->arena + (uint64_t) u * m->unit_bytes;
-    int e = nh_memcpy_h2d(base + m->pool.off[tensor][0], seeds, m->stream_len[tensor][0]);
-    e |= nh_memcpy_h2d(base + m->pool.off[tensor][1], words, m->stream_len[tensor][1]);
-    if (m->c.fmt == MF_SEED4P4) e |= nh_memcpy_h2d(base + m->pool.off[tensor][3], codes, m->stream_len[tensor][3]);
+    int e = arena_write(m, base + m->pool.off[tensor][0], seeds, m->stream_len[tensor][0]);
+    e |= arena_write(m, base + m->pool.off[tensor][1], words, m->stream_len[tensor][1]);
+    if (m->c.fmt == MF_SEED4P4) e |= arena_write(m, base + m->pool.off[tensor][3], codes, m->stream_len[tensor][3]);
     m->eb[u * 3 + tensor] = eb;
     return e ? -1 : 0;
 }
@@ -154,7 +200,8 @@ int nslm_moe_load_experts(NslmMoe* m, int layer, int which, const NsfTensor* t) 
             if (s == 2 || !m->stream_len[which][s]) continue;
             const uint64_t n = m->stream_len[which][s];
             if (t->s[s].len != n * (uint64_t) m->c.n_exp) return -1;
-            bad |= nsf_upload(base + m->pool.off[which][s], &t->s[s], (uint64_t) e * n, n);
+            if (m->arena_host) memcpy(m->arena_host + (base - m->arena) + m->pool.off[which][s], t->s[s].p + (uint64_t) e * n, n);
+            else bad |= nsf_upload(base + m->pool.off[which][s], &t->s[s], (uint64_t) e * n, n);
         }
         int32_t eb;
         memcpy(&eb, t->s[2].p + 4 * (size_t) e, 4);
@@ -195,7 +242,8 @@ int nslm_moe_finalize(NslmMoe* m) {
                 const int u = sl * E + x;
                 us[u] = s;
                 su[s] = u;
-                bad |= nh_memcpy_d2d(m->pool.vram + (uint64_t) s * m->unit_bytes, m->arena + (uint64_t) u * m->unit_bytes, m->unit_bytes);
+                if (m->arena_host) bad |= nh_memcpy_h2d(m->pool.vram + (uint64_t) s * m->unit_bytes, m->arena_host + (uint64_t) u * m->unit_bytes, m->unit_bytes);
+                else bad |= nh_memcpy_d2d(m->pool.vram + (uint64_t) s * m->unit_bytes, m->arena + (uint64_t) u * m->unit_bytes, m->unit_bytes);
             }
     }
     for (int sl = 0; sl < nl; ++sl)
@@ -215,6 +263,14 @@ int nslm_moe_finalize(NslmMoe* m) {
     bad |= nh_memset(m->pool.njobs, 0, 16);
     bad |= nh_memset(m->pool.stats, 0, 16);
     bad |= nh_memcpy_h2d(m->pool.tab, tab, sizeof(WSlice) * (size_t) units * 3);
+    if (m->cst) {   /* the prefetch's view: the same table and slots, its own job list and counters */
+        CachePool pre = m->pool;
+        pre.jobs = m->pool_pre.jobs; pre.njobs = m->pool_pre.njobs; pre.stats = m->pool_pre.stats;
+        m->pool_pre = pre;
+        bad |= nh_memset(pre.njobs, 0, 16);
+        bad |= nh_memset(pre.stats, 0, 16);
+    }
+    bad |= nh_device_sync();
     free(us); free(su); free(tab);
     m->final = !bad;
     return bad ? -1 : 0;
@@ -281,8 +337,24 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         kc_router(s, ra, m->rw + (size_t) layer * E * d, m->rb + (size_t) layer * E, xn, m->logit, m->score, m->ind, m->wt, T);
     }
     if (!m->resident) {   /* with every expert resident the table never changes: nothing to admit, nothing to copy */
+        if (m->pred_pending == layer) {   /* the predicted experts' copies land before the table is consulted */
+            nh_stream_wait_event((nh_stream_t) s, m->ev_pred[layer]);
+            m->pred_pending = -1;
+        }
         kc_cache_admit(s, &m->pool, layer, m->ind, P, 0);
         kc_cache_copy(s, &m->pool, 64);
+        if (m->cst && T <= MV_MAXT && layer + 1 < c->n_layer) {
+            /* decode: the next layer's likely experts, from its router on this layer's input; their slots may not be the ones
+               this layer's gathers are about to read (CACHE_PROTECT_PREV), and their copies run beside those gathers */
+            RouterArgs ra = {d, E, k, d / 2, c->route_scale};
+            kc_router(s, ra, m->rw + (size_t) (layer + 1) * E * d, m->rb + (size_t) (layer + 1) * E, xn, m->plogit, m->pscore, m->pind, m->pwt, T);
+            kc_cache_admit(s, &m->pool_pre, layer + 1, m->pind, P, CACHE_PROTECT_PREV);
+            nh_event_record(m->ev_admit, (nh_stream_t) s);
+            nh_stream_wait_event(m->cst, m->ev_admit);
+            kc_cache_copy((kc_stream_t) m->cst, &m->pool_pre, 8);
+            nh_event_record(m->ev_pred[layer + 1], m->cst);
+            m->pred_pending = layer + 1;
+        }
     }
     if (T <= MV_MAXT) {   /* decode: one gather pass per (token, expert) pair (engine/mova_cuda.c:1301-1307) */
         kc_mv_gu(s, c->fmt, gate, up, d, ff, xn, d, m->A, ff, m->ind, P, k, NULL);
@@ -329,6 +401,14 @@ int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {
 int nslm_moe_last_pairs(NslmMoe* m, int pairs, float* A, float* D) {
     if (nh_device_sync()) return -1;
     return (nh_memcpy_d2h(A, m->A, 4 * (size_t) pairs * m->c.ff) | nh_memcpy_d2h(D, m->D, 4 * (size_t) pairs * m->c.d)) ? -1 : 0;
+}
+int nslm_moe_prefetch_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses) {
+    uint32_t st[2] = {0, 0};
+    if (!m->cst) return -1;
+    if (nh_device_sync() || nh_memcpy_d2h(st, m->pool_pre.stats, 8)) return -1;
+    *hits = st[0];
+    *misses = st[1];
+    return 0;
 }
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses) {
     uint32_t st[2] = {0, 0};

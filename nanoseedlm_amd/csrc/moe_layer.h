@@ -24,6 +24,12 @@ typedef struct {
     int max_rows;  /* most tokens a step takes */
     int slots;     /* pool slots; 0 or >= n_layer * n_exp: all resident */
     float route_scale;
+    int host_units; /* 1: the experts' units live in pinned host memory that the GPU reads (the reference's layout where the expert
+                      set exceeds device memory, engine/mova_cuda.c:340-360); the pool's slots are the only copies in HBM */
+    int prefetch;   /* 1 (sigmoid composition, a pool smaller than the expert set, decode steps): after a layer's own experts are
+                      admitted, the next layer's router is run on this layer's input, its likely experts are admitted with
+                      CACHE_PROTECT_PREV and copied on a second stream, and the next layer's admit waits for that copy
+                      (engine/mova_cuda.c:1283-1303) */
 } NslmMoeCfg;
 
 typedef struct NslmMoe NslmMoe;
@@ -69,6 +75,8 @@ int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
 int nslm_moe_last_pairs(NslmMoe* m, int pairs, float* A, float* D);
 /* the slot table's counters and state (synchronises): hits, misses since open */
 int nslm_moe_cache_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
+/* the prefetch's own counters (synchronises): predicted experts already resident, predicted experts copied ahead */
+int nslm_moe_prefetch_stats(NslmMoe* m, uint32_t* hits, uint32_t* misses);
 /* the device slice table [n_exp] of a layer's tensor (0 gate, 1 up, 2 down): what kc_mv_gu / kc_mv_sel take */
 const WSlice* nslm_moe_tab(const NslmMoe* m, int layer, int tensor);
 /* the device address of a layer's BF16 router weight [n_exp][d] */

@@ -11,7 +11,8 @@ ROUTE_SOFTMAX, ROUTE_SIGMOID = 0, 1
 
 class NslmMoeCfg(C.Structure):
     _fields_ = [("n_layer", C.c_int), ("n_exp", C.c_int), ("top_k", C.c_int), ("d", C.c_int), ("ff", C.c_int), ("fmt", C.c_int),
-                ("router", C.c_int), ("max_rows", C.c_int), ("slots", C.c_int), ("route_scale", C.c_float)]
+                ("router", C.c_int), ("max_rows", C.c_int), ("slots", C.c_int), ("route_scale", C.c_float), ("host_units", C.c_int),
+                ("prefetch", C.c_int)]
 
 
 def _lib():
@@ -84,10 +85,10 @@ class MoeStack:
     """n_layer routed-expert layers resident in HBM: experts from seeded packs, one BF16 router per layer."""
 
     def __init__(self, n_layer, n_exp, top_k, d, ff, fmt=packs.MF_SEED4P4, router=ROUTE_SOFTMAX, max_rows=8, slots=0,
-                 route_scale=1.0):
+                 route_scale=1.0, host_units=0, prefetch=0):
         backend.require_gpu()
         self.L = _lib()
-        self.cfg = NslmMoeCfg(n_layer, n_exp, top_k, d, ff, fmt, router, max_rows, slots, route_scale)
+        self.cfg = NslmMoeCfg(n_layer, n_exp, top_k, d, ff, fmt, router, max_rows, slots, route_scale, host_units, prefetch)
         err = C.create_string_buffer(256)
         self.h = C.c_void_p(self.L.nslm_moe_open(C.byref(self.cfg), err, 256))
         if not self.h:
@@ -136,6 +137,12 @@ class MoeStack:
         h, m = C.c_uint32(0), C.c_uint32(0)
         if self.L.nslm_moe_cache_stats(self.h, C.byref(h), C.byref(m)):
             raise RuntimeError("nslm_moe_cache_stats failed")
+        return h.value, m.value
+
+    def prefetch_stats(self):
+        h, m = C.c_uint32(0), C.c_uint32(0)
+        if self.L.nslm_moe_prefetch_stats(self.h, C.byref(h), C.byref(m)):
+            raise RuntimeError("nslm_moe_prefetch_stats failed")
         return h.value, m.value
 
     def set_fused(self, on):

@@ -434,3 +434,57 @@ def test_checked_step_is_redone_when_a_wait_gives_up():
         L.kc_moe_decode_spin_limit(0)
     dx.free(); dio.free()
     st.close()
+
+
+def test_engine_order_host_units_and_next_layer_prefetch():
+    """The reference engine's expert block in its own order on the runtime layer (engine/mova_cuda.c:1279-1325): sigmoid router ->
+    wait for the predicted experts' copies -> admit -> copy -> next layer's router on this layer's input, admit with
+    CACHE_PROTECT_PREV, copies on a second stream behind an event -> gathers -> combine; the experts' units in pinned host
+    memory that the copy kernel reads through its device address (:340-360), a pool of 24 slots for 48 experts.
+    Residency must never change a result: the same steps on a stack with every expert resident in HBM, on the host-unit pool
+    without prefetch and on it with prefetch give the same bits, and the prefetch turns demand misses into hits."""
+    from nanoseedlm_amd import moe
+    rng = np.random.default_rng(909)
+    nl, E, k, d, ff = 3, 16, 4, 256, 128
+    layers = []
+    for l in range(nl):
+        gate, up, down = packs.seed4(rng, E, ff, d, eb=-21), packs.seed4(rng, E, ff, d, eb=-21), packs.seed4(rng, E, d, ff, eb=-20)
+        rw = packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32))
+        rb = packs.f32_to_bf16_bits((rng.standard_normal(E) * 0.01).astype(np.float32))
+        layers.append((gate, up, down, rw, rb))
+    stacks = []
+    for slots, host_units, prefetch in ((0, 0, 0), (24, 1, 0), (24, 1, 1)):
+        st = moe.MoeStack(nl, E, k, d, ff, fmt=packs.MF_SEED4, router=moe.ROUTE_SIGMOID, max_rows=8, slots=slots, route_scale=2.5,
+                          host_units=host_units, prefetch=prefetch)
+        for l, lay in enumerate(layers):
+            st.set_layer(l, *lay)
+        st.finalize()
+        stacks.append(st)
+    s = moe.new_stream()
+    r = packs.round_bf16
+    for rep in range(6):
+        T = (1, 3, 8, 2, 5, 1)[rep]
+        x = r(rng.standard_normal((T, d)).astype(np.float32))          # the residual stream, through the three layers
+        xs = [moe.DevBuf.from_array(x) for _ in stacks]
+        for l in range(nl):
+            xn = r(rng.standard_normal((T, d)).astype(np.float32))     # (stands for the layer's norm output)
+            dxn = moe.DevBuf.from_array(xn)
+            outs = []
+            for st, dio in zip(stacks, xs):
+                st.step(s, l, dxn.ptr, T, dio.ptr)
+                moe.device_sync()
+                outs.append(dio.to_array(np.float32, (T, d)))
+            assert not np.array_equal(outs[0], x)
+            for o in outs[1:]:
+                assert np.array_equal(o.view(np.uint32), outs[0].view(np.uint32)), (rep, l)
+            dxn.free()
+        for b in xs:
+            b.free()
+    h0, m0 = stacks[1].cache_stats()
+    h1, m1 = stacks[2].cache_stats()
+    ph, pm = stacks[2].prefetch_stats()
+    print(f"demand hits/misses without prefetch {h0}/{m0}, with {h1}/{m1}; predicted: resident already {ph}, copied ahead {pm}")
+    assert h0 + m0 == h1 + m1 and m0 > 0          # the same requests; 24 slots for 48 experts must evict
+    assert pm > 0 and m1 < m0                      # experts copied ahead of their layer are hits when it comes
+    for st in stacks:
+        st.close()
