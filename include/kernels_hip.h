@@ -144,6 +144,16 @@ void kc_swiglu(kc_stream_t s, const float* g, const float* u, float* a, int n);
 /* kc_swiglu + kc_pack_input_bf16 in one pass (no counterpart in the reference): y = the BF16 bits of kc_swiglu's values,
  * n % 8 == 0, g / u / y 16-byte aligned, y distinct from g and u */
 void kc_swiglu_pack(kc_stream_t s, const float* g, const float* u, uint16_t* y, size_t n);
+/* The batched step's first two launches folded (no counterpart in the reference, which routes, packs and groups in four):
+ * kc_mv_pack = kc_mv of a BF16 / Q8 / Q4 matrix (add = 0) for up to 64 rows in ONE launch, on the rows rounded to BF16 as the
+ * GEMM it stands in for multiplies them (engine/kernels_moe.cu:455-470; kc_mv's row sums over those values), that also
+ * leaves the rows' BF16 view px [T][K] (kc_pack_input_bf16's bits) for the GEMMs that follow; returns -1 (nothing launched)
+ * where kc_mv would not take its wave-a-row path (K % 8, x or px not 16-byte aligned, xs % 4, K > 4096 rows' worth of LDS).
+ * kq4_route_bucket = kq4_route + kc_bucket in one launch: ind / wt as kq4_route's, perm / tiles / ntiles as kc_bucket's for
+ * count = T * top_k; ntiles holds 2 * n_exp + 4 ints here, the last one zero before the first call (the launch leaves it zero). */
+int kc_mv_pack(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int xs, float* y, int ys, int T, uint16_t* px);
+void kq4_route_bucket(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int32_t* ind, float* wt, int T, int32_t* perm,
+                      MmTile* tiles, int32_t* ntiles);
 void kc_moe_combine(kc_stream_t s, const float* D, const float* w, const float* shared, float* x, int d, int k, int T);
 /* engine/kernels_qwen4.h:71, engine/kernels_qwen4.cu:514-516 */
 void kq4_moe_combine(kc_stream_t s, int d, int k, const float* D, const float* wt, const float* sh, const float* sg,

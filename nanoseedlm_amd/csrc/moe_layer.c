@@ -100,7 +100,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     bad |= nh_malloc((void**) &m->zero, 4 * (size_t) c->max_rows * c->d);
     bad |= nh_malloc((void**) &m->perm, 4 * (size_t) P);
     bad |= nh_malloc((void**) &m->tiles, sizeof(MmTile) * (size_t) m->max_tiles);
-    bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 3));
+    bad |= nh_malloc((void**) &m->ntiles, 4 * (size_t) (2 * c->n_exp + 4));   /* + kq4_route_bucket's ticket word */
     bad |= nh_malloc((void**) &m->sync, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d));
     m->fused = 1;
     m->pred_pending = -1;
@@ -129,6 +129,7 @@ NslmMoe* nslm_moe_open(const NslmMoeCfg* c, char* err, int errlen) {
     nh_memset(m->zero, 0, 4 * (size_t) c->max_rows * c->d);
     nh_memset(m->sync, 0, 4 * kc_moe_decode_sync_words(kc_moe_decode_max_rows(), c->d));
     nh_memset(m->rb, 0, 2 * (size_t) c->n_layer * c->n_exp);
+    nh_memset(m->ntiles, 0, 4 * (size_t) (2 * c->n_exp + 4));
     return m;
 }
 
@@ -315,6 +316,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         m->fused = 0;
         m->fallbacks++;
     }
+    int routed_and_grouped = 0;
     if (c->router == NSLM_ROUTE_SOFTMAX) {
         WSlice rw;
         memset(&rw, 0, sizeof rw);
@@ -325,13 +327,25 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         qc.top_k = k;
         if (T <= MV_MAXT) {
             kc_mv(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
-        } else if (d % 8 == 0 && ff % 8 == 0) {   /* the batched path's BF16 view of xn, made once and used three times */
-            kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);
-            kc_mm_packed(s, MF_BF16, rw, d, E, m->px, d, m->logit, E, T, 0, NULL);
+            kq4_route(s, &qc, m->logit, m->ind, m->wt, T);
         } else {
-            kc_mm(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+            /* The batched path: the logits by the decode path's row sums over the input rounded to BF16, as the GEMM
+               multiplies it (a 128-row GEMM is two workgroups: 16 us where this takes 5), the BF16 view of xn that the
+               three GEMMs read made by the same launch;
+               then routing and grouping in one launch.  Shapes the folded launches do not take go the reference's way
+               (engine/qwen4_cuda.c:1033-1034, 1058-1061: router matvec or GEMM, route, bucket). */
+            const int packed = d % 8 == 0 && ff % 8 == 0;
+            if (!(packed && T <= 64 && !kc_mv_pack(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, m->px))) {
+                if (packed) {
+                    kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);
+                    kc_mm_packed(s, MF_BF16, rw, d, E, m->px, d, m->logit, E, T, 0, NULL);
+                } else {
+                    kc_mm(s, MF_BF16, rw, d, E, xn, d, m->logit, E, T, 0, NULL);
+                }
+            }
+            kq4_route_bucket(s, &qc, m->logit, m->ind, m->wt, T, m->perm, m->tiles, m->ntiles);
+            routed_and_grouped = 1;
         }
-        kq4_route(s, &qc, m->logit, m->ind, m->wt, T);
     } else {
         RouterArgs ra = {d, E, k, d / 2, c->route_scale};
         kc_router(s, ra, m->rw + (size_t) layer * E * d, m->rb + (size_t) layer * E, xn, m->logit, m->score, m->ind, m->wt, T);
@@ -363,7 +377,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         /* BF16 views of the activations feed the MFMA path, as the reference's packed_layer() case does
            (engine/mova_cuda.c:1012-1035,1229,1308-1317): SwiGLU writes A as that view directly */
         const int packed = d % 8 == 0 && ff % 8 == 0;
-        kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
+        if (!routed_and_grouped) kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
         if (packed) {
             if (c->router != NSLM_ROUTE_SOFTMAX) kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);   /* else: made for the router */
             kc_mm_grouped_packed(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);

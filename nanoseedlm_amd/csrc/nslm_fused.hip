@@ -1009,14 +1009,8 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // One token is at most a few hundred items more than three workgroups a CU hold (C2: 784): that launch may use the
     // registers of four waves a SIMD instead of five (107 instead of 96, no spills: 35.0 -> 34.5 us).
     const bool few = a.T == 1;
-#ifndef NSLM_FEW_WAVES
-#define NSLM_FEW_WAVES 4
-#endif
-#ifndef NSLM_WG_CAP
-#define NSLM_WG_CAP 5
-#endif
-    void (*kern)(FusedArgs) = few ? (sg ? (sd ? k_moe_decode<P, true, true, NSLM_FEW_WAVES> : k_moe_decode<P, true, false, NSLM_FEW_WAVES>)
-                                        : (sd ? k_moe_decode<P, false, true, NSLM_FEW_WAVES> : k_moe_decode<P, false, false, NSLM_FEW_WAVES>))
+    void (*kern)(FusedArgs) = few ? (sg ? (sd ? k_moe_decode<P, true, true, 4> : k_moe_decode<P, true, false, 4>)
+                                        : (sd ? k_moe_decode<P, false, true, 4> : k_moe_decode<P, false, false, 4>))
                                   : (sg ? (sd ? k_moe_decode<P, true, true, 5> : k_moe_decode<P, true, false, 5>)
                                         : (sd ? k_moe_decode<P, false, true, 5> : k_moe_decode<P, false, false, 5>));
     static int cached[2][2][2] = {};   // resident workgroups per CU, by kernel variant (same LDS request every call)
@@ -1034,13 +1028,9 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // takes more, shorter items than one round holds (C2, items a pair -> us; 4 tokens: 24 -> 82.2, 40 -> 79.6, 64 -> 78.0;
     // 6 tokens: 24 -> 120.2, 32 -> 111.4, 48 -> 115.2; 8 tokens: 20 -> 135.4, 32 -> 131.2, 48 -> 138.9); where the row sums go
     // through LDS (C3) one round stayed ahead.
-    const int gmax = (per_cu < NSLM_WG_CAP ? per_cu : NSLM_WG_CAP) * cu_count(), P_ = a.T * a.kk;
+    const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
     a.ntile_g = few || !sg ? pick_one_round(P_, a.it_g, gmax, FUSED_TILES) : pick_by_cu_load(P_, a.it_g, cu_count(), FUSED_TILES);
     a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES);
-#ifdef NSLM_FUSED_TUNE   // development builds: item counts from the environment
-    if (getenv("NSLM_NG")) a.ntile_g = atoi(getenv("NSLM_NG"));
-    if (getenv("NSLM_ND")) a.ntile_d = atoi(getenv("NSLM_ND"));
-#endif
     const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     int grid = items < gmax ? (int) items : gmax;
     if (grid < 1) grid = 1;

@@ -90,22 +90,23 @@ __device__ __forceinline__ uint32_t float_order(float v) {
     const uint32_t b = __float_as_uint(v + 0.0f);   // -0 ranks as +0
     return b ^ ((uint32_t) ((int32_t) b >> 31) | 0x80000000u);
 }
-template <int MODE>
-__global__ void __launch_bounds__(256) k_topk_rank(int E, int k, const float* vals, int ld, const float* score, float scale, int32_t* ind,
-                                                   float* wt) {
+// row t of the launch, by a workgroup of NTHR threads (every thread reaches the end: callers may go on with a barrier)
+// COH: the selection is stored past the L2 of this workgroup's XCD (agent-scope atomic stores), for a reader in the same launch
+template <int MODE, int NTHR, bool COH = false>
+__device__ __forceinline__ void topk_row(int t, int E, int k, const float* vals, int ld, const float* score, float scale, int32_t* ind, float* wt) {
     __shared__ __attribute__((aligned(16))) unsigned long long key[TK_MAXE];   // 0 = no value: below every real key
     __shared__ unsigned long long skey[TK_MAXE / 2];                           // survivors of level 1 (at most 32 of every 64)
     __shared__ float pv[TK_MAXK], pw[TK_MAXK];
     __shared__ int pi[TK_MAXK];
     __shared__ int nsurv;
-    const int t = (int) blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const float* row = vals + (size_t) t * ld;
     const int E64 = (E + 63) & ~63;
-    for (int e = tid; e < E64; e += 256)
+    for (int e = tid; e < E64; e += NTHR)
         key[e] = e < E ? (unsigned long long) float_order(row[e]) << 32 | (uint32_t) (MODE == 0 ? e : ~e) : 0ull;
     if (tid == 0) nsurv = 0;
     __syncthreads();
-    for (int g = wv; g < E64 / 64; g += 4) {
+    for (int g = wv; g < E64 / 64; g += NTHR / 64) {
         const unsigned long long mine = key[64 * g + lane];
         int larger = 0;
 #pragma unroll 8
@@ -122,7 +123,7 @@ __global__ void __launch_bounds__(256) k_topk_rank(int E, int k, const float* va
     }
     __syncthreads();
     const int S = nsurv;
-    for (int j = tid; j < S; j += 256) {
+    for (int j = tid; j < S; j += NTHR) {
         const unsigned long long mine = skey[j];
         int rank = 0;
         for (int o = 0; o < S; ++o) rank += skey[o] > mine ? 1 : 0;
@@ -138,9 +139,15 @@ __global__ void __launch_bounds__(256) k_topk_rank(int E, int k, const float* va
     if (lane < k) {   // a wave's LDS accesses stay in order: every lane's pw is written before any lane sums
         float sum = 0.0f;
         for (int r = 0; r < k; ++r) sum += pw[r];
-        ind[(size_t) t * k + lane] = pi[lane];
+        if (COH) __hip_atomic_store(ind + (size_t) t * k + lane, pi[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else ind[(size_t) t * k + lane] = pi[lane];
         wt[(size_t) t * k + lane] = MODE == 0 ? pw[lane] / sum : pw[lane] / sum * scale;
     }
+}
+template <int MODE>
+__global__ void __launch_bounds__(256) k_topk_rank(int E, int k, const float* vals, int ld, const float* score, float scale, int32_t* ind,
+                                                   float* wt) {
+    topk_row<MODE, 256>((int) blockIdx.x, E, k, vals, ld, score, scale, ind, wt);
 }
 
 // ---- elementwise --------------------------------------------------------------------------------------------------------
@@ -205,7 +212,10 @@ __device__ __forceinline__ unsigned long long equal_lanes(int e, int nbits) {
     }
     return m;
 }
-__global__ void __launch_bounds__(64 * BK_WAVES) k_bucket(const int32_t* inds, int count, int n, int32_t* work, int32_t* perm, MmTile* tiles) {
+// COH: the selections were stored by other workgroups of this launch (agent-scope atomic loads)
+template <bool COH = false>
+__device__ __forceinline__ void bucket_all(const int32_t* inds, int count, int n, int32_t* work, int32_t* perm, MmTile* tiles) {
+    auto sel_at = [&](int i) { return COH ? __hip_atomic_load(inds + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : inds[i]; };
     extern __shared__ uint32_t hist[];   // [BK_WAVES][n]
     __shared__ int wsum[2][BK_WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -217,7 +227,7 @@ __global__ void __launch_bounds__(64 * BK_WAVES) k_bucket(const int32_t* inds, i
     for (int i = tid; i < BK_WAVES * n; i += 64 * BK_WAVES) hist[i] = 0;
     __syncthreads();
     for (int i = i0; i < i1; i += 64) {
-        int e = i + lane < i1 ? inds[i + lane] : -1;
+        int e = i + lane < i1 ? sel_at(i + lane) : -1;
         const bool live = (unsigned) e < (unsigned) n;   // an index outside the table is left out
         if (!live) e = 1 << (nbits - 1);
         const unsigned long long eq = equal_lanes(e, nbits);
@@ -261,7 +271,7 @@ __global__ void __launch_bounds__(64 * BK_WAVES) k_bucket(const int32_t* inds, i
     }
     __syncthreads();
     for (int i = i0; i < i1; i += 64) {
-        int e = i + lane < i1 ? inds[i + lane] : -1;
+        int e = i + lane < i1 ? sel_at(i + lane) : -1;
         const bool live = (unsigned) e < (unsigned) n;
         if (!live) e = 1 << (nbits - 1);
         const unsigned long long eq = equal_lanes(e, nbits), before = eq & ((1ull << lane) - 1ull);
@@ -271,6 +281,27 @@ __global__ void __launch_bounds__(64 * BK_WAVES) k_bucket(const int32_t* inds, i
             if (before == 0) mine[e] = at + (uint32_t) __popcll(eq);
         }
     }
+}
+__global__ void __launch_bounds__(64 * BK_WAVES) k_bucket(const int32_t* inds, int count, int n, int32_t* work, int32_t* perm, MmTile* tiles) {
+    bucket_all<false>(inds, count, n, work, perm, tiles);
+}
+// The batched softmax step's routing and grouping in one launch: workgroup t ranks row t (k_topk_rank<0>'s arithmetic), and the
+// workgroup that finishes last - a ticket in the word behind the bucket's work area, back at zero when the launch ends -
+// groups the launch's pairs (k_bucket's).  Nobody waits for anybody.
+__global__ void __launch_bounds__(64 * BK_WAVES) k_route_bucket(int E, int k, const float* logits, int ld, int32_t* ind, float* wt, int T, int32_t* work,
+                                                                int32_t* perm, MmTile* tiles) {
+    __shared__ int last;
+    topk_row<0, 64 * BK_WAVES, true>((int) blockIdx.x, E, k, logits, ld, (const float*) 0, 1.0f, ind, wt);
+    if (threadIdx.x == 0) {   // wave 0 stored the row's selection: those stores have left the wave before the ticket is taken
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        last = atomicAdd((unsigned*) &work[2 * E + 3], 1u) == (unsigned) (T - 1);
+    }
+    __syncthreads();
+    if (!last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (threadIdx.x == 0) __hip_atomic_store((unsigned*) &work[2 * E + 3], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bucket_all<true>(ind, T * k, E, work, perm, tiles);
 }
 
 // ---- expert slot table --------------------------------------------------------------------------------------------------
@@ -516,6 +547,18 @@ void kc_bucket(kc_stream_t s, const int32_t* inds, int count, int n, int32_t* pe
                                                        (int) (sizeof(uint32_t) * BK_WAVES * BUCKET_MAX_EXPERTS));
     (void) once;
     hipLaunchKernelGGL(k_bucket, dim3(1), dim3(64 * BK_WAVES), lds, (hipStream_t) s, inds, count, n, ntiles, perm, tiles);
+    host_note_launch();
+}
+void kq4_route_bucket(kc_stream_t s, const Qwen4Cfg* c, const float* logits, int32_t* ind, float* wt, int T, int32_t* perm, MmTile* tiles,
+                      int32_t* ntiles) {
+    if (T < 1) return;
+    if (c->n_exp < c->top_k || c->n_exp > TK_MAXE || c->top_k < 1 || c->top_k > TK_MAXK || c->n_exp > BUCKET_MAX_EXPERTS) { host_note_unsupported(); return; }
+    const size_t lds = sizeof(uint32_t) * BK_WAVES * (size_t) c->n_exp;
+    static const hipError_t once = hipFuncSetAttribute((const void*) k_route_bucket, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                       (int) (sizeof(uint32_t) * BK_WAVES * BUCKET_MAX_EXPERTS));
+    (void) once;
+    hipLaunchKernelGGL(k_route_bucket, dim3((unsigned) T), dim3(64 * BK_WAVES), lds, (hipStream_t) s, c->n_exp, c->top_k, logits, c->n_exp, ind, wt, T,
+                       ntiles, perm, tiles);
     host_note_launch();
 }
 void kc_cache_admit(kc_stream_t s, const CachePool* p, int sl, const int32_t* inds, int count, int flags) {

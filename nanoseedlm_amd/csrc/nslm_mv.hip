@@ -43,6 +43,7 @@ struct MvArgs {
     int ttot;             // dense modes with NT > 1: tokens of the launch; workgroup row blockIdx.y takes tokens NT y .. (nt = NT)
                           // (last, so that the one-token kernels read their arguments where they always did: a field
                           // added in the middle cost them a second round of argument loads, 0.3 us a launch)
+    uint16_t* px;         // k_mv_wide, dense: non-null = the staged rows also leave as BF16 bits [token][K] (the batched GEMMs' view)
 };
 #define MV_MAXJ 4
 #define MV_YBUF 1024   // virtual rows a workgroup takes at most (rpi <= 256 of them an iteration)
@@ -416,8 +417,10 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
         wA = a.ws[sl];
         if (MODE == GATEUP) wB = a.wu[sl];
     }
-    const float* xrow = a.x + (size_t) (DNW ? 0 : pair / a.xdiv) * a.xs;
-    const int nbk = a.K / 8, nt = DNW ? a.nt : 1;
+    // dense launches of more than MV_MAXT tokens (ttot > 0): the tokens are dealt to grid.y in runs of MV_MAXT
+    const int tg0 = (MODE == DENSE && a.ttot > 0) ? (int) blockIdx.y * MV_MAXT : 0;
+    const float* xrow = a.x + (size_t) (DNW ? tg0 : pair / a.xdiv) * a.xs;
+    const int nbk = a.K / 8, nt = !DNW ? 1 : (MODE == DENSE && a.ttot > 0) ? min(MV_MAXT, a.ttot - tg0) : a.nt;
     bool alA = ((uintptr_t) wA.p[0] & 15u) == 0;
     const bool alB = ((uintptr_t) wB.p[0] & 15u) == 0;
     int total = a.R;
@@ -425,9 +428,30 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
         total = 0;
         for (int j = 0; j < a.nj; ++j) total += a.Rj[j];
     }
-    for (int t = 0; t < nt; ++t)
-        for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[(size_t) t * (a.K / 4) + i] = ((const float4*) (xrow + (size_t) t * a.xs))[i];
+    // staging: a piece of every row is requested before the first is stored (a loop over the rows with a load and a store each
+    // is one memory round trip a row: 8 us of a 14 us launch at 8 rows of 2048)
+    for (int i = tid; i < a.K / 4; i += 256) {
+        float4 q[MV_MAXT];
+#pragma unroll
+        for (int t = 0; t < MV_MAXT; ++t) {
+            if (t >= nt) break;   // (uniform: no wait is needed between the rows' requests)
+            q[t] = ((const float4*) (xrow + (size_t) t * a.xs))[i];
+        }
+#pragma unroll
+        for (int t = 0; t < MV_MAXT; ++t) {
+            if (t >= nt) break;
+            if (MODE == DENSE && a.px) { q[t].x = bfr(q[t].x); q[t].y = bfr(q[t].y); q[t].z = bfr(q[t].z); q[t].w = bfr(q[t].w); }   // the rows as the GEMMs see them
+            ((float4*) xw)[(size_t) t * (a.K / 4) + i] = q[t];
+        }
+    }
     __syncthreads();
+    if (MODE == DENSE && a.px && blockIdx.x == 0) {   // one workgroup of each token run writes the run's BF16 view
+        for (int i = tid; i < nt * nbk; i += 256) {
+            const int t = i / nbk, j = i - t * nbk;
+            const float4 q0 = ((const float4*) xw)[(size_t) t * (a.K / 4) + 2 * j], q1 = ((const float4*) xw)[(size_t) t * (a.K / 4) + 2 * j + 1];
+            ((uint4*) (a.px + (size_t) (tg0 + t) * a.K))[j] = make_uint4(pack_bf2(q0.x, q0.y), pack_bf2(q0.z, q0.w), pack_bf2(q1.x, q1.y), pack_bf2(q1.z, q1.w));
+        }
+    }
     for (int rr = (int) blockIdx.x * 4 + wv; rr < total; rr += (int) gridDim.x * 4) {
         int r = rr, job = 0;
         if (MODE == MULTI) {   // the matrix this row belongs to (the rows of the matrices follow each other)
@@ -476,7 +500,7 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
                 if (lane == 0) a.y[(size_t) pair * a.ys + r] = a.f32out ? (s / (1.0f + expf(-s))) * u : bfr(silu_bf(bfr(s)) * bfr(u));
             } else if (lane == 0) {
                 if (MODE == MULTI) store_y(a.yj[job] + (size_t) t * a.ysj[job] + r, s, a.addj[job], a.f32out);
-                else store_y(a.y + (size_t) (MODE == DENSE ? t : pair) * a.ys + r, s, a.add, a.f32out);
+                else store_y(a.y + (size_t) (MODE == DENSE ? tg0 + t : pair) * a.ys + r, s, a.add, a.f32out);
             }
         }
     }
@@ -668,7 +692,15 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         return;
     }
     // Every other shape: the kernels' token loops hold MV_MAXT tokens, so more rows go in runs of MV_MAXT (a token's result does
-    // not depend on the run it is in).
+    // not depend on the run it is in): for the wave-a-row kernel the runs of one launch, dealt to grid.y.
+    if (T > MV_MAXT && wide_ok(fmt, K, x, xs, MV_MAXT)) {
+        MvArgs b = a;
+        b.nt = MV_MAXT;   // (sizes the staging)
+        b.ttot = T;
+        launch_wide<DENSE>(st, fmt, b, (T + MV_MAXT - 1) / MV_MAXT);
+        note_launch();
+        return;
+    }
     for (int t0 = 0; t0 < T; t0 += MV_MAXT) {
         MvArgs b = a;
         b.x = x + (size_t) t0 * xs;
@@ -678,6 +710,18 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         else hipLaunchKernelGGL(k_mv_any<DENSE>, dim3((unsigned) (R + 3) / 4, 1), dim3(256), 0, st, fmt, b);
     }
     note_launch();
+}
+
+int kc_mv_pack(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int xs, float* y, int ys, int T, uint16_t* px) {
+    if (T < 1 || T > MV_MULTI_MAXT || R < 1 || !wide_ok(fmt, K, x, xs, T < MV_MAXT ? T : MV_MAXT) || !aligned16(px)) return -1;
+    MvArgs a = {};
+    a.wd = w; a.x = x; a.y = y; a.K = K; a.R = R; a.xdiv = 1; a.xs = xs; a.ys = ys; a.f32out = g_store_f32;
+    a.nt = T < MV_MAXT ? T : MV_MAXT;
+    a.ttot = T;
+    a.px = px;
+    launch_wide<DENSE>((hipStream_t) s, fmt, a, (T + MV_MAXT - 1) / MV_MAXT);
+    note_launch();
+    return 0;
 }
 
 int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, float* const* y, const int* ys, const int* add, int K,

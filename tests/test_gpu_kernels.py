@@ -573,3 +573,89 @@ def test_mv_many_tokens_equal_single_token_calls(fmt, K, R, T):
         bad = np.argwhere(a.view(np.uint32) != b.view(np.uint32))
         assert not np.array_equal(a, y0) and len(bad) == 0, (add, len(bad), bad[:6].tolist())
         ya.free(); yb.free()
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_BF16, packs.MF_Q8, packs.MF_Q4])
+@pytest.mark.parametrize("T", [9, 19, 32, 64])
+def test_mv_wide_many_rows_in_one_launch(fmt, T):
+    """kc_mv of a BF16 / Q8 / Q4 matrix over more than 8 rows (one launch, the runs of 8 dealt to grid.y) gives every row the
+    bits of a call of up to 8 rows; kc_mv_pack gives kc_mv's bits for the rows rounded to BF16 (what the GEMM it stands in for
+    multiplies) and leaves kc_pack_input_bf16's view of the rows."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(91 + T + fmt)
+    K, R = 1024, 140
+    w = backend.WSlice()
+    if fmt == packs.MF_BF16:
+        bufs = [moe.DevBuf.from_array(packs.f32_to_bf16_bits((rng.standard_normal((R, K)) * 0.05).astype(np.float32)))]
+        w.p[0] = bufs[0].ptr.value
+    else:
+        pk = packs.affine(rng, 1, R, K, bits=4 if fmt == packs.MF_Q4 else 8, group=64)
+        bufs = [moe.DevBuf.from_array(pk[k][0]) for k in ("words", "scales", "biases")]
+        w.p[0], w.p[1], w.p[2], w.gs = bufs[0].ptr.value, bufs[1].ptr.value, bufs[2].ptr.value, 6
+    x = rng.standard_normal((T, K)).astype(np.float32)      # not BF16 values: the packed view must round
+    dx = moe.DevBuf.from_array(x)
+    ya, yb, yc = moe.DevBuf(4 * T * R), moe.DevBuf(4 * T * R), moe.DevBuf(4 * T * R)
+    px, py = moe.DevBuf(2 * T * K), moe.DevBuf(2 * T * K)
+    L.kc_mv(None, fmt, w, K, R, dx.ptr, K, ya.ptr, R, T, 0, None)
+    for t0 in range(0, T, 8):
+        L.kc_mv(None, fmt, w, K, R, dx.at(4 * t0 * K), K, yb.at(4 * t0 * R), R, min(8, T - t0), 0, None)
+    assert L.kc_mv_pack(None, fmt, w, K, R, dx.ptr, K, yc.ptr, R, T, px.ptr) == 0
+    L.kc_pack_input_bf16(None, dx.ptr, py.ptr, C.c_size_t(T * K))
+    dxr, yd = moe.DevBuf.from_array(packs.round_bf16(x)), moe.DevBuf(4 * T * R)
+    L.kc_mv(None, fmt, w, K, R, dxr.ptr, K, yd.ptr, R, T, 0, None)
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    a, b, c, dd = (v.to_array(np.float32, (T, R)) for v in (ya, yb, yc, yd))
+    assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32)) and np.array_equal(c.view(np.uint32), dd.view(np.uint32))
+    assert not np.array_equal(c, a)
+    dxr.free(); yd.free()
+    assert np.array_equal(px.to_array(np.uint16, (T, K)), py.to_array(np.uint16, (T, K)))
+    assert L.kc_mv_pack(None, fmt, w, K, R, dx.ptr, K, yc.ptr, R, 65, px.ptr) == -1      # more rows than one launch takes
+    for v in bufs + [dx, ya, yb, yc, px, py]:
+        v.free()
+
+
+@pytest.mark.parametrize("E,k,T", [(128, 8, 32), (64, 4, 16), (512, 10, 64), (16, 4, 9), (1000, 6, 27)])
+def test_route_bucket_equals_route_then_bucket(E, k, T):
+    """kq4_route_bucket: the batched step's routing and grouping in one launch - kq4_route's selection and weights,
+    kc_bucket's permutation, tiles and offsets, bit for bit; launch after launch on the same work area (the ticket word
+    behind it goes back to zero), logits with exact ties."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(17 * E + T)
+    cfg = backend.Qwen4Cfg()
+    cfg.n_exp, cfg.top_k = E, k
+    P, mt = T * k, T * k // 128 + E + 1
+    ia, ib, wa, wb = moe.DevBuf(4 * P), moe.DevBuf(4 * P), moe.DevBuf(4 * P), moe.DevBuf(4 * P)
+    pa, pb = moe.DevBuf(4 * P), moe.DevBuf(4 * P)
+    ta, tb = moe.DevBuf(16 * mt), moe.DevBuf(16 * mt)
+    na, nb = moe.DevBuf(4 * (2 * E + 4)), moe.DevBuf(4 * (2 * E + 4))
+    for b in (na, nb, ta, tb):
+        L.nh_memset(b.ptr, 0, C.c_size_t(b.nbytes))
+    for rep in range(4):
+        lg = packs.round_bf16(rng.standard_normal((T, E)).astype(np.float32))
+        if rep == 1:
+            lg = np.round(lg * 2) / 2                                   # many exact ties
+        if rep == 2:
+            lg[:, : E // 2] = lg[:, :1]                                 # half the experts tied with the first
+        dl = moe.DevBuf.from_array(lg.astype(np.float32))
+        L.kq4_route(None, C.byref(cfg), dl.ptr, ia.ptr, wa.ptr, T)
+        L.kc_bucket(None, ia.ptr, P, E, pa.ptr, ta.ptr, na.ptr)
+        L.kq4_route_bucket(None, C.byref(cfg), dl.ptr, ib.ptr, wb.ptr, T, pb.ptr, tb.ptr, nb.ptr)
+        moe.device_sync()
+        assert L.kc_last_error() == 0
+        assert np.array_equal(ia.to_array(np.int32, (T, k)), ib.to_array(np.int32, (T, k))), rep
+        assert np.array_equal(wa.to_array(np.uint32, (T, k)), wb.to_array(np.uint32, (T, k))), rep
+        assert np.array_equal(pa.to_array(np.int32, (P,)), pb.to_array(np.int32, (P,))), rep
+        wka, wkb = na.to_array(np.int32, (2 * E + 4,)), nb.to_array(np.int32, (2 * E + 4,))
+        assert np.array_equal(wka[:2 * E + 3], wkb[:2 * E + 3]) and wkb[2 * E + 3] == 0, rep
+        n = int(wka[0])
+        assert n > 0 and np.array_equal(ta.to_array(np.int32, (mt, 4))[:n], tb.to_array(np.int32, (mt, 4))[:n]), rep
+        dl.free()
+    for b in (ia, ib, wa, wb, pa, pb, ta, tb, na, nb):
+        b.free()
