@@ -428,20 +428,21 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
         total = 0;
         for (int j = 0; j < a.nj; ++j) total += a.Rj[j];
     }
-    // staging: a piece of every row is requested before the first is stored (a loop over the rows with a load and a store each
-    // is one memory round trip a row: 8 us of a 14 us launch at 8 rows of 2048)
-    for (int i = tid; i < a.K / 4; i += 256) {
-        float4 q[MV_MAXT];
+    // staging: with several rows a piece of every row is requested before the first is stored (a loop over the rows with a load
+    // and a store each is one memory round trip a row: 8 us of a 14 us launch at 8 rows of 2048)
+    if (nt == 1 && !(MODE == DENSE && a.px)) {
+        for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[i] = ((const float4*) xrow)[i];
+    } else {
+        for (int i = tid; i < a.K / 4; i += 256) {
+            float4 q[MV_MAXT];
 #pragma unroll
-        for (int t = 0; t < MV_MAXT; ++t) {
-            if (t >= nt) break;   // (uniform: no wait is needed between the rows' requests)
-            q[t] = ((const float4*) (xrow + (size_t) t * a.xs))[i];
-        }
+            for (int t = 0; t < MV_MAXT; ++t) q[t] = ((const float4*) (xrow + (size_t) min(t, nt - 1) * a.xs))[i];   // clamped: unconditional loads
 #pragma unroll
-        for (int t = 0; t < MV_MAXT; ++t) {
-            if (t >= nt) break;
-            if (MODE == DENSE && a.px) { q[t].x = bfr(q[t].x); q[t].y = bfr(q[t].y); q[t].z = bfr(q[t].z); q[t].w = bfr(q[t].w); }   // the rows as the GEMMs see them
-            ((float4*) xw)[(size_t) t * (a.K / 4) + i] = q[t];
+            for (int t = 0; t < MV_MAXT; ++t) {
+                if (t >= nt) break;
+                if (MODE == DENSE && a.px) { q[t].x = bfr(q[t].x); q[t].y = bfr(q[t].y); q[t].z = bfr(q[t].z); q[t].w = bfr(q[t].w); }   // the rows as the GEMMs see them
+                ((float4*) xw)[(size_t) t * (a.K / 4) + i] = q[t];
+            }
         }
     }
     __syncthreads();
