@@ -1007,8 +1007,10 @@ int pick_by_cu_load(int units, int iters, int cus, int nmax) {
 template <int P>
 int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // One token is at most a few hundred items more than three workgroups a CU hold (C2: 784): that launch may use the
-    // registers of four waves a SIMD instead of five (107 instead of 96, no spills: 35.0 -> 34.5 us).
-    const bool few = a.T == 1;
+    // registers of four waves a SIMD instead of five (107 instead of 96, no spills: 35.0 -> 34.5 us).  With the P = 4 column form the
+    // same holds up to four tokens (C2, four / five waves, us: 2 tokens 41.4 / 45.8, 3: 55.6 / 56.3, 4: 66.4 / 69.8, 5: 85.9 / 80.3,
+    // 8: 115.1 / 110.8; P = 3, C3: 2 tokens 166.5 / 157.7, 4: 272.6 / 263.7).
+    const bool few = a.T == 1 || (P == 4 && a.T <= 4);
     void (*kern)(FusedArgs) = few ? (sg ? (sd ? k_moe_decode<P, true, true, 4> : k_moe_decode<P, true, false, 4>)
                                         : (sd ? k_moe_decode<P, false, true, 4> : k_moe_decode<P, false, false, 4>))
                                   : (sg ? (sd ? k_moe_decode<P, true, true, 5> : k_moe_decode<P, true, false, 5>)
