@@ -205,6 +205,7 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
     MV_STAMP(1);
 
     const int eA = wA.eb, eB = wB.eb;
+    const bool single = SHFL && MODE != GATEUP && v1 - v0 <= rpi;   // (uniform over the workgroup)
     int par = 0;
     for (int vb = v0; vb < v1; vb += rpi, par ^= 1) {
         v = vb + lr;
@@ -230,7 +231,9 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
                         ybuf[t][(v - v0) >> 1] = a.f32out ? (gs / (1.0f + expf(-gs))) * us : bfr(silu_bf(bfr(gs)) * bfr(us));
                     }
                 } else if (active && ch == 0 && v < v1) {
-                    ybuf[t][v - v0] = s * NSLM_R32;
+                    // a workgroup with one iteration has no later wait that a store could hold up: its sums leave at once
+                    if (single) store_y(yb + (size_t) (DN ? t : pair) * ys + v, s * NSLM_R32, add, a.f32out);
+                    else ybuf[t][v - v0] = s * NSLM_R32;
                 }
             }
         } else {
@@ -259,6 +262,7 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         cur = nxt;
         MV_STAMP(2 + min((vb - v0) / rpi, 4));
     }
+    if (single) return;
     __syncthreads();
     const int nout = MODE == GATEUP ? (v1 - v0) >> 1 : v1 - v0, o0 = MODE == GATEUP ? v0 >> 1 : v0;
     for (int w = tid; w < nout * (NT > 1 ? nt_ : 1); w += NTHR) {
