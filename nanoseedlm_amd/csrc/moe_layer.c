@@ -351,8 +351,9 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         kc_router(s, ra, m->rw + (size_t) layer * E * d, m->rb + (size_t) layer * E, xn, m->logit, m->score, m->ind, m->wt, T);
     }
     if (!m->resident) {   /* with every expert resident the table never changes: nothing to admit, nothing to copy */
-        if (m->pred_pending == layer) {   /* the predicted experts' copies land before the table is consulted */
-            nh_stream_wait_event((nh_stream_t) s, m->ev_pred[layer]);
+        if (m->pred_pending >= 0) {   /* the predicted experts' copies land before the table is consulted - or changed: a caller
+                                         that does not go on with the predicted layer must not meet copies in flight either */
+            nh_stream_wait_event((nh_stream_t) s, m->ev_pred[m->pred_pending]);
             m->pred_pending = -1;
         }
         kc_cache_admit(s, &m->pool, layer, m->ind, P, 0);
