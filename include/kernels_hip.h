@@ -172,6 +172,13 @@ void kc_heads_deq(kc_stream_t s, int fmt, WSlice W, const uint32_t* G, int H, in
 /* Rows [0,R) of one slice of any format decoded to BF16 bits [R][K] (seeds with the slice's own eb; SEED4 too):
  * the bit-exact weight regeneration check. */
 void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out);
+/* kc_mm_grouped_packed for a caller that knows an upper bound of MmTile.count: a decode step of T rows chooses no expert
+ * more than T times, so no tile holds more than tile_rows = T pairs.  Up to 32 the launch uses workgroups with one
+ * multiplying wave (four a CU instead of two; the tiles are decode-bound).  The bound is a promise: pairs of a tile beyond
+ * it are not computed.  tile_rows < 1 or > 32: as kc_mm_grouped_packed. */
+void kc_mm_grouped_packed_rows(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
+                               int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
+                               int tile_rows);
 /* 1: the matvec family stores unrounded f32 instead of BF16-rounded values (for comparison with CPU references that do
  * not round, nslm/lib_cpu_seed4.c).  Process-global like kc_seed_gemm_f32; default 0 = the reference's store. */
 void kc_store_f32(int on);

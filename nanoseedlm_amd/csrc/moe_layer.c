@@ -381,11 +381,12 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         if (!routed_and_grouped) kc_bucket(s, m->ind, P, E, m->perm, m->tiles, m->ntiles);
         if (packed) {
             if (c->router != NSLM_ROUTE_SOFTMAX) kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);   /* else: made for the router */
-            kc_mm_grouped_packed(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
-            kc_mm_grouped_packed(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
+            /* a step of T rows chooses no expert more than T times: no tile holds more than T pairs */
+            kc_mm_grouped_packed_rows(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T);
+            kc_mm_grouped_packed_rows(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T);
             kc_swiglu_pack(s, m->G, m->U, (uint16_t*) m->A, (size_t) P * ff);
-            kc_mm_grouped_packed(s, c->fmt, down, ff, d, (const uint16_t*) m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
-                                 m->max_tiles, NULL);
+            kc_mm_grouped_packed_rows(s, c->fmt, down, ff, d, (const uint16_t*) m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
+                                      m->max_tiles, T);
         } else {
             kc_mm_grouped_dev(s, c->fmt, gate, d, ff, xn, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);
             kc_mm_grouped_dev(s, c->fmt, up, d, ff, xn, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, NULL);

@@ -438,7 +438,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         const MmTile tl = tiles[blockIdx.y];
         wt = ws[tl.slice];
         start = tl.start;
-        count = tl.count;
+        count = min(tl.count, BN);   // (a tile never holds more than the launch was told: see mm_grouped)
     } else {
         wt = wd;
         start = (int) blockIdx.y * BN;
@@ -553,18 +553,28 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
 #pragma unroll
         for (int u = 0; u < RECD; ++u) load_rec(u, rec[u]);
         lookup(rec[0], look[0]);
-        for (int s0 = 0; s0 < nsteps; s0 += RECD) {
-#pragma unroll
-            for (int u = 0; u < RECD; ++u) {
-                if (s0 + u >= nsteps) break;
-                lookup(rec[(u + 1) % RECD], look[(u + 1) & 1]);   // the next step's table reads travel under this step's decode
-                produce(s0 + u, rec[u], look[u & 1]);
-                load_rec(s0 + u + RECD, rec[u]);
-                MM_STAMP(256, s0 + u, 8);
-                lds_barrier();
-                MM_STAMP(256, s0 + u, 9);
-            }
+        auto one = [&](int s, auto uc) {
+            constexpr int u = decltype(uc)::value;
+            lookup(rec[(u + 1) % RECD], look[(u + 1) & 1]);   // the next step's table reads travel under this step's decode
+            produce(s, rec[u], look[u & 1]);
+            load_rec(s + RECD, rec[u]);
+            MM_STAMP(256, s, 8);
+            lds_barrier();
+            MM_STAMP(256, s, 9);
+        };
+        // whole rounds of the record ring in a loop with one way out (a conditional exit per step costs the loop a
+        // register move per record word and step), the steps left over after it
+        int s0 = 0;
+        for (; s0 + RECD <= nsteps; s0 += RECD) {
+            one(s0, std::integral_constant<int, 0>{});
+            one(s0 + 1, std::integral_constant<int, 1>{});
+            one(s0 + 2, std::integral_constant<int, 2>{});
+            one(s0 + 3, std::integral_constant<int, 3>{});
         }
+        static_assert(RECD == 4, "the unrolling above");
+        if (s0 < nsteps) one(s0, std::integral_constant<int, 0>{});
+        if (s0 + 1 < nsteps) one(s0 + 1, std::integral_constant<int, 1>{});
+        if (s0 + 2 < nsteps) one(s0 + 2, std::integral_constant<int, 2>{});
         return;
     }
 
@@ -714,13 +724,16 @@ void mm_dense(hipStream_t st, int fmt, WSlice w, int K, int R, const void* x, in
 }
 template <bool PACKED>
 void mm_grouped(hipStream_t st, int fmt, const WSlice* ws, int K, int R, const void* x, int xs, float* y, int ys, int xdiv,
-                const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int grid_tiles) {
+                const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int grid_tiles, int tile_rows) {
     if (grid_tiles < 1 || R < 1) return;
     MmArgs a = {K, R, 0, xs, ys, xdiv, 0, host_store_f32()};
     WSlice none = {};
     if (PACKED && stream_ok(fmt, K, xs, x, 0)) {
-        // grouped tiles are mostly a few pairs of one expert: decode-bound, so a short ring buys two workgroups a CU
-        launch_mm_stream<1, 4, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
+        // grouped tiles are mostly a few pairs of one expert: decode-bound, so a short ring buys two workgroups a CU - and
+        // where the caller knows that no tile holds more than 32 pairs, one multiplying wave instead of four buys four
+        const dim3 grid((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles);
+        if (tile_rows <= 32) launch_mm_stream<1, 1, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
+        else launch_mm_stream<1, 4, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
         return;
     }
     launch_mm<1, PACKED>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
@@ -745,19 +758,24 @@ void kc_mm_packed(kc_stream_t s, int fmt, WSlice w, int K, int R, const uint16_t
 void kc_mm_grouped(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
                    int xdiv, const int32_t* perm, const MmTile* tiles, int ntiles, const uint32_t* G) {
     (void) G;
-    mm_grouped<false>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nullptr, ntiles);
+    mm_grouped<false>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nullptr, ntiles, MMT_BN);
 }
 void kc_mm_grouped_dev(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const float* x, int xs, float* y, int ys,
                        int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int max_tiles,
                        const uint32_t* G) {
     (void) G;
-    mm_grouped<false>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, ntiles, max_tiles);
+    mm_grouped<false>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, ntiles, max_tiles, MMT_BN);
 }
 void kc_mm_grouped_packed(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
                           int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
                           const uint32_t* G) {
     (void) G;
-    mm_grouped<true>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nt, max_tiles);
+    mm_grouped<true>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nt, max_tiles, MMT_BN);
+}
+void kc_mm_grouped_packed_rows(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
+                               int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
+                               int tile_rows) {
+    mm_grouped<true>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nt, max_tiles, tile_rows < 1 ? MMT_BN : tile_rows);
 }
 
 }   // extern "C"

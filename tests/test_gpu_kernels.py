@@ -659,3 +659,52 @@ def test_route_bucket_equals_route_then_bucket(E, k, T):
         dl.free()
     for b in (ia, ib, wa, wb, pa, pb, ta, tb, na, nb):
         b.free()
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("T", [3, 20, 32])
+def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
+    """kc_mm_grouped_packed_rows with the caller's bound on the pairs of a tile (a decode step of T rows: no expert more than
+    T times) against kc_mm_grouped_packed on the same tiles, bit for bit - the narrow workgroup shape changes no sum.  R 72:
+    not a multiple of a tile; top-4 of 9 experts, so most experts hold several pairs."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(100 * fmt + T)
+    E, k, R, K = 9, 4, 72, 256
+    p = make_pack(rng, fmt, E, R, K)
+    seeds = moe.DevBuf.from_array(p["seeds"])
+    words = moe.DevBuf.from_array(p["coefs"] if fmt == packs.MF_SEED4P4 else p["nibs"])
+    codes = moe.DevBuf.from_array(p["codes"]) if fmt == packs.MF_SEED4P4 else None
+    arr = (backend.WSlice * E)()
+    for e in range(E):
+        arr[e].p[0] = seeds.ptr.value + e * R * K // 4
+        arr[e].p[1] = words.ptr.value + e * R * K // 4
+        if codes is not None:
+            arr[e].p[3] = codes.ptr.value + e * R * K // 16
+        arr[e].eb = int(p["eb"][e])
+    tab = moe.DevBuf(C.sizeof(arr))
+    backend.check(L.nh_memcpy_h2d(tab.ptr, arr, C.c_size_t(C.sizeof(arr))), "nh_memcpy_h2d")
+    P = T * k
+    ind = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)   # distinct experts a row
+    di = moe.DevBuf.from_array(ind)
+    mt = P // 128 + E + 1
+    perm, tiles, work = moe.DevBuf(4 * P), moe.DevBuf(16 * mt), moe.DevBuf(4 * (2 * E + 4))
+    L.nh_memset(work.ptr, 0, C.c_size_t(work.nbytes))
+    L.nh_memset(tiles.ptr, 0, C.c_size_t(tiles.nbytes))
+    x = moe.DevBuf.from_array(packs.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32)))
+    ya, yb = moe.DevBuf(4 * P * R), moe.DevBuf(4 * P * R)
+    L.nh_memset(ya.ptr, 0xFF, C.c_size_t(ya.nbytes))
+    L.nh_memset(yb.ptr, 0xFF, C.c_size_t(yb.nbytes))
+    moe.device_sync()
+    L.kc_bucket(None, di.ptr, P, E, perm.ptr, tiles.ptr, work.ptr)
+    L.kc_mm_grouped_packed(None, fmt, tab.ptr, K, R, x.ptr, K, ya.ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, None)
+    L.kc_mm_grouped_packed_rows(None, fmt, tab.ptr, K, R, x.ptr, K, yb.ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T)
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    a, b = ya.to_array(np.uint32, (P, R)), yb.to_array(np.uint32, (P, R))
+    assert not (a == 0xFFFFFFFF).any()
+    assert np.array_equal(a, b)
+    for buf in (seeds, words, tab, di, perm, tiles, work, x, ya, yb) + ((codes,) if codes is not None else ()):
+        buf.free()
