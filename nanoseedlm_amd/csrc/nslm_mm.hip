@@ -456,22 +456,19 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     const int nsteps = a.K / WK;
 
     if (producer) {
-        const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = r0 + rr, nbk = a.K / 8;
-        const bool live = row < a.R;
-        const bool al4 = (((uintptr_t) wt.p[0] | (uintptr_t) wt.p[1]) & 3u) == 0;
-        // this thread's two blocks of step s
-        auto load_rec = [&](int s, MmRec2& r) {
-            if (s >= nsteps || !live) return;
+        // rows past R decode row R - 1 again (never stored)
+        const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = min(r0 + rr, a.R - 1), nbk = a.K / 8;
+        // This thread's two blocks of step s.  Always the same loads - steps past the end request the last step again, and a
+        // stream at any 2-byte boundary is read by the same instruction (the load is typed with that alignment) - so that the
+        // compiler knows how many loads are in flight at every use: with the loads inside conditions it had waited, after
+        // every third and fourth step, for the records it had requested a moment before.
+        typedef uint32_t u32_a2 __attribute__((aligned(2)));
+        auto load_rec = [&](int s_, MmRec2& r) {
+            const int s = min(s_, nsteps - 1);
             if (seedf) {
                 const size_t g = (size_t) row * nbk + (size_t) s * (WK / 8) + 2 * jb;   // even: the pair shares a dword and a codes byte
-                const NSLM_GLOBAL uint16_t *sp = gp<uint16_t>(wt.p[0]) + g, *cp = gp<uint16_t>(wt.p[1]) + g;
-                if (al4) {
-                    r.u = *(const NSLM_GLOBAL uint32_t*) sp;
-                    r.v = *(const NSLM_GLOBAL uint32_t*) cp;
-                } else {
-                    r.u = sp[0] | (uint32_t) sp[1] << 16;
-                    r.v = cp[0] | (uint32_t) cp[1] << 16;
-                }
+                r.u = *(const NSLM_GLOBAL u32_a2*) (gp<uint16_t>(wt.p[0]) + g);
+                r.v = *(const NSLM_GLOBAL u32_a2*) (gp<uint16_t>(wt.p[1]) + g);
                 if (FMT == MF_SEED4P4) r.c = gp<uint8_t>(wt.p[3])[g >> 1];
                 return;
             }
@@ -500,7 +497,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
             }
         };
         auto produce = [&](int s, const MmRec2& r, const Look& k) {
-            float f[2][8];   // rows past R decode their zeroed records: harmless, their outputs are never stored
+            float f[2][8];
             {
                 if (seedf) {
                     const uint32_t up[2] = {r.u << 16, r.u}, word[2] = {r.v & 0xFFFFu, r.v >> 16};
