@@ -37,46 +37,6 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #define BK 32           // K per step
 #define LDW 40          // LDS row stride in BF16 elements (80 bytes: 16-byte fragment reads are conflict-free)
 
-// the 8 weights of block j of row r as f32 (seeds exact and unrounded; BF16 / Q8 / Q4 as their BF16 values)
-__device__ __forceinline__ void tile_block(int fmt, const WSlice& w, const uint32_t* tab, int r, int K, int j, float (&o)[8]) {
-    const int nbk = K / 8;
-    if (fmt == MF_SEED4P4 || fmt == MF_SEED4) {
-        const size_t g = (size_t) r * nbk + j;
-        const uint32_t seed = gp<uint16_t>(w.p[0])[g], word = gp<uint16_t>(w.p[1])[g];
-        int is[8], code;
-        if (fmt == MF_SEED4P4) {
-            block_isum<4>(tab, seed, word, is);
-            code = (gp<uint8_t>(w.p[3])[g >> 1] >> ((g & 1) * 4)) & 15;
-        } else {
-            block_isum<3>(tab, seed, word, is);
-            code = (int) (word & 15u);
-        }
-        const float sc = pow2f(w.eb + code) * NSLM_R32;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) o[c] = (float) is[c] * sc;
-    } else if (fmt == MF_BF16) {
-        const uint4 v = ldg16(gp<uint16_t>(w.p[0]) + (size_t) r * K + (size_t) j * 8);
-        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(u[i] << 16); o[2 * i + 1] = __uint_as_float(u[i] & 0xFFFF0000u); }
-    } else {
-        const size_t e0 = (size_t) r * K + (size_t) j * 8, gi = e0 >> group_shift(w);
-        const float s = bf(gp<uint16_t>(w.p[1])[gi]), b = bf(gp<uint16_t>(w.p[2])[gi]);
-        if (fmt == MF_Q8) {
-            const uint2 q = ldg8(gp<uint32_t>(w.p[0]) + e0 / 4);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                o[i] = bfr(s * (float) ((q.x >> (8 * i)) & 255u) + b);
-                o[4 + i] = bfr(s * (float) ((q.y >> (8 * i)) & 255u) + b);
-            }
-        } else {
-            const uint32_t q = gp<uint32_t>(w.p[0])[e0 / 8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) o[i] = bfr(s * (float) ((q >> (4 * i)) & 15u) + b);
-        }
-    }
-}
-
 // MT: 32-token tiles per consumer wave (the workgroup covers 128 * MT tokens or pairs).  NTERM: BF16 terms per weight.
 //
 // 512 threads: waves 0-3 are consumers (MFMA only: wave w owns tokens [32 MT w, 32 MT (w+1)) x all 64 rows), waves 4-7
