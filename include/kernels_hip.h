@@ -285,6 +285,10 @@ int kc_moe_decode_error_word(void);
 /* polls a wait between workgroups makes before it gives up (0: the default, 2^21 - seconds).  A host that shares the GPU
  * between streams may want a shorter bound; tests set a tiny one to drive the error path while every kernel still exits. */
 void kc_moe_decode_spin_limit(unsigned polls);
+/* Which of the library's two persistent kernels a step of up to MV_MAXT tokens takes (the same bits either way): 0 (default) the
+ * one with a workgroup per CU where the shape fits it (hidden width 64 * 2^n <= 2048, T * pairs * ff <= 65536), else the one
+ * with a workgroup per (pair, row tile); 1 always the latter; 2 as 0.  Process-global, for comparisons. */
+void kc_moe_decode_kernel(int which);
 int kc_moe_decode(kc_stream_t s, int fmt, const uint16_t* router_w, const WSlice* gate, const WSlice* up, const WSlice* down,
                   int n_exp, int top_k, int d, int ff, const float* x, int xs, int T, float* out, int os, float* logits,
                   int32_t* ind, float* wt, float* A, float* D, uint32_t* sync);

@@ -410,6 +410,11 @@ int nslm_moe_fused_error(NslmMoe* m) {
     return (int) w;
 }
 
+int nslm_moe_fused_words(NslmMoe* m, int first, int n, uint32_t* out) {
+    if (first < 0 || n < 0 || (size_t) first + (size_t) n > kc_moe_decode_sync_words(kc_moe_decode_max_rows(), m->c.d)) return -1;
+    return nh_device_sync() || nh_memcpy_d2h(out, m->sync + first, 4 * (size_t) n) ? -1 : 0;
+}
+
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {
     if (nh_device_sync()) return -1;
     return (nh_memcpy_d2h(ind, m->ind, 4 * (size_t) T * m->c.top_k) | nh_memcpy_d2h(wt, m->wt, 4 * (size_t) T * m->c.top_k)) ? -1 : 0;

@@ -67,6 +67,10 @@ int nslm_moe_fused_mode(const NslmMoe* m);
 int nslm_moe_fallbacks(const NslmMoe* m);
 /* 0, or non-zero when a grid barrier of the fused kernel gave up since open (synchronises) */
 int nslm_moe_fused_error(NslmMoe* m);
+/* n words of the persistent kernels' sync area from word `first`, copied to the host (synchronises): behind the error word
+ * (kc_moe_decode_error_word()) lie which wait gave up (word + 1) and workgroup 0's phase timeline (64-bit wall-clock ticks, 100 MHz,
+ * from word + 2) */
+int nslm_moe_fused_words(NslmMoe* m, int first, int n, uint32_t* out);
 /* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
 /* the last step's intermediates per (token, expert) pair, copied to the host (synchronises): A [pairs][ff] = the SwiGLU outputs

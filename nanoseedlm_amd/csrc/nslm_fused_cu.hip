@@ -1,0 +1,580 @@
+// nslm_fused_cu.hip - the routed-expert decode step of up to MV_MAXT tokens as one persistent kernel with ONE workgroup per CU
+// (k_moe_decode_cu).  Same arithmetic, instruction for instruction, as the kernel of nslm_fused.hip (and so as the five
+// separate launches, engine/qwen4_cuda.c:1023-1083): what differs is who computes what, and how the results travel.
+//
+//   - A workgroup is 12 or 16 waves and owns its CU.  What every workgroup of the other kernel does for itself - polling and
+//     ranking the logits, caching the chosen experts' slices, staging the input in the form the matvec reads - happens once a
+//     CU, and the waves of a CU go through the phases together: no wave is left alone on its SIMD in a phase's tail.
+//   - Gate + up: a token's (pair, row) tasks are dealt evenly, a contiguous run to each CU; inside the CU a wave takes the next
+//     task when it is ready for one (the row's chunks over the wave's lanes, row sums by xor-shuffles), no workgroup barrier
+//     inside the pass.
+//   - The SwiGLU outputs A are the only data that crosses CUs.  A CU's waves count their tasks off in LDS as their stores of a
+//     token's values are acknowledged; the wave that completes the count arrives for the CU on a two-level counter (groups of
+//     CUs, then the groups), and the last arrival of all raises the token's ready words, one per group of CUs, which one lane
+//     per CU polls.  Then every CU reads the token's A once, as BF16.  (Values that carried the generation themselves, polled
+//     in place by every thread that needs them, were a round trip shorter on paper; in practice 256 CUs polling 48 KB starved
+//     the very stores they were waiting for, and so did 256 CUs polling one word per CU.)
+//   - Down: CU c owns output rows [c rpc, (c + 1) rpc) of EVERY pair of the token, so the weighted sum of the experts is a
+//     sum inside the workgroup - no second exchange and no waiting for another CU behind the down rows.
+//   - Several tokens: gate + up of all tokens first, then the down passes; a token's A has been on its way for a whole pass
+//     when its down pass needs it, so only a one-token launch waits for the exchange.
+//   - Every instruction outside the row loops counts (a CU's waves all execute it at the same moment): what can be computed
+//     on the host arrives in the arguments, and no index is formed by an integer division.
+// Shapes: hidden width d = 64 * 2^n <= 2048 (a row's chunks fit a wave and the row sums are shuffles), T * pairs * ff <=
+// FUSED_XA_MAX, the workgroup's LDS <= 160 KB.  Other shapes stay with the kernel of nslm_fused.hip.
+#include "nslm_fused_dev.h"
+
+using namespace nslm;
+
+namespace {
+
+#define CU_LDS_MAX (160 * 1024)
+#define CU_LDS_MIN (82 * 1024)   // more than half a CU's LDS: two of these workgroups never share a CU
+#define CU_LG 4                  // router logits a CU forms
+#define CU_PRE_MAXE 256          // experts whose slice tables are copied to LDS while the logits are on their way
+
+// x / d for x < 2^32 / d', d' = the power of two >= d: one multiply (m = ceil(2^32 / d); d = 1: m = 0 stands for x itself)
+struct FastDiv {
+    uint32_t m;
+};
+inline FastDiv fastdiv_of(uint32_t d) { return FastDiv{d <= 1 ? 0u : (uint32_t) ((0x100000000ull + d - 1) / d)}; }
+__device__ __forceinline__ uint32_t operator/(uint32_t x, FastDiv f) { return f.m ? __umulhi(x, f.m) : x; }
+
+// What the host works out once per launch (offsets into the workgroup's dynamic LDS in 4-byte words, each a multiple of 4)
+struct CuParams {
+    int xg;      // [T][Lg * xpad] the tokens' inputs in the form the gate + up matvec reads
+    int xd;      // [kk][Ld * xpad] one token's A, all pairs, in the form the down matvec reads
+    int scr;     // [NTHR] down pass: the threads' partial sums (rows that do not fit a shuffle)
+    int pk;      // [T][KP] ranking: the logits' keys
+    int rv;      // [T][E4] the logits
+    int dsum;    // [kk][rpc] the down rows of the token in hand, rounded to BF16
+    int ri;      // [T][32] expert by rank
+    int rw;      // [T][36] weight by rank (+ the shared expert's 1)
+    int rn;      // [MV_MAXT + 16] the rows' RMSNorm scales, the waves' partial sums of a norm
+    int cnt;     // [2][MV_MAXT] per token: this CU's gate + up tasks handed out / finished
+    int av;      // [T][n_c * vpt] this CU's SwiGLU outputs until the token's last task is done
+    int lgs;     // [16] the logits this CU forms, until one wave stores them
+    int sel;     // [3 + T * kk * 3] WSlice: the shared expert's slices; with more than CU_PRE_MAXE experts the pairs' slices
+    int pre;     // [3][E] WSlice: the layer's slice tables (E <= CU_PRE_MAXE)
+    int total;
+    int G;                // CUs = workgroups
+    int lgL;              // log2 of the chunks in a gate / up row (Lg)
+    int rpw, tpp, Wt;     // gate + up: virtual rows a wave-task, tasks a pair, tasks a token
+    int n_c, ncu_act;     // tasks a CU and token; CUs that have tasks
+    int rpc;              // down: output rows a CU owns
+    int rpi, rows_t, nit; // down: (pair, row)s an iteration of the workgroup, (pair, row)s a token and CU, iterations a token
+    int nbp;              // blocks of 8 in a row of A
+    int vpt, lgV;         // SwiGLU outputs a task (rpw / 2) and its log2
+    int E4, KP;           // E padded to 4; keys a token (E padded to 16)
+    FastDiv by_tpp, by_rpc, by_Ld, by_nbp, by_kk, by_E;
+};
+
+#ifdef NSLM_CU_STAMPS
+__device__ unsigned long long g_cstamp[4096 + 256 * 16 * 8];
+#endif
+template <int P, bool SHFL_D, int NTHR>
+__global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c) {
+    constexpr int NW = NTHR / 64, XP = xpad<P>();
+    extern __shared__ __attribute__((aligned(16))) float dyn[];
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int G = c.G, T = a.T, E = a.E, kk = a.kk, Lg = a.Lg, Ld = a.Ld, E4 = c.E4, rpc = c.rpc;
+    float* const xg = dyn + c.xg;
+    float* const xd = dyn + c.xd;
+    uint32_t* const scr = (uint32_t*) (dyn + c.scr);
+    float* const rv = dyn + c.rv;
+    float* const dsum = dyn + c.dsum;
+    int* const ri_s = (int*) (dyn + c.ri);
+    float* const rw_s = dyn + c.rw;
+    float* const rn_s = dyn + c.rn;
+    uint32_t* const cnt_s = (uint32_t*) (dyn + c.cnt);
+    WSlice* const sel = (WSlice*) (dyn + c.sel);
+    uint4* const pre = (uint4*) (dyn + c.pre);
+    uint32_t* const pk = (uint32_t*) (dyn + c.pk);
+    float* const avs = dyn + c.av;
+    float* const lgs = dyn + c.lgs;
+    const bool preload = E <= CU_PRE_MAXE;
+    // phase timeline of workgroup 0 (wall clock ticks) beside the error word
+    unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
+#ifdef NSLM_CU_STAMPS   // development builds: every workgroup's timeline
+#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); g_cstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } } while (0)
+#define WSTAMP(i) do { if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + (i)] = wall_clock64(); } while (0)
+#define DSTAMP(i) do { if (tid == 0) g_cstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
+#else
+#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
+#define WSTAMP(i) do { } while (0)
+#define DSTAMP(i) do { } while (0)
+#endif
+    STAMP(0);
+
+    // ---- what does not depend on the routing: generation, tables, slice tables, norm scales, the staged input, the logits ----
+    const uint32_t gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
+    const TableWords<NTHR> tw = tables_fetch<NTHR>();
+    // the layer's three slice tables, 16 bytes a thread and round, three rounds (unconditional: with more experts than the LDS
+    // copy takes, pieces that are not kept)
+    static_assert(3 * CU_PRE_MAXE * sizeof(WSlice) / 16 <= 3 * NTHR, "three rounds cover the slice tables");
+    const int per = E * (int) (sizeof(WSlice) / 16), npre = 3 * per;   // 16-byte pieces of a table, of the three
+    auto pre_piece = [&](int u) {
+        const int i = min(tid + u * NTHR, npre - 1), which = (i >= per ? 1 : 0) + (i >= 2 * per ? 1 : 0);
+        const WSlice* tb = which == 0 ? a.gate : which == 1 ? a.up : a.down;
+        return *((const uint4*) tb + (i - which * per));
+    };
+    const uint4 pw0 = pre_piece(0), pw1 = pre_piece(1), pw2 = pre_piece(2);
+    loads_issued();
+    if (a.nw) {   // the rows' scales, as the norm kernel sums them: 256 threads, thread i takes x[i], x[i + 256], ..
+        for (int t = 0; t < T; ++t) {
+            float ss = 0.0f;
+            if (tid < 256) {
+                const float* xi = a.x + (size_t) t * a.xs;
+#pragma unroll
+                for (int j = 0; j < NSLM_NORM_NR; ++j) {
+                    const int k = tid + j * 256;
+                    const float xv = xi[min(k, a.d - 1)];
+                    const float v = k < a.d ? xv : 0.0f;
+                    ss = fmaf(v, v, ss);
+                }
+                for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+                if (lane == 0) rn_s[MV_MAXT + wv] = ss;
+            }
+            __syncthreads();
+            if (tid == 0) rn_s[t] = rsqrtf(((rn_s[MV_MAXT] + rn_s[MV_MAXT + 1]) + (rn_s[MV_MAXT + 2] + rn_s[MV_MAXT + 3])) / (float) a.d + a.neps);
+            __syncthreads();
+        }
+    }
+    const uint32_t tag = gen + 1u;
+    unsigned long long* lg64 = (unsigned long long*) (a.sync + FUSED_CULG_WORDS);   // [FUSED_CULG_LINES][16]: a line a CU's logits
+    uint16_t* const xa16 = (uint16_t*) (a.sync + FUSED_XA_WORDS);   // [token][pair][ff]: the SwiGLU outputs as BF16 bits
+    if (tid < 2 * MV_MAXT) cnt_s[tid] = 0u;
+    // Router logits: CU c forms items [CU_LG c, CU_LG c + CU_LG) of the [token][expert] table, a wave an item (the last waves:
+    // the first ones stage the input meanwhile), and gathers them in LDS; one wave then stores them into the CU's own 128-byte
+    // line (item i at word 16 (i / CU_LG) + i % CU_LG), which is written once, by one instruction.  (A line that 16 CUs each
+    // wrote a word of, while every CU polled it, took 1.7 us from the last store to the first CU that saw all of it; a line
+    // written once is seen 0.4 us later.  Few items a CU: a CU's vector-memory path takes 1.5 us to load twelve router rows.)
+    const int lg0 = CU_LG * (int) blockIdx.x, lgn = max(0, min(CU_LG, T * E - lg0));
+    if (wv >= NW - lgn) {
+        const int u = NW - 1 - wv, item = lg0 + u, t = (int) ((uint32_t) item / c.by_E), e = item - t * E;
+        const float lv = router_logit(a.rw + (size_t) e * a.d, a.x + (size_t) t * a.xs, a.d, a.nw, a.nw ? rn_s[t] : 1.0f);
+        if (lane == 0) lgs[u] = lv;
+        WSTAMP(4);
+    }
+    tables_store<NTHR>(tab, tw);
+    if (preload) {
+        if (tid < npre) pre[tid] = pw0;
+        if (tid + NTHR < npre) pre[tid + NTHR] = pw1;
+        if (tid + 2 * NTHR < npre) pre[tid + 2 * NTHR] = pw2;
+    }
+    {   // the tokens' inputs, normalised on the way when nw is given (the values kq4_norm1p would have stored)
+        const int nb = a.d >> 3;
+        for (int t = 0; t < T; ++t)
+            for (int b = tid; b < nb; b += NTHR) {
+                const float* src = a.x + (size_t) t * a.xs + (size_t) b * 8;
+                const float4 q0 = *(const float4*) src, q1 = *(const float4*) (src + 4);
+                float v[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                if (a.nw) {
+                    const float4 w0 = *(const float4*) (a.nw + (size_t) b * 8), w1 = *(const float4*) (a.nw + (size_t) b * 8 + 4);
+                    const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+                    const float rn = rn_s[t];
+#pragma unroll
+                    for (int cc = 0; cc < 8; ++cc) v[cc] = v[cc] * rn * (1.0f + w[cc]);
+                }
+                store_block<P>(xg + t * (Lg * XP), b, v);
+            }
+    }
+    if (a.ns && tid < 3) {   // the shared expert's slices (field by field: a struct copy of a kernel argument goes through scratch memory)
+#define PUT_SH(i) do { WSlice* q = &sel[i]; q->p[0] = a.sh[i].p[0]; q->p[1] = a.sh[i].p[1]; q->p[2] = a.sh[i].p[2]; q->p[3] = a.sh[i].p[3]; q->eb = a.sh[i].eb; q->gs = a.sh[i].gs; } while (0)
+        if (tid == 0) PUT_SH(0);
+        if (tid == 1) PUT_SH(1);
+        if (tid == 2) PUT_SH(2);
+#undef PUT_SH
+    }
+    STAMP(1);
+    __syncthreads();   // every wave has used its copy of the generation; tables, slice tables, inputs and this CU's logits are in LDS
+    if (tid < lgn) {
+        const float lv = lgs[tid];
+        st_agent(lg64 + 16 * (int) blockIdx.x + tid, (unsigned long long) __float_as_uint(lv) | (unsigned long long) tag << 32);
+        a.logits[lg0 + tid] = lv;
+    }
+    uint32_t arrived = 0;
+    if (tid == 0) arrived = arrive_issue(a.sync, gen);
+
+    // Every wait of this kernel is a bounded poll; a thread that has once given up (error word set, results void) waits for
+    // nothing any more, so the grid drains quickly.
+    uint32_t polls_left = a.spin;
+    // ---- the logits of every token, polled until they carry this launch's generation (bounded) -----------------------------
+    // rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order.  The
+    // logits are BF16 values, so (order-preserving upper half of the float | index) is a unique 32-bit key and rank = number of
+    // larger keys; the thread that has polled a logit leaves its key.
+    for (int t = 0; t < T; ++t)
+        for (int e = tid; e < c.KP; e += NTHR) {
+            float v = __uint_as_float(0xFF800000u);
+            uint32_t key = 0u;   // absent: below every real key
+            if (e < E) {
+                const int item = t * E + e;
+                const unsigned long long* lw = lg64 + 16 * (item / CU_LG) + item % CU_LG;
+                unsigned long long w = ld_agent(lw);
+                for (; (uint32_t) (w >> 32) != tag; w = ld_agent(lw)) {
+                    __builtin_amdgcn_s_sleep(2);
+                    if (polls_left == 0 || --polls_left == 0) {
+                        atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                        a.sync[FUSED_ERR_WORD + 1] = 0x10000000u | (uint32_t) (t * E + e);
+                        break;
+                    }
+                }
+                v = __uint_as_float((uint32_t) w);
+                const uint32_t b = __float_as_uint(v + 0.0f);   // -0 counts as +0, as in a float compare
+                key = ((b ^ ((uint32_t) ((int32_t) b >> 31) | 0x80000000u)) & 0xFFFF0000u) | (uint32_t) e;
+            }
+            if (e < E4) rv[t * E4 + e] = v;
+            pk[t * c.KP + e] = key;
+        }
+    __syncthreads();
+    STAMP(2);
+    // four lanes an expert, each counts over a quarter of the token's keys (read four at a time as LDS broadcasts); the quarters
+    // meet by two shuffles, so a rank needs no second pass through LDS
+    {
+        const int part = lane & 3, q4 = c.KP >> 2;
+        for (int t = 0; t < T; ++t)
+            for (int e0 = 16 * wv; e0 < E; e0 += NTHR / 4) {   // (a wave 16 experts: uniform over the wave, whose shuffles these are)
+                const int e = e0 + (lane >> 2);
+                const uint32_t* kt = pk + t * c.KP;
+                const uint32_t ke = kt[min(e, c.KP - 1)];
+                int g = 0;
+#pragma unroll 2
+                for (int o = part * q4; o < (part + 1) * q4; o += 4) {
+                    const uint4 q = *(const uint4*) &kt[o];
+                    g += (q.x > ke ? 1 : 0) + (q.y > ke ? 1 : 0) + (q.z > ke ? 1 : 0) + (q.w > ke ? 1 : 0);
+                }
+                g += __shfl_xor(g, 1);
+                g += __shfl_xor(g, 2);
+                if (part == 0 && e < E && g < a.k) ri_s[t * 32 + g] = e;
+            }
+    }
+    __syncthreads();
+    DSTAMP(8);
+    // the routing weights (softmax over the k chosen logits): wave t for token t (the combine reads them, barriers later)
+    if (wv < T) {
+        const int t = wv;
+        float* rw = rw_s + t * 36;
+        const int* ri = ri_s + t * 32;
+        if (lane < a.k) rw[lane] = expf(rv[t * E4 + ri[lane]] - rv[t * E4 + ri[0]]);
+        if (lane < a.k) {
+            float top = 0.0f;
+            for (int r = 0; r < a.k; ++r) top += rw[r];
+            rw[lane] = rw[lane] / top;   // every lane has read all k values before any lane writes
+        }
+        if (a.ns && lane == a.k) rw[a.k] = 1.0f;
+        if ((int) blockIdx.x == t % G && lane < a.k) {   // one writer per token publishes the routing
+            a.ind[(size_t) t * a.k + lane] = ri[lane];
+            a.wt[(size_t) t * a.k + lane] = rw[lane];
+        }
+    }
+    if (!preload) {   // more experts than the LDS copy of the slice tables takes: the pairs' slices from memory
+        for (int p = tid; p < T * kk; p += NTHR) {
+            const int t = (int) ((uint32_t) p / c.by_kk), j = p - t * kk;
+            if (j < a.k) {
+                const int e = ri_s[t * 32 + j];
+                sel[3 + p * 3] = a.gate[e];
+                sel[3 + p * 3 + 1] = a.up[e];
+                sel[3 + p * 3 + 2] = a.down[e];
+            }
+        }
+        __syncthreads();
+    }
+    // slice `which` (0 gate, 1 up, 2 down) of pair (t, j), in LDS
+    auto slice = [&](int t, int j, int which) -> const WSlice& {
+        if (j >= a.k) return sel[which];
+        if (preload) return ((const WSlice*) pre)[which * E + ri_s[t * 32 + j]];
+        return sel[3 + (t * kk + j) * 3 + which];
+    };
+    STAMP(3);
+
+    // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
+    const int q_lo = (int) blockIdx.x * c.n_c, n_loc = max(0, min(c.n_c, c.Wt - q_lo));   // this CU's tasks a token
+    const int lr = lane >> c.lgL, ch = lane & (Lg - 1);
+    {
+        // The CU's tasks of a token go to whichever wave asks next: a wave whose records arrive late, or that shares its SIMD
+        // with more waves, takes fewer.  A wave asks for its next task before it computes the current one, so that task's
+        // records travel meanwhile.  Task = (token, index in the CU's run); token T = none left.
+        int ct = 0;   // the token this wave draws from
+        auto claim = [&](int& t, int& i) {
+            for (;;) {
+                if (ct >= T || n_loc == 0) { t = T; i = 0; return; }
+                uint32_t got = 0;
+                if (lane == 0) got = atomicAdd(&cnt_s[ct], 1u);
+                got = __builtin_amdgcn_readfirstlane(got);
+                if ((int) got < n_loc) { t = ct; i = (int) got; return; }
+                ++ct;
+            }
+        };
+        // (the loads are unconditional - past the last task, the records of pair 0's first rows once more: a load under a
+        // condition keeps the compiler from counting the loads in flight, and it then waits for the next task's records
+        // before it computes the current one)
+        auto fetch = [&](int t, int i) {
+            const bool ok = t < T;
+            const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), v = (q - j * c.tpp) * c.rpw + lr;
+            const WSlice& w = slice(ok ? t : 0, j, v & 1);
+            return load_chunk<P>(w, (uint32_t) (v >> 1) * (uint32_t) Lg + (uint32_t) ch, true, true);
+        };
+        int t, i;
+        claim(t, i);
+        Chunk cur = fetch(t, i);
+        WSTAMP(0);
+        uint32_t mine = 0;   // tasks of the token in hand this wave has finished
+        const int nav = c.n_c << c.lgV;   // SwiGLU outputs a CU and token at most
+        while (t < T) {
+            int tn, inx;
+            claim(tn, inx);
+            const Chunk nxt = fetch(tn, inx);
+            const int q = q_lo + i, j = (int) ((uint32_t) q / c.by_tpp), v = (q - j * c.tpp) * c.rpw + lr;
+            float acc[1] = {0.0f};
+            chunk_dot<P, 1, true>(cur, slice(t, j, v & 1).eb, tab, xg + t * (Lg * XP) + ch * XP, 0, 1, acc);
+            float s = acc[0];
+            for (int o = Lg >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            const float other = __shfl_xor(s, Lg);
+            // (results leave after the loop: a store here would sit in front of the wait for the next task's records)
+            if (ch == 0 && !(v & 1)) avs[t * nav + (i << c.lgV) + (lr >> 1)] = bfr(silu_bf(bfr(s * NSLM_R32)) * bfr(other * NSLM_R32));
+            ++mine;
+#ifdef NSLM_CU_STAMPS
+            if (mine == 1) WSTAMP(5);
+            if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 6] = mine;
+            if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+#endif
+            if (tn != t) {   // The wave's last task of token t: it adds its tasks to the CU's count.  The wave that completes the
+                             // count stores the CU's values of the token (as BF16 for the other CUs, as f32 for the caller), and once
+                             // they are acknowledged arrives for the CU; the last CU of all raises the token's ready words.
+                WSTAMP(1);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                uint32_t before = 0;
+                if (lane == 0) before = atomicAdd(&cnt_s[MV_MAXT + t], mine);
+                before = __builtin_amdgcn_readfirstlane(before);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                if (before + mine == (uint32_t) n_loc) {
+                    for (int u = lane; u < (n_loc << c.lgV); u += 64) {
+                        const int qq = q_lo + (u >> c.lgV), jj = (int) ((uint32_t) qq / c.by_tpp);
+                        const size_t at = (size_t) (t * kk + jj) * a.ff + (size_t) (((qq - jj * c.tpp) << c.lgV) + (u & (c.vpt - 1)));
+                        const float av = avs[t * nav + u];
+                        st_agent(xa16 + at, (uint16_t) (__float_as_uint(av) >> 16));
+                        a.A[at] = av;
+                    }
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    if (lane == 0) {
+                        uint32_t* bar = a.sync + FUSED_CU_WORDS + t * FUSED_CU_TOKEN_WORDS;   // [32 group lines][root line][32 ready lines]
+                        const uint32_t g = blockIdx.x % BAR_GROUPS, ncu = (uint32_t) c.ncu_act, ng = ncu < BAR_GROUPS ? ncu : BAR_GROUPS;
+                        const uint32_t in_group = (ncu - g + BAR_GROUPS - 1) / BAR_GROUPS;
+                        if (atomicAdd(bar + 32 * g, 1u) == in_group - 1) {
+                            st_agent(bar + 32 * g, 0u);
+                            if (atomicAdd(bar + 32 * BAR_GROUPS, 1u) == ng - 1) {
+                                st_agent(bar + 32 * BAR_GROUPS, 0u);
+#pragma unroll
+                                for (uint32_t r = 0; r < BAR_GROUPS; ++r) st_agent(bar + 32 * (BAR_GROUPS + 1 + r), tag);
+                            }
+                        }
+                    }
+                }
+                mine = 0;
+                WSTAMP(2);
+            }
+            cur = nxt;
+            t = tn;
+            i = inx;
+        }
+    }
+    // Housekeeping, off the critical path: the lines of this kernel's logits table that this launch did not write, and the
+    // other step kernels' table (every launch of theirs rewrites all of it, the rows it does not use with zero: a word that
+    // does not carry the current generation is then never older than one launch), are left at zero.
+    {
+        unsigned long long* lgo = (unsigned long long*) (a.sync + FUSED_LOGIT_WORDS);
+        const int used = (T * E + CU_LG - 1) / CU_LG;
+        for (int w = (int) blockIdx.x * NTHR + tid; w < FG_MAXT * E; w += G * NTHR) st_agent(lgo + w, 0ull);
+        for (int w = (int) blockIdx.x * NTHR + tid; w < (FUSED_CULG_LINES - used) * 16; w += G * NTHR) st_agent(lg64 + 16 * used + w, 0ull);
+    }
+    if (tid == 0) arrive_finish(a.sync, (uint32_t) G, gen, arrived);
+    STAMP(4);
+
+    // ---- down: CU c owns rows [c rpc, (c + 1) rpc) of every pair; a thread a chunk of a (pair, row); then the experts' sum --------
+    const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
+    const int dl = (int) ((uint32_t) tid / c.by_Ld), dch = tid - dl * Ld;
+    auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
+        const int g = min(it * c.rpi + dl, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
+        const WSlice& w = slice(min(t, T - 1), jj, 2);
+        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch, true, true);
+    };
+    Chunk dcur = fetch_d(0, 0);
+    float* part = (float*) scr;
+    for (int t = 0; t < T; ++t) {
+        // the token's A is complete when the last CU has raised the ready words: lane 0 polls the word of this CU's group (bounded)
+        if (tid == 0) {
+            const uint32_t* rdy = a.sync + FUSED_CU_WORDS + t * FUSED_CU_TOKEN_WORDS + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS);
+            while (ld_agent(rdy) != tag) {
+                __builtin_amdgcn_s_sleep(2);
+                if (polls_left == 0 || --polls_left == 0) {
+                    atomicExch(&a.sync[FUSED_ERR_WORD], 1u);
+                    a.sync[FUSED_ERR_WORD + 1] = 0x20000000u | (uint32_t) t;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+        if (t == 0) STAMP(5);
+        // all pairs' A of the token, 16 bytes (a block of 8 values) a thread, staged as the down matvec reads it
+        for (int b = tid; b < kk * c.nbp; b += NTHR) {
+            const int j = (int) ((uint32_t) b / c.by_nbp), bb = b - j * c.nbp;
+            const unsigned long long* src = (const unsigned long long*) (xa16 + ((size_t) t * kk + j) * a.ff + (size_t) bb * 8);
+            const unsigned long long lo = ld_agent(src), hi = ld_agent(src + 1);
+            const float v[8] = {bf((uint32_t) lo & 0xFFFFu), bf((uint32_t) (lo >> 16) & 0xFFFFu), bf((uint32_t) (lo >> 32) & 0xFFFFu), bf((uint32_t) (lo >> 48)),
+                                bf((uint32_t) hi & 0xFFFFu), bf((uint32_t) (hi >> 16) & 0xFFFFu), bf((uint32_t) (hi >> 32) & 0xFFFFu), bf((uint32_t) (hi >> 48))};
+            store_block<P>(xd + j * (Ld * XP), bb, v);
+        }
+        __syncthreads();
+        if (t == 0) STAMP(6);
+        for (int it = 0; it < c.nit; ++it) {
+            const bool last = it + 1 == c.nit;
+            const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
+            const int g = it * c.rpi + dl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
+            const bool ok = dl < c.rpi && g < c.rows_t && rr < nr;
+            float acc[1] = {0.0f};
+            if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + dch * XP, 0, 1, acc);
+            if (SHFL_D) {
+                float s = acc[0];
+                for (int o = Ld >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+                if (ok && dch == 0) {
+                    const float dv = bfr(s * NSLM_R32);
+                    dsum[g] = dv;
+                    a.D[((size_t) t * kk + j) * a.d + r0 + rr] = dv;
+                }
+            } else {
+                part[tid] = acc[0];
+                __syncthreads();
+                const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
+                if (tid < c.rpi && gs < c.rows_t && rs < nr) {
+                    float s = 0.0f;
+                    for (int cc = 0; cc < Ld; ++cc) s += part[tid * Ld + cc];
+                    const float dv = bfr(s * NSLM_R32);
+                    dsum[gs] = dv;
+                    a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
+                }
+                if (!last) __syncthreads();   // part is written again by the next iteration
+            }
+            dcur = dnxt;
+        }
+        __syncthreads();
+        // out = sum_j wt_j D_j in j order (kq4_moe_combine's FMA chain), the shared expert's pair with weight 1 last
+        if (tid < nr) {
+            const float* rw = rw_s + t * 36;
+            float acc = 0.0f;
+            for (int jj = 0; jj < kk; ++jj) acc = fmaf(rw[jj], dsum[jj * rpc + tid], acc);
+            const size_t at = (size_t) t * a.os + r0 + tid;
+            a.out[at] = a.res ? bfr(a.res[at] + bfr(acc)) : acc;
+        }
+        // (the next token's staging writes xd, which every thread has finished reading before the barrier above; dsum and part
+        // are next written behind the next token's first barrier)
+    }
+    STAMP(7);
+#undef STAMP
+#undef WSTAMP
+#undef DSTAMP
+}
+
+template <int P, bool SD, int NTHR>
+int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds) {
+    void (*kern)(FusedArgs, CuParams) = k_moe_decode_cu<P, SD, NTHR>;
+    static size_t lds_set = 0;   // the largest dynamic-LDS request this kernel has been prepared for
+    static int resident = 0;
+    if (lds > lds_set) {
+        if (hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return -1;
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, NTHR, lds) != hipSuccess || per_cu < 1) return -1;
+        resident = per_cu;
+        lds_set = lds;
+    }
+    if (resident < 1) return -1;
+    hipLaunchKernelGGL(kern, dim3((unsigned) c.G), dim3(NTHR), lds, st, a, c);
+    host_note_launch();
+    return 0;
+}
+
+int log2_of(int v) {
+    int l = 0;
+    while ((1 << l) < v) ++l;
+    return l;
+}
+
+}   // namespace
+
+namespace nslm {
+
+// 0 launched; -1 the shape is not this kernel's (nothing launched)
+int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
+    if (a.T < 1 || a.T > MV_MAXT) return -1;
+    if (a.Lg > 32 || (a.Lg & (a.Lg - 1))) return -1;                       // a row's chunks: a power of two inside a wave
+    if ((long) a.T * a.kk * a.ff > FUSED_XA_MAX || a.ff % 64 || a.kk > 33) return -1;
+    const int G = fused_cu_count();
+    if (G < 1 || a.E > 1024 || (long) a.T * a.E > (long) CU_LG * (G < FUSED_CULG_LINES ? G : FUSED_CULG_LINES)) return -1;   // (a CU forms CU_LG logits)
+    a.grid = G;
+    CuParams c = {};
+    c.G = G;
+    c.lgL = log2_of(a.Lg);
+    c.rpw = 64 / a.Lg;
+    c.tpp = 2 * a.ff / c.rpw;
+    c.Wt = a.kk * c.tpp;
+    c.n_c = (c.Wt + G - 1) / G;
+    c.ncu_act = (c.Wt + c.n_c - 1) / c.n_c;
+    c.rpc = (a.d + G - 1) / G;
+    c.rows_t = a.kk * c.rpc;
+    c.nbp = a.ff / 8;
+    c.E4 = (a.E + 3) & ~3;
+    // 12 or 16 waves: the workgroup whose rounds (tasks a wave in gate + up, iterations in down) cost the CU's SIMDs the least
+    long best_cost = -1;
+    int nthr = 0;
+    for (int cand = 768; cand <= 1024; cand += 256) {
+        const int nw = cand / 64, rounds_g = (c.n_c + nw - 1) / nw, rpi = cand / a.Ld, rounds_d = (c.rows_t + rpi - 1) / rpi;
+        const long cost = (long) (2 * rounds_g + rounds_d) * nw;
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; nthr = cand; }
+    }
+    c.rpi = nthr / a.Ld;
+    c.nit = (c.rows_t + c.rpi - 1) / c.rpi;
+    c.KP = (a.E + 15) & ~15;
+    c.vpt = c.rpw / 2;
+    c.lgV = log2_of(c.vpt);
+    c.by_E = fastdiv_of((uint32_t) a.E);
+    c.by_tpp = fastdiv_of((uint32_t) c.tpp);
+    c.by_rpc = fastdiv_of((uint32_t) c.rpc);
+    c.by_Ld = fastdiv_of((uint32_t) a.Ld);
+    c.by_nbp = fastdiv_of((uint32_t) c.nbp);
+    c.by_kk = fastdiv_of((uint32_t) a.kk);
+    const int xp = P == 4 ? xpad<4>() : xpad<3>(), ws = (int) (sizeof(WSlice) / 4);
+    int o = 0;
+    auto take = [&](int words) { const int at = o; o += (words + 3) & ~3; return at; };
+    c.xg = take(a.T * a.Lg * xp);
+    c.xd = take(a.kk * a.Ld * xp);
+    c.scr = take(nthr);
+    c.pk = take(a.T * c.KP);
+    c.rv = take(a.T * c.E4);
+    c.dsum = take(a.kk * c.rpc);
+    c.ri = take(a.T * 32);
+    c.rw = take(a.T * 36);
+    c.rn = take(MV_MAXT + 16);
+    c.cnt = take(2 * MV_MAXT);
+    c.av = take(a.T * c.n_c * c.vpt);
+    c.lgs = take(16);
+    c.sel = take((3 + (a.E <= CU_PRE_MAXE ? 0 : a.T * a.kk * 3)) * ws);
+    c.pre = take(a.E <= CU_PRE_MAXE ? 3 * a.E * ws : 0);
+    c.total = o;
+    size_t lds = (size_t) c.total * 4;
+    if (lds > CU_LDS_MAX) return -1;
+    if (lds < CU_LDS_MIN) lds = CU_LDS_MIN;
+    if (P == 4) {
+        if (nthr == 768) return sd ? launch_one<4, true, 768>(st, a, c, lds) : launch_one<4, false, 768>(st, a, c, lds);
+        return sd ? launch_one<4, true, 1024>(st, a, c, lds) : launch_one<4, false, 1024>(st, a, c, lds);
+    }
+    if (nthr == 768) return sd ? launch_one<3, true, 768>(st, a, c, lds) : launch_one<3, false, 768>(st, a, c, lds);
+    return sd ? launch_one<3, true, 1024>(st, a, c, lds) : launch_one<3, false, 1024>(st, a, c, lds);
+}
+
+}   // namespace nslm
+
+#ifdef NSLM_CU_STAMPS
+extern "C" int kc_moe_decode_cu_stamps(unsigned long long* host) {
+    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_cstamp), sizeof(unsigned long long) * (4096 + 256 * 16 * 8));
+}
+#endif
