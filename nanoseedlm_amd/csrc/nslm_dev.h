@@ -214,15 +214,21 @@ __device__ __forceinline__ uint32_t coef_bytes(uint32_t cc, int odd) {
     const uint32_t t = cc & 0x0F0F0F0Fu, u = (cc >> 4) & 0x0F0F0F0Fu;   // (q0, q2 | q0', q2'), (q1, q3 | q1', q3')
     return __builtin_amdgcn_perm(u, t, odd ? 0x07030602u : 0x05010400u);
 }
-// sl: stream bits 0..31 (the seed below 16 bits of g), g: bits 16..47.  G[j] = byte j of V_0..V_3 with the nibbles made signed:
-// columns 2j (low nibbles) and 2j + 1 (high nibbles).
-__device__ __forceinline__ void col_bytes_p4(uint32_t sl, uint32_t g, uint32_t (&G)[6]) {
-    const uint32_t sh = g >> 16;
+// the sum of the four coefficients of a coefficient operand (even-column form): a dot product with ones, the constant from a scalar register
+__device__ __forceinline__ int dot8ones(uint32_t a) {
+    int d;
+    asm("v_dot8_i32_i4 %0, %1, %2, 0" : "=v"(d) : "v"(a), "s"(0x01010101u));
+    return d;
+}
+// up: any word whose upper 16 bits are the seed, g: stream bits 16..47.  G[j] = byte j of V_0..V_3 with the nibbles made signed:
+// columns 2j (low nibbles) and 2j + 1 (high nibbles).  V_p's bytes 0..3 are one funnel shift of (g : up) by 17 + p, its bytes
+// 4 and 5 one shift of g - no word of the stream's low 32 bits is formed first.
+__device__ __forceinline__ void col_bytes_p4(uint32_t up, uint32_t g, uint32_t (&G)[6]) {
     uint32_t vl[4], vh[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-        vl[p] = __builtin_amdgcn_alignbit(sh, sl, 1 + p);
-        vh[p] = sh >> (1 + p);
+        vl[p] = __builtin_amdgcn_alignbit(g, up, 17 + p);
+        vh[p] = g >> (17 + p);
     }
     const uint32_t a01 = __builtin_amdgcn_perm(vl[1], vl[0], 0x05010400u), b01 = __builtin_amdgcn_perm(vl[1], vl[0], 0x07030602u);
     const uint32_t a23 = __builtin_amdgcn_perm(vl[3], vl[2], 0x05010400u), b23 = __builtin_amdgcn_perm(vl[3], vl[2], 0x07030602u);

@@ -319,6 +319,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         claim(t, i);
         Chunk cur = fetch(t, i);
         WSTAMP(0);
+#ifdef NSLM_CU_STAMPS
+        const unsigned long long ck0 = clock64();
+#endif
         uint32_t mine = 0;   // tasks of the token in hand this wave has finished
         const int nav = c.n_c << c.lgV;   // SwiGLU outputs a CU and token at most
         while (t < T) {
@@ -343,6 +346,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                              // count stores the CU's values of the token (as BF16 for the other CUs, as f32 for the caller), and once
                              // they are acknowledged arrives for the CU; the last CU of all raises the token's ready words.
                 WSTAMP(1);
+#ifdef NSLM_CU_STAMPS
+                if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 3] = clock64() - ck0;
+#endif
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 uint32_t before = 0;
                 if (lane == 0) before = atomicAdd(&cnt_s[MV_MAXT + t], mine);
@@ -447,8 +453,16 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 __syncthreads();
                 const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
                 if (tid < c.rpi && gs < c.rows_t && rs < nr) {
+                    // the row's partial sums in chunk order; eight are read before the first is added (a chunk past the row's
+                    // last counts +0, which leaves the sum's bits alone)
                     float s = 0.0f;
-                    for (int cc = 0; cc < Ld; ++cc) s += part[tid * Ld + cc];
+                    for (int c0 = 0; c0 < Ld; c0 += 8) {
+                        float pv[8];
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) pv[cc] = part[tid * Ld + min(c0 + cc, Ld - 1)];
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
+                    }
                     const float dv = bfr(s * NSLM_R32);
                     dsum[gs] = dv;
                     a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
@@ -462,7 +476,17 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         if (tid < nr) {
             const float* rw = rw_s + t * 36;
             float acc = 0.0f;
-            for (int jj = 0; jj < kk; ++jj) acc = fmaf(rw[jj], dsum[jj * rpc + tid], acc);
+            for (int j0 = 0; j0 < kk; j0 += 8) {   // (eight experts' values read before the first is used; the chain's order is j's)
+                float wv8[8], dv8[8];
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj) {
+                    wv8[jj] = rw[min(j0 + jj, kk - 1)];
+                    dv8[jj] = dsum[min(j0 + jj, kk - 1) * rpc + tid];
+                }
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj)
+                    if (j0 + jj < kk) acc = fmaf(wv8[jj], dv8[jj], acc);
+            }
             const size_t at = (size_t) t * a.os + r0 + tid;
             a.out[at] = a.res ? bfr(a.res[at] + bfr(acc)) : acc;
         }

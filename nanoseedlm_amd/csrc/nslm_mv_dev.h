@@ -116,7 +116,7 @@ __device__ __forceinline__ void block_dot(const int (&is)[8], float e2, int b, c
 // The column form of a P = 4 block against NT tokens' 12 staged values: every column's sum is converted and used as soon as it
 // is formed (eleven sums and their float images held at once cost the persistent kernels their five waves a SIMD).
 template <int NT>
-__device__ __forceinline__ void cols_dot(uint32_t sl, uint32_t g, uint32_t be, float e2, int b, const float* xr, int xstride, float (&acc)[NT]) {
+__device__ __forceinline__ void cols_dot(uint32_t up, uint32_t g, uint32_t be, float e2, int b, const float* xr, int xstride, float (&acc)[NT]) {
     float4 xa[NT][3];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -126,13 +126,13 @@ __device__ __forceinline__ void cols_dot(uint32_t sl, uint32_t g, uint32_t be, f
         xa[t][2] = *(const float4*) (xb + 8);
     }
     uint32_t G[6];
-    col_bytes_p4(sl, g, G);
+    col_bytes_p4(up, g, G);
     const uint32_t bo = be << 4;
     float d[NT];
     auto xv = [&](int t, int m) { const float4& q = xa[t][m >> 2]; return (m & 3) == 0 ? q.x : (m & 3) == 1 ? q.y : (m & 3) == 2 ? q.z : q.w; };
 #pragma unroll
     for (int m = 0; m < 12; ++m) {
-        const float z = (float) (m == 11 ? dot8z(be, 0x01010101u) : dot8z(G[m >> 1], (m & 1) ? bo : be));
+        const float z = (float) (m == 11 ? dot8ones(be) : dot8z(G[m >> 1], (m & 1) ? bo : be));
 #pragma unroll
         for (int t = 0; t < NT; ++t) d[t] = m == 0 ? z * xv(t, 0) : fmaf(z, xv(t, m), d[t]);
     }
@@ -147,12 +147,14 @@ __device__ __forceinline__ void chunk_dot(const Chunk& ck, int eb, const uint32_
     (void) nt;
     static_assert(!PAIRED || P == 3 || COLS, "blocks in pairs: P = 3 only (the column form has one order)");
     if constexpr (COLS) {
+        const uint32_t ebase = (uint32_t) (eb + 127) << 23;   // 2^eb as f32 bits: a block's scale is this plus its code in the exponent field
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
             const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
             const uint32_t g = stream_of(tab, (b & 1) ? ss >> 16 : ss & 0xFFFFu);
-            const uint32_t sl = __builtin_amdgcn_perm(g, ss, (b & 1) ? 0x05040302u : 0x05040100u);   // seed | g << 16
-            cols_dot<NT>(sl, g, coef_bytes(cc, b & 1), pow2f(eb + (int) ((ck.codes >> (4 * b)) & 15u)), b, xr, xstride, acc);
+            const uint32_t up = (b & 1) ? ss : ss << 16;   // only the upper 16 bits are read
+            const float e2 = __uint_as_float((((ck.codes >> (4 * b)) & 15u) << 23) + ebase);
+            cols_dot<NT>(up, g, coef_bytes(cc, b & 1), e2, b, xr, xstride, acc);
         }
     } else if constexpr (PAIRED) {
 #pragma unroll
