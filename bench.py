@@ -230,7 +230,8 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         # Its launch duration is the step's event time: HIP events over the timed region on the launch stream (launches are
         # queued back to back, so there is no gap between them unless the step is wrapped in a graph).
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_moe_decode (one launch per step)",
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
+                               kernel=("k_moe_decode_cu" if T <= 3 and name[:2] == "c2" else "k_moe_decode") + " (one launch per step)",
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part, **counters_of(name))
         ind.free(); A.free()
     else:
@@ -245,7 +246,8 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
     desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",
             "c3": "C3 mixed-format layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880 Q4-g64 projections (q, k, v, o, shared gate / up / down)"}[name[:2]]
     res["config"] = {"workload": f"{desc}, batch {T}", "layers_rotated": n_layers, "inputs_rotated": NX,
-                     "launch": "stream" if no_graph else "hipGraph per step"}
+                     "launch": "stream" if no_graph else "hipGraph per step",
+                     "router_weight": "bf16 (cast of the fp32 ~N(0, 0.02) draw; the reference has no f32 weight format)"}
     res["cpu_sample"] = dict(shapes=[(ff, d), (ff, d), (d, ff)], reps=k, fmt=fmt)
     st.close()
     return res

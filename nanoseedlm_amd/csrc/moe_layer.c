@@ -419,6 +419,10 @@ int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt) {
     if (nh_device_sync()) return -1;
     return (nh_memcpy_d2h(ind, m->ind, 4 * (size_t) T * m->c.top_k) | nh_memcpy_d2h(wt, m->wt, 4 * (size_t) T * m->c.top_k)) ? -1 : 0;
 }
+int nslm_moe_last_logits(NslmMoe* m, int T, float* logits) {
+    if (T < 1 || T > m->c.max_rows || nh_device_sync()) return -1;
+    return nh_memcpy_d2h(logits, m->logit, 4 * (size_t) T * m->c.n_exp) ? -1 : 0;
+}
 int nslm_moe_last_pairs(NslmMoe* m, int pairs, float* A, float* D) {
     if (nh_device_sync()) return -1;
     return (nh_memcpy_d2h(A, m->A, 4 * (size_t) pairs * m->c.ff) | nh_memcpy_d2h(D, m->D, 4 * (size_t) pairs * m->c.d)) ? -1 : 0;

@@ -73,6 +73,9 @@ int nslm_moe_fused_error(NslmMoe* m);
 int nslm_moe_fused_words(NslmMoe* m, int first, int n, uint32_t* out);
 /* the last step's routing, copied to the host (synchronises the device): ind [T][top_k], wt [T][top_k] */
 int nslm_moe_last_routing(NslmMoe* m, int T, int32_t* ind, float* wt);
+/* the last step's router logits [T][n_exp] as the kernels formed them (softmax router: the BF16-rounded values the selection
+ * was made on), copied to the host (synchronises) */
+int nslm_moe_last_logits(NslmMoe* m, int T, float* logits);
 /* the last step's intermediates per (token, expert) pair, copied to the host (synchronises): A [pairs][ff] = the SwiGLU outputs
  * the down projections read, D [pairs][d] = the experts' outputs the combine sums.  Pair t * top_k + j of nslm_moe_step (the
  * batched path's A is the packed BF16 view: read it as uint16 [pairs][ff] in the first half of the buffer). */

@@ -22,6 +22,8 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <atomic>
+
 #include "nslm_fused_dev.h"
 
 using namespace nslm;
@@ -769,7 +771,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     }
 }
 
-uint32_t g_spin_limit = SPIN_LIMIT;
+std::atomic<uint32_t> g_spin_limit{SPIN_LIMIT};   // (any thread may set it while another launches)
 
 int g_kernel_choice = 0;   // kc_moe_decode_kernel: 0 the faster kernel for the shape, 1 a workgroup an item, 2 a workgroup a CU where it fits
 
@@ -828,11 +830,18 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
                                         : (sd ? k_moe_decode<P, false, true, 4> : k_moe_decode<P, false, false, 4>))
                                   : (sg ? (sd ? k_moe_decode<P, true, true, 5> : k_moe_decode<P, true, false, 5>)
                                         : (sd ? k_moe_decode<P, false, true, 5> : k_moe_decode<P, false, false, 5>));
-    static int cached[2][2][2] = {};   // resident workgroups per CU, by kernel variant (same LDS request every call)
+    // resident workgroups per CU, by kernel variant, for the largest LDS request seen (the request grows with max(d, ff): a launch
+    // that asks for more than the cached answer covered asks the occupancy calculator again, and raises the kernel's limit above 48 KB)
+    static int cached[2][2][2] = {};
+    static size_t cached_lds[2][2][2] = {};
     int& per_cu = cached[few][sg][sd];
-    if (!per_cu && (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds) != hipSuccess || per_cu < 1)) {
-        per_cu = 0;
-        return -1;
+    if (!per_cu || lds > cached_lds[few][sg][sd]) {
+        if (lds > 48 * 1024 && hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return -1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, lds) != hipSuccess || per_cu < 1) {
+            per_cu = 0;
+            return -1;
+        }
+        cached_lds[few][sg][sd] = lds;
     }
     // The grid must be resident at once (workgroups wait for each other's data): at most what the device holds, and no more than
     // five workgroups a CU (the most that was tried).  Items per pair (an item = a run of a pair's iterations, as
@@ -970,7 +979,9 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
-    if (g_kernel_choice != 1 && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
+    // one workgroup per CU: ahead up to three tokens (C2, us, a workgroup per CU / per item: 1 token 23.3 / 25.9, 2: 38.1 / 39.4, 3: 50.8 / 51.8,
+    // 4: 64.2 / 62.0, 8: 102.9 / 103.0)
+    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= 3)) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);

@@ -124,6 +124,13 @@ class MoeStack:
             raise RuntimeError("nslm_moe_last_routing failed")
         return ind, wt
 
+    def last_logits(self, T):
+        """The last step's router logits [T][n_exp] as the GPU formed them (what its selection was made on)."""
+        lg = np.zeros((T, self.cfg.n_exp), dtype=np.float32)
+        if self.L.nslm_moe_last_logits(self.h, T, lg.ctypes.data_as(C.c_void_p)):
+            raise RuntimeError("nslm_moe_last_logits failed")
+        return lg
+
     def last_pairs(self, pairs):
         """The last step's per-pair intermediates: A [pairs][ff] (SwiGLU outputs; uint16 BF16 bits in the batched path's packed
         layout are returned as the raw f32 buffer - see moe_layer.h) and D [pairs][d] (expert outputs)."""

@@ -96,6 +96,8 @@ def test_c2_layer_step_128_experts(oracle, T):
     oi, _ = oracle.route_softmax(lg, k)
     assert np.mean([len(set(ind[t]) & set(oi[t])) / k for t in range(T)]) >= 0.9
     assert np.allclose(wt.sum(1), 1.0, atol=1e-5)
+    from test_gpu_moe import check_routing_on_gpu_logits
+    check_routing_on_gpu_logits(oracle, st, T, k, xn, rw, ind, wt)
     # the layer output from the GPU's own routing, token 0 and the last token
     for t in sorted({0, T - 1}):
         ys = np.stack([expert_ref(oracle, gate, up, down, int(ind[t, j]), xn[t], gemm=False) for j in range(k)])
@@ -215,6 +217,8 @@ def test_c3_mixed_format_layer(be, oracle, T):
     lg = packs.round_bf16((xn.astype(np.float64) @ W.T).astype(np.float32))
     oi, _ = oracle.route_softmax(lg, k)
     assert np.mean([len(set(ind[t]) & set(oi[t])) / k for t in range(T)]) >= 0.9 and all(len(set(ind[t])) == k for t in range(T))
+    from test_gpu_moe import check_routing_on_gpu_logits
+    check_routing_on_gpu_logits(oracle, st, T, k, xn, rw, ind, wt)
     tokens = sorted({0, T - 1})
     check_stages(oracle, gate, up, down, xn, ind, wt, A, D, out, tokens, gemm=gemm)
     end_to_end(oracle, gate, up, down, xn, ind, wt, out, tokens, gemm=gemm)

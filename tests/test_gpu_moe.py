@@ -34,6 +34,19 @@ def expert_ref(orc, gate, up, down, e, x, gemm):
     return r((wd @ a).astype(np.float32)).astype(np.float64)
 
 
+def check_routing_on_gpu_logits(oracle, st, T, k, xn, rw, ind, wt):
+    """The selection must be exactly the oracle's on the logits the GPU itself formed (ties included), the weights within 1e-5,
+    and those logits within one BF16 ulp of the float64 x . W."""
+    lg = st.last_logits(T)
+    oi, ow = oracle.route_softmax(lg, k)
+    assert np.array_equal(ind, oi), (ind, oi)
+    assert np.max(np.abs(wt - ow)) <= 1e-5
+    ref = xn.astype(np.float64) @ packs.bf16_bits_to_f32(rw).astype(np.float64).T
+    mag = np.abs(xn).astype(np.float64) @ np.abs(packs.bf16_bits_to_f32(rw)).astype(np.float64).T
+    assert np.all(np.abs(lg - ref) <= np.abs(ref) / 128 + 2e-6 * mag + 1e-30)
+    assert np.array_equal(lg, packs.round_bf16(lg))          # BF16 values
+
+
 @pytest.mark.parametrize("router", [0, 1])
 @pytest.mark.parametrize("T", [1, 5, 8, 20, 27])
 @pytest.mark.parametrize("slots", [0, 20])
@@ -83,6 +96,7 @@ def test_moe_step(oracle, router, T, slots):
             if router == 0:
                 lg = r((xn.astype(np.float64) @ W.T).astype(np.float32))
                 oi, ow = oracle.route_softmax(lg, k)
+                check_routing_on_gpu_logits(oracle, st, T, k, xn, rw, ind, wt)
             else:
                 _, _, oi, ow = oracle.route_sigmoid(rw, rb, xn, k, d // 2, 2.5)
             agree = np.mean([len(set(ind[t]) & set(oi[t])) / k for t in range(T)])
