@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """bench.py - the SeedLM decode-in-matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1|c3b16|c4b1|c4b16] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2b1|c2b8|c2b32|c0|c1|c3b1|c3b16|c4b1|c4b16] [--matrices N] [--no-cpu]
 
 A step is one pass of the workload over one batch of seeded synthetic input already resident in HBM:
   c2b1 (default; the configuration the metric is quoted on): one MoE decode layer step at batch 1 - 128 experts seeded
@@ -9,7 +9,8 @@ A step is one pass of the workload over one batch of seeded synthetic input alre
         gather, down gather, combine).  Steps rotate over `layers` resident layers and 16 inputs so the selected experts
         change from step to step and the traffic comes from HBM, not from the 256 MB Infinity Cache.
   c2b8 / c2b32: the same at 8 and 32 tokens (32: grouping + grouped MFMA GEMMs).
-  c0:   dense GEMV, W 4096x4096 P=4, batch 1, rotating over 64 matrices (604 MB).
+  c0:   dense GEMV, W 4096x4096 P=4, batch 1, rotating over --matrices 64 matrices (604 MB); the line also carries the same
+        launches on one matrix, resident in the Infinity Cache (roofline.cache_resident).
   c1:   prefill GEMM, W 14336x4096 P=4, X bf16 [512 x 4096].
   c3b1 / c3b16: the mixed-format layer - 64 experts P=3 top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880
         Q4-g64 projections (q, k, v, o and the shared expert's gate / up / down) - at batch 1 and 16.
@@ -326,7 +327,7 @@ def model_workload(name, steps, warmup, no_graph, branches=False, splits=32):
     return res
 
 
-def dense_workload(name, steps, warmup):
+def dense_workload(name, steps, warmup, matrices=64):
     from nanoseedlm_amd import backend, moe, packs
     L = backend.hip()
     rng = np.random.default_rng(20261125)
@@ -334,7 +335,7 @@ def dense_workload(name, steps, warmup):
     e0, e1 = moe.Event(), moe.Event()
     if name == "c0":
         R = K = 4096
-        NM = 64
+        NM = max(1, matrices)   # 64 (604 MB: every launch reads its records from HBM); 1 = the matrix stays in the 256 MB Infinity Cache
         p = packs.seed4p4(rng, NM, R, K, eb=-22)
         ds, dc, de = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
         x = moe.DevBuf.from_array(rng.standard_normal(K).astype(np.float32))
@@ -349,7 +350,28 @@ def dense_workload(name, steps, warmup):
         def run(i):
             L.kc_mv(stream, packs.MF_SEED4P4, sl[i % NM], K, R, x.ptr, K, y.ptr, R, 1, 0, None)
         bytes_step, flops, T = R * K * 36 / 64.0, 2.0 * R * K, 1
-        desc, bound = "C0 dense seeded GEMV: W 4096x4096 P=4, batch 1, rotating over 64 matrices", "hbm"
+        desc, bound = f"C0 dense seeded GEMV: W 4096x4096 P=4, batch 1, rotating over {NM} matri{'x' if NM == 1 else 'ces'}", "hbm"
+        sample = dict(shapes=[(R, K)], reps=1, fmt=packs.MF_SEED4P4)
+    elif name == "deq":
+        # The weights' form of the decode alone, through a product entry point: kc_slice_deq regenerates the BF16 weights of a
+        # 4096 x 4096 P=4 slice (the exact integer sums on v_dot2_i32_i16, one convert and one multiply a weight), rotating over
+        # the matrices.  Reads 9.4 MB of records and writes 33.6 MB a launch.
+        R = K = 4096
+        NM = max(1, matrices)
+        p = packs.seed4p4(rng, NM, R, K, eb=-22)
+        ds, dc, de = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
+        y = moe.DevBuf(2 * R * K)
+        sl = []
+        for i in range(NM):
+            w = backend.WSlice()
+            w.p[0], w.p[1], w.p[3] = ds.ptr.value + i * R * K // 4, dc.ptr.value + i * R * K // 4, de.ptr.value + i * R * K // 16
+            w.eb = -22
+            sl.append(w)
+
+        def run(i):
+            L.kc_slice_deq(stream, packs.MF_SEED4P4, sl[i % NM], K, R, y.ptr)
+        bytes_step, flops, T = R * K * 36 / 64.0, 0.0, 1
+        desc, bound = f"weights of a 4096x4096 P=4 slice regenerated as BF16 (kc_slice_deq), rotating over {NM} matrices", "hbm"
         sample = dict(shapes=[(R, K)], reps=1, fmt=packs.MF_SEED4P4)
     else:
         R, K, T = 14336, 4096, 512
@@ -380,10 +402,26 @@ def dense_workload(name, steps, warmup):
     ms = e1.ms_since(e0) / steps
     fail_on_kernel_error()
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
+    resident = None
+    if name == "c0":
+        # The same launches on ONE matrix, which then stays in the Infinity Cache (9.4 MB of 256 MB), as the reference's kernel
+        # bench offers beside its rotating mode (harness/nslm-mova-kbench.c:8-9,149).  If this is no faster than the rotating
+        # figure, HBM is not what bounds the kernel.
+        for i in range(warmup):
+            L.kc_mv(stream, packs.MF_SEED4P4, sl[0], K, R, x.ptr, K, y.ptr, R, 1, 0, None)
+        moe.device_sync()
+        e0.record(stream)
+        for i in range(steps):
+            L.kc_mv(stream, packs.MF_SEED4P4, sl[0], K, R, x.ptr, K, y.ptr, R, 1, 0, None)
+        e1.record(stream)
+        e1.sync()
+        rms = e1.ms_since(e0) / steps
+        fail_on_kernel_error()
+        resident = dict(launch_us=rms * 1e3, achieved=bytes_step / rms / 1e6, frac=bytes_step / rms / 1e6 / HBM_PEAK_GBS, matrices=1)
     if bound == "hbm":
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_mv_seed<dense>",
-                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, **counters_of(name))
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_mv_seed<dense>" if name == "c0" else "k_deq",
+                               launch_us=ms * 1e3, algorithmic_bytes=bytes_step, cache_resident=resident, **counters_of(name))
     else:
         res["roofline"] = dict(bound="mfma", achieved=flops / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",
                                frac=flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, kernel="k_mm_stream<2, 8> (BF16 activations, 512-token tile)",
@@ -456,6 +494,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c2b1")
     ap.add_argument("--layers", type=int, default=4)
+    ap.add_argument("--matrices", type=int, default=64, help="c0: matrices the launches rotate over (64: records from HBM; 1: resident in the Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="plain stream launches even for multi-launch steps")
     ap.add_argument("--graph", action="store_true", help="one hipGraph per step even when the step is a single launch")
@@ -477,7 +516,7 @@ def main():
     elif a.workload[:2] == "c4":
         r = model_workload(a.workload, a.steps, a.warmup, a.no_graph, a.branches, a.splits)
     else:
-        r = dense_workload(a.workload, a.steps, a.warmup)
+        r = dense_workload(a.workload, a.steps, a.warmup, a.matrices)
     gbs = r["bytes_per_step"] / r["ms_per_step"] / 1e6
     line = {
         "metric": METRIC, "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

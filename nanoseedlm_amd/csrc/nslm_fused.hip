@@ -34,10 +34,10 @@ namespace {
 // whatever comes before the pass (a wait for other workgroups, the staging of the activations).
 template <int P, bool GATEUP>
 __device__ __forceinline__ Chunk first_chunk(const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1) {
-    const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L, vv = v0 + lr;
-    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
+    (void) rpi;
+    const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L, vv = min(v0 + lr, v1 - 1);   // (rows past the last: the last row's records)
     const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
-    return load_chunk<P>(w, (uint32_t) (GATEUP ? vv >> 1 : vv) * (uint32_t) L + (uint32_t) ch, lr < rpi && vv < v1, al);
+    return load_chunk<P>(w, (uint32_t) (GATEUP ? vv >> 1 : vv) * (uint32_t) L + (uint32_t) ch);
 }
 
 // rows [v0, v1) of one pair: the k_mv_seed loop with the activations in LDS (xl, chunk-padded).  emit(row, sum, other)
@@ -47,12 +47,10 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
                                           const uint32_t* tab, const float* xl, float (*part)[256], Emit emit) {
     const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
-    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
-    auto fetch = [&](int vv) {
-        const bool ok = active && vv < v1;
-        const int r = GATEUP ? vv >> 1 : vv;
-        const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
-        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
+    auto fetch = [&](int vv) {   // (rows past the last: the last row's records once more)
+        const int vc = min(vv, v1 - 1), r = GATEUP ? vc >> 1 : vc;
+        const WSlice& w = (GATEUP && (vc & 1)) ? wB : wA;
+        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch);
     };
     int par = 0;
     for (int vb = v0; vb < v1; vb += rpi, par ^= 1) {
@@ -453,12 +451,10 @@ __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const W
                                             const uint32_t* tab, const float* xl, int xstride, int nt, float* part, Emit emit) {
     const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
-    const bool al = streams_aligned(P, wA) && (!GATEUP || streams_aligned(P, wB));
-    auto fetch = [&](int vv) {
-        const bool ok = active && vv < v1;
-        const int r = GATEUP ? vv >> 1 : vv;
-        const WSlice& w = (GATEUP && (vv & 1)) ? wB : wA;
-        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
+    auto fetch = [&](int vv) {   // (rows past the last: the last row's records once more)
+        const int vc = min(vv, v1 - 1), r = GATEUP ? vc >> 1 : vc;
+        const WSlice& w = (GATEUP && (vc & 1)) ? wB : wA;
+        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch);
     };
     int par = 0;
     for (int vb = v0; vb < v1; vb += rpi, par ^= 1) {

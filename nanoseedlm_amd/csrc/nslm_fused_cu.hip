@@ -2,7 +2,7 @@
 // (k_moe_decode_cu).  Same arithmetic, instruction for instruction, as the kernel of nslm_fused.hip (and so as the five
 // separate launches, engine/qwen4_cuda.c:1023-1083): what differs is who computes what, and how the results travel.
 //
-//   - A workgroup is 12 or 16 waves and owns its CU.  What every workgroup of the other kernel does for itself - polling and
+//   - A workgroup is 16 waves and owns its CU.  What every workgroup of the other kernel does for itself - polling and
 //     ranking the logits, caching the chosen experts' slices, staging the input in the form the matvec reads - happens once a
 //     CU, and the waves of a CU go through the phases together: no wave is left alone on its SIMD in a phase's tail.
 //   - Gate + up: a token's (pair, row) tasks are dealt evenly, a contiguous run to each CU; inside the CU a wave takes the next
@@ -313,7 +313,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             const bool ok = t < T;
             const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), v = (q - j * c.tpp) * c.rpw + lr;
             const WSlice& w = slice(ok ? t : 0, j, v & 1);
-            return load_chunk<P>(w, (uint32_t) (v >> 1) * (uint32_t) Lg + (uint32_t) ch, true, true);
+            return load_chunk<P>(w, (uint32_t) (v >> 1) * (uint32_t) Lg + (uint32_t) ch);
         };
         int t, i;
         claim(t, i);
@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
         const int g = min(it * c.rpi + dl, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
         const WSlice& w = slice(min(t, T - 1), jj, 2);
-        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch, true, true);
+        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch);
     };
     Chunk dcur = fetch_d(0, 0);
     float* part = (float*) scr;
@@ -547,14 +547,9 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     c.rows_t = a.kk * c.rpc;
     c.nbp = a.ff / 8;
     c.E4 = (a.E + 3) & ~3;
-    // 12 or 16 waves: the workgroup whose rounds (tasks a wave in gate + up, iterations in down) cost the CU's SIMDs the least
-    long best_cost = -1;
-    int nthr = 0;
-    for (int cand = 768; cand <= 1024; cand += 256) {
-        const int nw = cand / 64, rounds_g = (c.n_c + nw - 1) / nw, rpi = cand / a.Ld, rounds_d = (c.rows_t + rpi - 1) / rpi;
-        const long cost = (long) (2 * rounds_g + rounds_d) * nw;
-        if (best_cost < 0 || cost < best_cost) { best_cost = cost; nthr = cand; }
-    }
+    // 16 waves: four a SIMD get through a block's dependent instruction chains faster than three (C2, one token: 22.6 against
+    // 23.3 us with 12 waves, whose tasks divide evenly among them; 4 tokens 62.5 against 64.2)
+    const int nthr = 1024;
     c.rpi = nthr / a.Ld;
     c.nit = (c.rows_t + c.rpi - 1) / c.rpi;
     c.KP = (a.E + 15) & ~15;
@@ -587,11 +582,7 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     size_t lds = (size_t) c.total * 4;
     if (lds > CU_LDS_MAX) return -1;
     if (lds < CU_LDS_MIN) lds = CU_LDS_MIN;
-    if (P == 4) {
-        if (nthr == 768) return sd ? launch_one<4, true, 768>(st, a, c, lds) : launch_one<4, false, 768>(st, a, c, lds);
-        return sd ? launch_one<4, true, 1024>(st, a, c, lds) : launch_one<4, false, 1024>(st, a, c, lds);
-    }
-    if (nthr == 768) return sd ? launch_one<3, true, 768>(st, a, c, lds) : launch_one<3, false, 768>(st, a, c, lds);
+    if (P == 4) return sd ? launch_one<4, true, 1024>(st, a, c, lds) : launch_one<4, false, 1024>(st, a, c, lds);
     return sd ? launch_one<3, true, 1024>(st, a, c, lds) : launch_one<3, false, 1024>(st, a, c, lds);
 }
 

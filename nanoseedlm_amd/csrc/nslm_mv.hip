@@ -123,15 +123,12 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         wA = a.ws[sl];
         if (MODE == GATEUP) wB = a.wu[sl];
     }
-    const bool al = true;
-
     // first records in flight before the first wait
     int v = v0 + lr;
-    auto fetch = [&](int vv) {
-        const bool ok = active && vv < v1;
-        const int r = MODE == GATEUP ? vv >> 1 : vv;
-        const WSlice& w = (MODE == GATEUP && (vv & 1)) ? wB : wA;
-        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch, ok, al);
+    auto fetch = [&](int vv) {   // (rows past the workgroup's last: its last row's records once more)
+        const int vc = min(vv, v1 - 1), r = MODE == GATEUP ? vc >> 1 : vc;
+        const WSlice& w = (MODE == GATEUP && (vc & 1)) ? wB : wA;
+        return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch);
     };
     Chunk cur = fetch(v);
     loads_issued();

@@ -12,23 +12,29 @@ struct Chunk {
 
 // A chunk's records: 16 bytes of seeds, 16 of coefficient (nibble) words, 4 of exponent codes.  The streams of a slice may start
 // at any 2-byte (codes: 1-byte) boundary - the loads are typed with that alignment, and the target reads a misaligned
-// 16-byte unit in one instruction all the same - so there is one code path, no branch on the alignment and no join for the
-// compiler to put a wait at.  `al` is kept in the signature for the callers and not used.
+// unit in one instruction all the same - so there is one code path and no branch on the alignment.  The loads are
+// unconditional (callers clamp `unit` to a chunk that exists): after a load under a condition the compiler no longer knows how
+// many loads are in flight and waits for all of them before the next use of any loaded value - the activations' staging then
+// waited for the records.
 typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
 typedef uint32_t u32_a1 __attribute__((aligned(1)));
 template <int P>
-__device__ __forceinline__ Chunk load_chunk(const WSlice& w, uint32_t unit, bool ok, bool al) {
-    (void) al;
+__device__ __forceinline__ Chunk load_chunk(const WSlice& w, uint32_t unit) {
     Chunk c;
-    c.sd = make_uint4(0, 0, 0, 0);
-    c.cw = c.sd;
     c.codes = 0;
-    if (!ok) return c;
-    const u32x4_a2 s4 = *(const NSLM_GLOBAL u32x4_a2*) (gp<uint8_t>(w.p[0]) + (size_t) unit * 16);
-    const u32x4_a2 c4 = *(const NSLM_GLOBAL u32x4_a2*) (gp<uint8_t>(w.p[1]) + (size_t) unit * 16);
-    c.sd = make_uint4(s4.x, s4.y, s4.z, s4.w);
-    c.cw = make_uint4(c4.x, c4.y, c4.z, c4.w);
+    // In pieces, in the order the blocks are decoded - the codes, then seeds and coefficient words of blocks 0..3, then of blocks
+    // 4..7: a wave's loads return in the order they went out, and so do the whole launch's requests to the memory, so when every
+    // wave asks for its records at once the first pieces of all of them arrive before any last piece does.  A thread starts
+    // on its first blocks when 20 of its 36 bytes are there.
+    typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+    const NSLM_GLOBAL uint8_t* ps = gp<uint8_t>(w.p[0]) + (size_t) unit * 16;
+    const NSLM_GLOBAL uint8_t* pc = gp<uint8_t>(w.p[1]) + (size_t) unit * 16;
     if (P == 4) c.codes = *(const NSLM_GLOBAL u32_a1*) (gp<uint8_t>(w.p[3]) + (size_t) unit * 4);
+    const u32x2_a2 s0 = *(const NSLM_GLOBAL u32x2_a2*) ps, c0 = *(const NSLM_GLOBAL u32x2_a2*) pc;
+    asm volatile("" ::: "memory");   // (keeps the halves apart: left alone, the compiler joins them into 16-byte loads again)
+    const u32x2_a2 s1 = *(const NSLM_GLOBAL u32x2_a2*) (ps + 8), c1 = *(const NSLM_GLOBAL u32x2_a2*) (pc + 8);
+    c.sd = make_uint4(s0.x, s0.y, s1.x, s1.y);
+    c.cw = make_uint4(c0.x, c0.y, c1.x, c1.y);
     return c;
 }
 __device__ __forceinline__ bool streams_aligned(int P, const WSlice& w) {
