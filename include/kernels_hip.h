@@ -175,7 +175,7 @@ void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out)
 /* kc_mm_grouped_packed for a caller that knows an upper bound of MmTile.count: a decode step of T rows chooses no expert
  * more than T times, so no tile holds more than tile_rows = T pairs.  Up to 32 the launch uses workgroups with one
  * multiplying wave (four a CU instead of two; the tiles are decode-bound).  The bound is a promise: pairs of a tile beyond
- * it are not computed.  tile_rows < 1 or > 32: as kc_mm_grouped_packed. */
+ * it are not computed, and their results are stored as NaN so that a broken promise shows.  tile_rows < 1 or > 32: as kc_mm_grouped_packed. */
 void kc_mm_grouped_packed_rows(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
                                int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
                                int tile_rows);

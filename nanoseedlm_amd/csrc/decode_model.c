@@ -85,7 +85,11 @@ NslmModel* nslm_model_open(const NslmModelCfg* c, char* err, int errlen) {
         return NULL;
     }
     NslmModel* m = (NslmModel*) calloc(1, sizeof *m);
-    if (m) m->next_pos = -1;
+    if (!m) {
+        snprintf(err, (size_t) errlen, "model: out of memory");
+        return NULL;
+    }
+    m->next_pos = -1;
     m->c = *c;
     if (m->c.n_splits <= 0) m->c.n_splits = 32;
     NslmMoeCfg mc = {c->n_layer, c->n_exp, c->top_k, c->d, c->ff, MF_SEED4P4, NSLM_ROUTE_SOFTMAX, c->max_rows, 0, 1.0f, 0, 0};
@@ -404,11 +408,18 @@ int nslm_model_step(NslmModel* m, kc_stream_t s, int T) {
     }
     kc_argmax(s, m->logits, m->ids, c->vocab, T);
     kc_rows_advance(s, m->ri, T);
-    m->next_pos += 1;
-    return kc_last_error() ? -1 : 0;
+    if (kc_last_error()) return -1;            /* (a launch failed: the host's bound stays) */
+    if (!nslm_stream_capturing(s)) m->next_pos += 1;   /* a captured step launched nothing: its replays are counted when launched */
+    return 0;
 }
 
 int nslm_model_steps_left(const NslmModel* m) { return m->next_pos < 0 ? 0 : m->c.max_ctx - m->next_pos; }
+int nslm_model_launch(NslmModel* m, NslmGraph* g, kc_stream_t s) {
+    if (!g || m->next_pos < 0 || m->next_pos >= m->c.max_ctx) return -1;
+    if (nslm_graph_launch(g, s)) return -1;
+    m->next_pos += 1;
+    return 0;
+}
 int nslm_model_account(NslmModel* m, int steps) {
     if (m->next_pos < 0 || m->next_pos + steps > m->c.max_ctx || m->next_pos + steps < 0) return -1;
     m->next_pos += steps;

@@ -60,12 +60,15 @@ int nslm_model_fill_cache(NslmModel* m, int T, int upto, uint64_t seed);
  * two side streams joined by events, which a captured step turns into parallel graph branches.  Steps of up to 8 rows. */
 int nslm_model_set_branches(NslmModel* m, int on);
 /* -1 (nothing launched) when a sequence slot is full: a step writes the cache at every row's position, and the positions
- * advance on the device, so the host keeps the bound - the largest position given to nslm_model_start plus the steps issued
- * since.  A step captured into a graph counts once when captured; replays are accounted with nslm_model_account(m, n)
- * before they are launched (-1: they would run past max_ctx; n < 0 takes steps back, e.g. the capture call itself, which
- * launches nothing).  On the device the positions saturate at max_ctx - 1, so even an unaccounted replay stays inside the cache. */
+ * advance on the device, so the host keeps the bound - the largest position given to nslm_model_start plus the steps that
+ * ran since.  A step that succeeds on a stream that is not capturing counts one; a step recorded into a graph counts
+ * nothing (it launched nothing), and every replay through nslm_model_launch counts one (-1, nothing launched: it would run
+ * past max_ctx).  A caller that replays the graph by other means (as a child of its own graph) accounts with
+ * nslm_model_account(m, n) before it launches (-1: the n steps would run past max_ctx; n < 0 takes steps back).  On the
+ * device the positions saturate at max_ctx - 1, so even an unaccounted replay stays inside the cache. */
 int nslm_model_step(NslmModel* m, kc_stream_t s, int T);
 int nslm_model_steps_left(const NslmModel* m);
+int nslm_model_launch(NslmModel* m, NslmGraph* g, kc_stream_t s);
 int nslm_model_account(NslmModel* m, int steps);
 /* synchronising reads: the current ids, the last step's logits [T][vocab]; -1 also when a wait inside the persistent expert
  * kernel gave up since open (the results are void then) */

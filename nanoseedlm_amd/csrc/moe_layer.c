@@ -33,6 +33,7 @@ struct NslmMoe {
     int fused;                  /* 1: steps of the softmax composition up to kc_moe_decode_max_rows() rows take kc_moe_decode;
                                    2: the same, and every such step is checked and redone by the separate launchers if it failed */
     int fallbacks;              /* checked steps that were redone */
+    long fused_steps;           /* steps the persistent kernel took */
 };
 
 static uint64_t pad256(uint64_t n) { return (n + 255) & ~(uint64_t) 255; }
@@ -291,6 +292,7 @@ int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, i
     if (kc_moe_decode_layer(s, c->fmt, m->rw + (size_t) layer * E * c->d, tab, tab + E, tab + 2 * E, E, c->top_k, c->d, c->ff, xn, c->d, T, out,
                             c->d, m->logit, m->ind, m->wt, m->A, m->D, m->sync, shared, res, norm_w, norm_eps))
         return 1;
+    m->fused_steps++;
     return kc_last_error() ? -1 : 0;
 }
 
@@ -304,6 +306,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
     if (m->fused && m->resident && c->router == NSLM_ROUTE_SOFTMAX && T <= kc_moe_decode_max_rows() &&
         !kc_moe_decode(s, c->fmt, m->rw + (size_t) layer * E * d, gate, up, down, E, k, d, ff, xn, d, T, io, d, m->logit, m->ind,
                        m->wt, m->A, m->D, m->sync)) {   /* the whole step in one persistent kernel */
+        m->fused_steps++;
         if (m->fused != 2) return kc_last_error() ? -1 : 0;
         /* checked: the kernel's workgroups wait for each other, and a wait that gave up (the grid was not resident at once:
            another stream's kernel held the CUs) has left void results and the sync words in no defined state.  Then the words
@@ -402,6 +405,7 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 void nslm_moe_set_fused(NslmMoe* m, int on) { m->fused = on; }
 int nslm_moe_fused_mode(const NslmMoe* m) { return m->fused; }
 int nslm_moe_fallbacks(const NslmMoe* m) { return m->fallbacks; }
+long nslm_moe_fused_steps(const NslmMoe* m) { return m->fused_steps; }
 void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }
 const uint16_t* nslm_moe_router_w(const NslmMoe* m, int layer) { return m->rw + (size_t) layer * m->c.n_exp * m->c.d; }
 int nslm_moe_fused_error(NslmMoe* m) {

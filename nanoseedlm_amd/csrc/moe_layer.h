@@ -65,6 +65,7 @@ int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, i
 void nslm_moe_set_fused(NslmMoe* m, int on);
 int nslm_moe_fused_mode(const NslmMoe* m);
 int nslm_moe_fallbacks(const NslmMoe* m);
+long nslm_moe_fused_steps(const NslmMoe* m);   /* steps that the persistent kernel took (launched, not necessarily without error) */
 /* 0, or non-zero when a grid barrier of the fused kernel gave up since open (synchronises) */
 int nslm_moe_fused_error(NslmMoe* m);
 /* n words of the persistent kernels' sync area from word `first`, copied to the host (synchronises): behind the error word
@@ -97,6 +98,7 @@ typedef struct NslmGraph NslmGraph;
 int nslm_graph_begin(kc_stream_t s);                 /* start capturing s */
 NslmGraph* nslm_graph_end(kc_stream_t s);            /* end capture and instantiate; NULL on failure */
 int nslm_graph_launch(NslmGraph* g, kc_stream_t s);
+int nslm_stream_capturing(kc_stream_t s);           /* 1 while s records into a graph */
 void nslm_graph_free(NslmGraph* g);
 
 #ifdef __cplusplus

@@ -186,9 +186,6 @@ __device__ __forceinline__ void rank_logits(const float* rv, int E, int k, uint3
     }
 }
 
-#ifdef NSLM_FUSED_STAMPS
-__device__ unsigned long long g_fstamp[1024 * 32];
-#endif
 template <int P, bool SHFL_G, bool SHFL_D, int WAVES>
 __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // WAVES waves a SIMD: five = at most 96 registers
     extern __shared__ float xl[];   // activations of the current pair: max(d, ff) floats, chunk-padded
@@ -204,17 +201,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t G = (uint32_t) a.grid;
     const int P_ = a.T * a.kk;
-    // phase timeline of workgroup 0 (wall clock ticks) beside the error word: a built-in profile that costs six stores
-    unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
-#ifdef NSLM_FUSED_STAMPS   // development builds: every workgroup's timeline
-#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); if (blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + (i)] = wall_clock64(); } } while (0)
-#define DSTAMP(i) do { if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + (i)] = wall_clock64(); } while (0)
-    if (tid == 0 && blockIdx.x < 1024) g_fstamp[blockIdx.x * 32 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
-#else
-#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)   // i < 6: the stamps share the error word's line
-#define DSTAMP(i) do { } while (0)
-#endif
-    STAMP(0);
     // the generation: lane 0 of every wave reads it (all sense words are equal); the workgroup arrives further down
     const uint32_t my_gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
     unsigned long long* lg64 = (unsigned long long*) (a.sync + FUSED_LOGIT_WORDS);
@@ -248,7 +234,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         staged = ((int) blockIdx.x / a.ntile_g) / a.kk;
         stage_input<P>(a.x + (size_t) staged * a.xs, a.d, xl, a.nw, a.nw ? rn_s[staged] : 1.0f);
     }
-    STAMP(1);
     // No grid barrier: what the other workgroups produce here are the logits, and those say themselves when they are there.
     __syncthreads();   // every wave has used its copy of the generation
     uint32_t arrived = 0;
@@ -256,7 +241,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         s_tag = my_gen + 1u;
         arrived = arrive_issue(a.sync, my_gen);
     }
-    STAMP(2);
 
     // ---- route: every workgroup ranks the logits of the token it needs itself (cheap, and nobody waits for a router) ----
     // rank(e) = how many experts come before e (larger logit, or equal logit and higher index): k_q4_route's order
@@ -284,29 +268,14 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             rv[e] = v;
         }
         __syncthreads();
-        unsigned long long tq[4] = {0, 0, 0, 0};
-        (void) tq;
-#ifdef NSLM_FUSED_STAMPS
-        tq[0] = wall_clock64();
-#endif
         rank_logits(rv, a.E, a.k, (uint32_t*) &part[0][0], ri_s);
-#ifdef NSLM_FUSED_STAMPS
-        tq[1] = wall_clock64();
-#endif
         __syncthreads();
-#ifdef NSLM_FUSED_STAMPS
-        tq[2] = wall_clock64();
-#endif
         if (tid < 3 * a.k) {   // the chosen experts' slices, fetched side by side
             const int which = tid / a.k, j = tid - which * a.k;
             sl_s[which][j] = (which == 0 ? a.gate : which == 1 ? a.up : a.down)[ri_s[j]];
         }
         if (a.ns && tid >= 253) sl_s[tid - 253][a.k] = a.sh[tid - 253];
         __syncthreads();
-#ifdef NSLM_FUSED_STAMPS
-        tq[3] = wall_clock64();
-        if (tid == 0 && blockIdx.x < 1024) for (int q = 0; q < 4; ++q) g_fstamp[blockIdx.x * 32 + 11 + q] = tq[q];
-#endif
         weighted = false;
     };
     // The routing weights of the token last routed: softmax over the k chosen logits.  Only the combine needs them, so this
@@ -333,7 +302,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
-        if (item == (int) blockIdx.x) DSTAMP(8);
         const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
         const Chunk c0 = first_chunk<P, true>(sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1);
         route_weights(t);
@@ -343,11 +311,9 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             staged = t;
             __syncthreads();
         }
-        if (item == (int) blockIdx.x) DSTAMP(9);
         float* Ap = a.A + (size_t) p * a.ff;
         rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
                                    [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
-        if (item == (int) blockIdx.x) DSTAMP(10);
         wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
         __syncthreads();
         if (tid == 0 && atomicAdd(&pairw[p * 64], 1u) == (uint32_t) (a.ntile_g - 1)) {
@@ -361,7 +327,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         route_weights(t);
     }
     if (tid == 0) arrive_finish(a.sync, G, my_gen, arrived);   // here most workgroups are about to wait for their pair anyway
-    STAMP(3);
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
     // the first down item's records do not depend on phase 2: they are requested before the wait for the pair
@@ -393,15 +358,12 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         }
         __syncthreads();
         wg_acquire();
-        if (item == (int) blockIdx.x) STAMP(4);   // the first down item's pair is ready
         stage_row<P>(a.A + (size_t) p * a.ff, a.ff, xl, true);
         staged = -1;
         __syncthreads();
-        if (item == (int) blockIdx.x) DSTAMP(16);
         float* Dp = a.D + (size_t) p * a.d;
         rows_pass<P, false, SHFL_D>(d0, sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1, tab, xl, part,
                                     [&](int r, float s, float) { st_agent(Dp + r, bfr(s)); });
-        if (item == (int) blockIdx.x) DSTAMP(17);
         wg_release();
         __syncthreads();
         if (j != a.kk - 1) {
@@ -420,7 +382,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             }
             __syncthreads();
             wg_acquire();
-            if (item == (int) blockIdx.x) DSTAMP(18);
             for (int r = v0 + tid; r < v1; r += 256) {
                 float acc = 0.0f;
                 for (int jj = 0; jj < a.kk; ++jj) acc = fmaf(rw_s[jj], ld_agent(a.D + ((size_t) t * a.kk + jj) * a.d + r), acc);
@@ -428,9 +389,6 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             }
         }
     }
-    STAMP(5);
-#undef STAMP
-#undef DSTAMP
 }
 
 // ---- 9 to 24 tokens: the pairs of one expert share its decoded blocks ---------------------------------------------------
@@ -1005,6 +963,14 @@ int kc_moe_decode_static(kc_stream_t s, int fmt, const uint16_t* router_w, const
         host_note_unsupported();
         return -3;
     }
+    // what kc_moe_decode_layer would refuse is refused here, before anything is launched (the clear included)
+    {
+        int L1, r1;
+        bool s1;
+        if ((fmt != MF_SEED4P4 && fmt != MF_SEED4) || n_exp < top_k || host_store_f32() || d % 8 || ((uintptr_t) x & 15u) || xs % 4 || ((uintptr_t) router_w & 15u) ||
+            !shape_of(d, true, &L1, &r1, &s1) || (T > MV_MAXT && (!s1 || T * top_k > FG_MAXP)))
+            return -1;
+    }
     if (clear) {   // by a kernel, not a memset node: callers may be capturing
         hipLaunchKernelGGL(k_words_zero, dim3(64), dim3(256), 0, (hipStream_t) s, base, (size_t) NA_SYNC_WORDS);
         host_note_launch();
@@ -1023,8 +989,3 @@ int kc_moe_decode_static(kc_stream_t s, int fmt, const uint16_t* router_w, const
 
 }   // extern "C"
 
-#ifdef NSLM_FUSED_STAMPS
-extern "C" int kc_moe_decode_stamps(unsigned long long* host) {
-    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_fstamp), sizeof(unsigned long long) * 1024 * 32);
-}
-#endif

@@ -69,9 +69,6 @@ struct CuParams {
     FastDiv by_tpp, by_rpc, by_Ld, by_nbp, by_kk, by_E;
 };
 
-#ifdef NSLM_CU_STAMPS
-__device__ unsigned long long g_cstamp[4096 + 256 * 16 * 8];
-#endif
 template <int P, bool SHFL_D, int NTHR>
 __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c) {
     constexpr int NW = NTHR / 64, XP = xpad<P>();
@@ -94,18 +91,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     float* const avs = dyn + c.av;
     float* const lgs = dyn + c.lgs;
     const bool preload = E <= CU_PRE_MAXE;
-    // phase timeline of workgroup 0 (wall clock ticks) beside the error word
-    unsigned long long* stamp = (unsigned long long*) (a.sync + FUSED_ERR_WORD + 2);
-#ifdef NSLM_CU_STAMPS   // development builds: every workgroup's timeline
-#define STAMP(i) do { if (tid == 0) { if (blockIdx.x == 0) stamp[i] = wall_clock64(); g_cstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } } while (0)
-#define WSTAMP(i) do { if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + (i)] = wall_clock64(); } while (0)
-#define DSTAMP(i) do { if (tid == 0) g_cstamp[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
-#else
-#define STAMP(i) do { if (blockIdx.x == 0 && tid == 0) stamp[i] = wall_clock64(); } while (0)
-#define WSTAMP(i) do { } while (0)
-#define DSTAMP(i) do { } while (0)
-#endif
-    STAMP(0);
 
     // ---- what does not depend on the routing: generation, tables, slice tables, norm scales, the staged input, the logits ----
     const uint32_t gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
@@ -155,7 +140,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         const int u = NW - 1 - wv, item = lg0 + u, t = (int) ((uint32_t) item / c.by_E), e = item - t * E;
         const float lv = router_logit(a.rw + (size_t) e * a.d, a.x + (size_t) t * a.xs, a.d, a.nw, a.nw ? rn_s[t] : 1.0f);
         if (lane == 0) lgs[u] = lv;
-        WSTAMP(4);
     }
     tables_store<NTHR>(tab, tw);
     if (preload) {
@@ -187,7 +171,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         if (tid == 2) PUT_SH(2);
 #undef PUT_SH
     }
-    STAMP(1);
     __syncthreads();   // every wave has used its copy of the generation; tables, slice tables, inputs and this CU's logits are in LDS
     if (tid < lgn) {
         const float lv = lgs[tid];
@@ -228,7 +211,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             pk[t * c.KP + e] = key;
         }
     __syncthreads();
-    STAMP(2);
     // four lanes an expert, each counts over a quarter of the token's keys (read four at a time as LDS broadcasts); the quarters
     // meet by two shuffles, so a rank needs no second pass through LDS
     {
@@ -250,7 +232,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             }
     }
     __syncthreads();
-    DSTAMP(8);
     // the routing weights (softmax over the k chosen logits): wave t for token t (the combine reads them, barriers later)
     if (wv < T) {
         const int t = wv;
@@ -286,7 +267,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         if (preload) return ((const WSlice*) pre)[which * E + ri_s[t * 32 + j]];
         return sel[3 + (t * kk + j) * 3 + which];
     };
-    STAMP(3);
 
     // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
     const int q_lo = (int) blockIdx.x * c.n_c, n_loc = max(0, min(c.n_c, c.Wt - q_lo));   // this CU's tasks a token
@@ -318,10 +298,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         int t, i;
         claim(t, i);
         Chunk cur = fetch(t, i);
-        WSTAMP(0);
-#ifdef NSLM_CU_STAMPS
-        const unsigned long long ck0 = clock64();
-#endif
         uint32_t mine = 0;   // tasks of the token in hand this wave has finished
         const int nav = c.n_c << c.lgV;   // SwiGLU outputs a CU and token at most
         while (t < T) {
@@ -337,18 +313,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             // (results leave after the loop: a store here would sit in front of the wait for the next task's records)
             if (ch == 0 && !(v & 1)) avs[t * nav + (i << c.lgV) + (lr >> 1)] = bfr(silu_bf(bfr(s * NSLM_R32)) * bfr(other * NSLM_R32));
             ++mine;
-#ifdef NSLM_CU_STAMPS
-            if (mine == 1) WSTAMP(5);
-            if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 6] = mine;
-            if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 7] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
-#endif
             if (tn != t) {   // The wave's last task of token t: it adds its tasks to the CU's count.  The wave that completes the
                              // count stores the CU's values of the token (as BF16 for the other CUs, as f32 for the caller), and once
                              // they are acknowledged arrives for the CU; the last CU of all raises the token's ready words.
-                WSTAMP(1);
-#ifdef NSLM_CU_STAMPS
-                if (lane == 0) g_cstamp[4096 + (blockIdx.x * 16 + wv) * 8 + 3] = clock64() - ck0;
-#endif
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 uint32_t before = 0;
                 if (lane == 0) before = atomicAdd(&cnt_s[MV_MAXT + t], mine);
@@ -378,7 +345,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                     }
                 }
                 mine = 0;
-                WSTAMP(2);
             }
             cur = nxt;
             t = tn;
@@ -395,7 +361,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         for (int w = (int) blockIdx.x * NTHR + tid; w < (FUSED_CULG_LINES - used) * 16; w += G * NTHR) st_agent(lg64 + 16 * used + w, 0ull);
     }
     if (tid == 0) arrive_finish(a.sync, (uint32_t) G, gen, arrived);
-    STAMP(4);
 
     // ---- down: CU c owns rows [c rpc, (c + 1) rpc) of every pair; a thread a chunk of a (pair, row); then the experts' sum --------
     const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
@@ -421,7 +386,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             }
         }
         __syncthreads();
-        if (t == 0) STAMP(5);
         // all pairs' A of the token, 16 bytes (a block of 8 values) a thread, staged as the down matvec reads it
         for (int b = tid; b < kk * c.nbp; b += NTHR) {
             const int j = (int) ((uint32_t) b / c.by_nbp), bb = b - j * c.nbp;
@@ -432,7 +396,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             store_block<P>(xd + j * (Ld * XP), bb, v);
         }
         __syncthreads();
-        if (t == 0) STAMP(6);
         for (int it = 0; it < c.nit; ++it) {
             const bool last = it + 1 == c.nit;
             const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
@@ -493,10 +456,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         // (the next token's staging writes xd, which every thread has finished reading before the barrier above; dsum and part
         // are next written behind the next token's first barrier)
     }
-    STAMP(7);
-#undef STAMP
-#undef WSTAMP
-#undef DSTAMP
 }
 
 template <int P, bool SD, int NTHR>
@@ -588,8 +547,3 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
 
 }   // namespace nslm
 
-#ifdef NSLM_CU_STAMPS
-extern "C" int kc_moe_decode_cu_stamps(unsigned long long* host) {
-    return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_cstamp), sizeof(unsigned long long) * (4096 + 256 * 16 * 8));
-}
-#endif

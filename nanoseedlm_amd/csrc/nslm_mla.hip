@@ -395,11 +395,6 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
     int p0, p1;
     split_range(a, pos, split, &p0, &p1);
     const bool live = h < a.n_head;
-#ifdef NSLM_MLA_DEV   // development builds only: a.pad[1] switches parts of the tile loop off (1 loads, 2 decode, 4 scores, 8 P c)
-    const int abl = a.pad[1];
-#else
-    constexpr int abl = 0;
-#endif
 
     // The group's queries, staged once for the four waves: thread e loads 4 consecutive values of head e / 128 (latent) or
     // e / 16 (RoPE part); heads past n_head read head 0 and are zeroed.  The loads are issued here and converted after the
@@ -431,7 +426,6 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
     };
     // Keys past the split's end read its last key (finite values; their scores are masked), so no load is conditional.
     auto load_tile = [&](int p) {
-        if (abl & 1) return;
         const int rb = kv0 + p, last = p1 - 1 - p;
         if (rb + MA_KB <= kv.nv || rb >= kv.nv) {   // the tile lies in one segment of the view (uniform): 32-bit offsets from its first row
             const bool first = rb < kv.nv;
@@ -496,7 +490,6 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
         }
     };
     auto store_tile = [&]() {
-        if (abl & 2) return;
         uint32_t D[8][4], dr[4];
         bool exact = false;
         if (FMT == KV_FP8) {
@@ -574,7 +567,6 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
         f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;   // two chains over the wave's 9 k-slices
 #pragma unroll
         for (int ks = 0; ks < KH; ++ks) {
-            if (abl & 4) break;
             const bf16x8 a0 = *(const bf16x8*) &Ks[(16 * su + c) * KLD + 32 * (sk + ks) + 8 * g];
             if (ks & 1) s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s1, 0, 0, 0);
             else s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
@@ -611,7 +603,6 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
         const bf16x8 ph = __builtin_bit_cast(bf16x8, bh), pl = __builtin_bit_cast(bf16x8, bl);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (abl & 8) break;
             const int tile = w * MT + mt;
             const bf16x8 vt = *(const bf16x8*) &Vt[(16 * tile + c) * MA_KB + 8 * (g ^ ((c >> 1) & 3) ^ (tile & 3))];
             acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vt, ph, acc[mt], 0, 0, 0);

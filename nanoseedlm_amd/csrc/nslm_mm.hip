@@ -368,13 +368,6 @@ struct MmRec2 {
     uint32_t u, v, c;  // seeds: two seeds, two coefficient words, the codes byte; Q8 / Q4: the group's scale and bias bits
 };
 
-#ifdef NSLM_MM_STAMPS   // development builds only: wall-clock stamps of every workgroup behind the T x ys results
-#define MM_STAMP(t, step, slot) do { } while (0)
-#define MM_WG_STAMP(t, slot) do { if (tid == (t)) { ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + (slot)] = wall_clock64(); ((unsigned long long*) (Y + (size_t) a.T * a.ys))[blockIdx.x * 8 + 4 + (slot)] = clock64(); } } while (0)
-#else
-#define MM_STAMP(t, step, slot) do { } while (0)
-#define MM_WG_STAMP(t, slot) do { } while (0)
-#endif
 template <int CT, int NCW, int XCH, int FMT>
 __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice wd, const WSlice* ws, const uint16_t* X, float* Y,
                                                    const int32_t* perm, const MmTile* tiles, const int32_t* ntiles) {
@@ -387,7 +380,6 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     __shared__ int srow[BN], drow[BN];
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
-    MM_WG_STAMP(0, 0);
     const bool producer = wv >= NCW;
     const bool grouped = tiles != nullptr;
     if (grouped && ntiles && (int) blockIdx.y >= *ntiles) return;
@@ -399,6 +391,13 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         wt = ws[tl.slice];
         start = tl.start;
         count = min(tl.count, BN);   // (a tile never holds more than the launch was told: see mm_grouped)
+        if (BN < MMT_BN && tl.count > BN) {
+            // a broken promise is made visible: the pairs this launch cannot reach are stored as NaN, not left stale
+            for (int i = BN * BM + tid; i < tl.count * BM; i += NTHR) {
+                const int orow = r0 + i % BM;
+                if (orow < a.R) Y[(size_t) perm[tl.start + i / BM] * a.ys + orow] = __uint_as_float(0x7FC00000u);
+            }
+        }
     } else {
         wt = wd;
         start = (int) blockIdx.y * BN;
@@ -499,7 +498,6 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
                     }
                 }
             }
-            MM_STAMP(256, s, 10);
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 *(uint4*) &Wsm[s & 1][rr][16 * jb + 8 * h] = make_uint4(cvt_pk_bf16(f[h][0], f[h][1]), cvt_pk_bf16(f[h][2], f[h][3]),
@@ -515,9 +513,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
             lookup(rec[(u + 1) % RECD], look[(u + 1) & 1]);   // the next step's table reads travel under this step's decode
             produce(s, rec[u], look[u & 1]);
             load_rec(s + RECD, rec[u]);
-            MM_STAMP(256, s, 8);
             lds_barrier();
-            MM_STAMP(256, s, 9);
         };
         // whole rounds of the record ring in a loop with one way out (a conditional exit per step costs the loop a
         // register move per record word and step), the steps left over after it
@@ -578,9 +574,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     // One weight step: chunk m multiplies out of fragment set (m even ? fa : fb) while the next chunk's fragments travel
     // into the other set; with MT odd the sets have swapped roles when the step ends.
     auto step = [&](int s, bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
-        MM_STAMP(0, s, 0);
         lds_barrier();   // weight step s is in tile s & 1
-        MM_STAMP(0, s, 1);
         bf16x8 bq[4][2];
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
@@ -597,10 +591,8 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
 #pragma unroll
                 for (int n = 0; n < 2; ++n)
                     acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(((m & 1) ? fb : fa)[kk], bq[kk][n], acc[m][n], 0, 0, 0);
-            MM_STAMP(0, s, 2 + m);
         }
     };
-    MM_WG_STAMP(0, 1);
     if (nsteps > 0) {
 #pragma unroll
         for (int c = 0; c < XCH - 1; ++c) fetch(c / CT, c % CT, c);
@@ -615,7 +607,6 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         else step(s + 1, f0, f1);
     }
     wait_vm<0>();
-    MM_WG_STAMP(0, 2);
     // accumulator element v of lane l: token row 8 * (v / 4) + 4 * (l / 32) + v % 4, weight column l % 32
     const bool plain = !a.add && !a.f32out;
 #pragma unroll
@@ -634,7 +625,6 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
                 else store_y(yo, acc[m][n][v], a.add, a.f32out);
             }
         }
-    MM_WG_STAMP(0, 3);
 }
 template <int NCW, int XCH>
 constexpr size_t mm_stream_lds() { return (size_t) (NCW * XCH * XCHUNK + 2 * BM * LDW2) * sizeof(uint16_t); }

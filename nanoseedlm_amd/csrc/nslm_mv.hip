@@ -50,12 +50,6 @@ struct MvArgs {
 
 enum { DENSE = 0, GATHER = 1, GATEUP = 2, MULTI = 3 };
 
-#ifdef NSLM_MV_STAMPS   // development builds only: wall-clock stamps of every workgroup
-__device__ unsigned long long g_mvstamp[8192 * 16];
-#define MV_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 8192) { g_mvstamp[blockIdx.x * 16 + (i)] = wall_clock64(); g_mvstamp[blockIdx.x * 16 + 8 + (i)] = clock64(); } } while (0)
-#else
-#define MV_STAMP(i) do { } while (0)
-#endif
 // SHFL: L is a power of two <= 64 (<= 32 for GATEUP): row sums by wave shuffles, no barrier.  Otherwise through LDS.
 // NTHR: threads a workgroup (256; 512 or 1024 for one-token SHFL launches whose rows fill more than four waves a CU - the
 // row and the tables are then fetched once per CU instead of once per four waves).
@@ -76,7 +70,6 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
     const int tid = threadIdx.x, L = a.L, rpi = a.rpi;
     const int lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
-    MV_STAMP(0);
     constexpr bool DN = MODE == DENSE || MODE == MULTI;   // all tokens against one matrix
     const int pair = DN ? 0 : (int) blockIdx.y;
     int job = 0, wg = (int) blockIdx.x;
@@ -132,7 +125,6 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
     };
     Chunk cur = fetch(v);
     loads_issued();
-    MV_STAMP(5);
     if (NT == 1) {
         // The row goes through LDS once per workgroup and from there into each thread's registers (the 256 / L threads that
         // share a chunk do not each fetch it).  Every load of the prologue - tables, row, records - is requested before the
@@ -199,7 +191,6 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
             xreg[4 * i] = q.x; xreg[4 * i + 1] = q.y; xreg[4 * i + 2] = q.z; xreg[4 * i + 3] = q.w;
         }
     }
-    MV_STAMP(1);
 
     const int eA = wA.eb, eB = wB.eb;
     const bool single = SHFL && MODE != GATEUP && v1 - v0 <= rpi;   // (uniform over the workgroup)
@@ -257,7 +248,6 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
             }
         }
         cur = nxt;
-        MV_STAMP(2 + min((vb - v0) / rpi, 4));
     }
     if (single) return;
     __syncthreads();
@@ -268,11 +258,7 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         if (MODE == GATEUP) *yo = ybuf[t][r];
         else store_y(yo, ybuf[t][r], add, a.f32out);
     }
-    MV_STAMP(7);
 }
-#ifdef NSLM_MV_STAMPS
-extern "C" int kc_mv_stamps(unsigned long long* host) { return (int) hipMemcpyFromSymbol(host, HIP_SYMBOL(g_mvstamp), sizeof(unsigned long long) * 8192 * 16); }
-#endif
 
 // ---- generic path: every format, one wave per row --------------------------------------------------------------------
 template <int MODE>

@@ -118,6 +118,10 @@ NslmGraph* nslm_graph_end(void* s) {
     return new NslmGraph{g, ex};
 }
 int nslm_graph_launch(NslmGraph* g, void* s) { return (int) hipGraphLaunch(g->exec, (hipStream_t) s); }
+int nslm_stream_capturing(void* s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing((hipStream_t) s, &st) == hipSuccess && st == hipStreamCaptureStatusActive;
+}
 void nslm_graph_free(NslmGraph* g) {
     if (!g) return;
     (void) hipGraphExecDestroy(g->exec);

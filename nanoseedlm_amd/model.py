@@ -87,15 +87,13 @@ class DecodeModel:
         backend.check(self.L.nslm_graph_begin(stream), "nslm_graph_begin")
         self.step(stream, T)
         g = C.c_void_p(self.L.nslm_graph_end(stream))
-        backend.check(self.L.nslm_model_account(self.h, -1), "nslm_model_account")   # the capture call launched nothing
         if not g:
             raise RuntimeError("graph capture failed")
         return g
 
     def launch(self, g, stream):
         """One replay of a captured step; refused (RuntimeError) when a sequence slot is full."""
-        backend.check(self.L.nslm_model_account(self.h, 1), "nslm_model_account: the cache slot is full")
-        backend.check(self.L.nslm_graph_launch(g, stream), "nslm_graph_launch")
+        backend.check(self.L.nslm_model_launch(self.h, g, stream), "nslm_model_launch: the cache slot is full, or the launch failed")
 
     def steps_left(self):
         return int(self.L.nslm_model_steps_left(self.h))

@@ -161,6 +161,11 @@ class MoeStack:
     def fallbacks(self):
         return self.L.nslm_moe_fallbacks(self.h)
 
+    def fused_steps(self):
+        """Steps that the persistent kernel took since the stack was made."""
+        self.L.nslm_moe_fused_steps.restype = C.c_long
+        return int(self.L.nslm_moe_fused_steps(self.h))
+
     def fused_error(self):
         return self.L.nslm_moe_fused_error(self.h)
 

@@ -661,17 +661,13 @@ def test_route_bucket_equals_route_then_bucket(E, k, T):
         b.free()
 
 
-@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
-@pytest.mark.parametrize("T", [3, 20, 32])
-def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
-    """kc_mm_grouped_packed_rows with the caller's bound on the pairs of a tile (a decode step of T rows: no expert more than
-    T times) against kc_mm_grouped_packed on the same tiles, bit for bit - the narrow workgroup shape changes no sum.  R 72:
-    not a multiple of a tile; top-4 of 9 experts, so most experts hold several pairs."""
+def _grouped_rows_case(fmt, T, ind, rng):
+    """kc_bucket on ind [T][4] of 9 experts, then kc_mm_grouped_packed and kc_mm_grouped_packed_rows(tile_rows = T) on the same
+    tiles (R 72: not a multiple of a tile): both results as uint32 [P][R], and the permutation."""
     import ctypes as C
     from nanoseedlm_amd import backend, moe
     backend.require_gpu()
     L = backend.hip()
-    rng = np.random.default_rng(100 * fmt + T)
     E, k, R, K = 9, 4, 72, 256
     p = make_pack(rng, fmt, E, R, K)
     seeds = moe.DevBuf.from_array(p["seeds"])
@@ -687,8 +683,7 @@ def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
     tab = moe.DevBuf(C.sizeof(arr))
     backend.check(L.nh_memcpy_h2d(tab.ptr, arr, C.c_size_t(C.sizeof(arr))), "nh_memcpy_h2d")
     P = T * k
-    ind = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)   # distinct experts a row
-    di = moe.DevBuf.from_array(ind)
+    di = moe.DevBuf.from_array(np.ascontiguousarray(ind, dtype=np.int32))
     mt = P // 128 + E + 1
     perm, tiles, work = moe.DevBuf(4 * P), moe.DevBuf(16 * mt), moe.DevBuf(4 * (2 * E + 4))
     L.nh_memset(work.ptr, 0, C.c_size_t(work.nbytes))
@@ -703,8 +698,33 @@ def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
     L.kc_mm_grouped_packed_rows(None, fmt, tab.ptr, K, R, x.ptr, K, yb.ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T)
     moe.device_sync()
     assert L.kc_last_error() == 0
-    a, b = ya.to_array(np.uint32, (P, R)), yb.to_array(np.uint32, (P, R))
-    assert not (a == 0xFFFFFFFF).any()
-    assert np.array_equal(a, b)
+    a, b, pm = ya.to_array(np.uint32, (P, R)), yb.to_array(np.uint32, (P, R)), perm.to_array(np.int32, (P,))
     for buf in (seeds, words, tab, di, perm, tiles, work, x, ya, yb) + ((codes,) if codes is not None else ()):
         buf.free()
+    return a, b, pm
+
+
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+@pytest.mark.parametrize("T", [3, 20, 32])
+def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
+    """kc_mm_grouped_packed_rows with the caller's bound on the pairs of a tile (a decode step of T rows: no expert more than
+    T times) against kc_mm_grouped_packed on the same tiles, bit for bit - the narrow workgroup shape changes no sum.
+    Top-4 of 9 experts, so most experts hold several pairs."""
+    rng = np.random.default_rng(100 * fmt + T)
+    ind = np.stack([rng.permutation(9)[:4] for _ in range(T)])   # distinct experts a row
+    a, b, _ = _grouped_rows_case(fmt, T, ind, rng)
+    assert not (a == 0xFFFFFFFF).any()
+    assert np.array_equal(a, b)
+
+
+def test_mm_grouped_packed_rows_marks_a_broken_bound():
+    """The bound is the caller's promise.  Indices that break it (10 rows that all name expert 2 four times: one tile of 40
+    pairs under tile_rows = 10) leave the tile's first 32 pairs as kc_mm_grouped_packed computes them and the pairs beyond as
+    NaN - never the buffer's old contents."""
+    rng = np.random.default_rng(77)
+    T = 10
+    a, b, pm = _grouped_rows_case(packs.MF_SEED4P4, T, np.full((T, 4), 2), rng)
+    assert not (a == 0xFFFFFFFF).any()
+    assert np.array_equal(np.sort(pm), np.arange(40))
+    assert np.array_equal(b[pm[:32]], a[pm[:32]])
+    assert (b[pm[32:]] == 0x7FC00000).all()

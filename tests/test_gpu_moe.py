@@ -333,6 +333,41 @@ def test_steps_of_changing_size_share_the_barrier_words():
     st.close()
 
 
+def test_small_shape_then_long_rows_in_one_process():
+    """The per-item step kernel's launcher keeps the number of workgroups a CU holds per kernel variant; the LDS a workgroup
+    asks for grows with the longer of hidden and expert width (8192: 51,200 bytes, above the 48 KB a kernel may have without
+    asking).  A small shape first, then the long rows, in one process, through that kernel: no wait gives up, and the bits
+    are those of the separate launches."""
+    from nanoseedlm_amd import backend, moe
+    L = backend.hip()
+    rng = np.random.default_rng(8192)
+    L.kc_moe_decode_kernel(1)   # the per-item kernel at every size
+    try:
+        for d, ff in ((256, 192), (8192, 512), (256, 192)):
+            E, k = 4, 2
+            st = moe.MoeStack(1, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=8)
+            gate, up, down = packs.seed4p4(rng, E, ff, d, eb=-23), packs.seed4p4(rng, E, ff, d, eb=-23), packs.seed4p4(rng, E, d, ff, eb=-22)
+            st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+            st.finalize()
+            for T in (1, 8):
+                dx = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32)))
+                outs = []
+                for fused in (1, 0):
+                    st.set_fused(fused)
+                    dio = moe.DevBuf.from_array(np.zeros((T, d), dtype=np.float32))
+                    st.step(None, 0, dx.ptr, T, dio.ptr)
+                    outs.append(dio.to_array(np.float32, (T, d)))
+                    dio.free()
+                    assert st.fused_error() == 0, (d, T, fused)
+                dx.free()
+                assert np.abs(outs[1]).max() > 0
+                assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), (d, T)
+            assert st.fused_steps() == 2   # both sizes went through the kernel, none was refused to the separate launches
+            st.close()
+    finally:
+        L.kc_moe_decode_kernel(0)
+
+
 def _small_stack(rng, E=32, k=4, d=512, ff=256, nl=2):
     from nanoseedlm_amd import moe
     st = moe.MoeStack(nl, E, k, d, ff, fmt=packs.MF_SEED4P4, router=moe.ROUTE_SOFTMAX, max_rows=24)
