@@ -52,7 +52,7 @@ struct CuParams {
     int rw;      // [T][36] weight by rank (+ the shared expert's 1)
     int rn;      // [MV_MAXT + 16] the rows' RMSNorm scales, the waves' partial sums of a norm
     int cnt;     // [2][MV_MAXT] per token: this CU's gate + up tasks handed out / finished
-    int av;      // [T][n_c * vpt] this CU's SwiGLU outputs until the token's last task is done
+    int av;      // [T][n_c * vpt][2] this CU's gate and up row sums until the token's last task is done
     int lgs;     // [16] the logits this CU forms, until one wave stores them
     int sel;     // [3 + T * kk * 3] WSlice: the shared expert's slices; with more than CU_PRE_MAXE experts the pairs' slices
     int pre;     // [3][E] WSlice: the layer's slice tables (E <= CU_PRE_MAXE)
@@ -95,16 +95,12 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     // ---- what does not depend on the routing: generation, tables, slice tables, norm scales, the staged input, the logits ----
     const uint32_t gen = ld_agent(a.sync + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS));
     const TableWords<NTHR> tw = tables_fetch<NTHR>();
-    // the layer's three slice tables, 16 bytes a thread and round, three rounds (unconditional: with more experts than the LDS
-    // copy takes, pieces that are not kept)
-    static_assert(3 * CU_PRE_MAXE * sizeof(WSlice) / 16 <= 3 * NTHR, "three rounds cover the slice tables");
-    const int per = E * (int) (sizeof(WSlice) / 16), npre = 3 * per;   // 16-byte pieces of a table, of the three
-    auto pre_piece = [&](int u) {
-        const int i = min(tid + u * NTHR, npre - 1), which = (i >= per ? 1 : 0) + (i >= 2 * per ? 1 : 0);
-        const WSlice* tb = which == 0 ? a.gate : which == 1 ? a.up : a.down;
-        return *((const uint4*) tb + (i - which * per));
-    };
-    const uint4 pw0 = pre_piece(0), pw1 = pre_piece(1), pw2 = pre_piece(2);
+    // the layer's three slice tables, 16 bytes of each a thread (unconditional: with more experts than the LDS copy takes,
+    // pieces that are not kept)
+    static_assert(CU_PRE_MAXE * sizeof(WSlice) / 16 <= NTHR, "a thread a piece covers a slice table");
+    const int per = E * (int) (sizeof(WSlice) / 16);   // 16-byte pieces of a table
+    const int piece = min(tid, per - 1);
+    const uint4 pw0 = ((const uint4*) a.gate)[piece], pw1 = ((const uint4*) a.up)[piece], pw2 = ((const uint4*) a.down)[piece];
     loads_issued();
     if (a.nw) {   // the rows' scales, as the norm kernel sums them: 256 threads, thread i takes x[i], x[i + 256], ..
         for (int t = 0; t < T; ++t) {
@@ -142,10 +138,10 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         if (lane == 0) lgs[u] = lv;
     }
     tables_store<NTHR>(tab, tw);
-    if (preload) {
-        if (tid < npre) pre[tid] = pw0;
-        if (tid + NTHR < npre) pre[tid + NTHR] = pw1;
-        if (tid + 2 * NTHR < npre) pre[tid + 2 * NTHR] = pw2;
+    if (preload && tid < per) {
+        pre[tid] = pw0;
+        pre[per + tid] = pw1;
+        pre[2 * per + tid] = pw2;
     }
     {   // the tokens' inputs, normalised on the way when nw is given (the values kq4_norm1p would have stored)
         const int nb = a.d >> 3;
@@ -271,6 +267,16 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
     const int q_lo = (int) blockIdx.x * c.n_c, n_loc = max(0, min(c.n_c, c.Wt - q_lo));   // this CU's tasks a token
     const int lr = lane >> c.lgL, ch = lane & (Lg - 1);
+    // a lane's share of a task's addresses, formed once: gate or up (a task's rows come in pairs: Lg <= 32), and where in the
+    // task's records the lane reads
+    const int wsel = lr & 1;
+    const uint32_t lane_unit = (uint32_t) (lr >> 1) * (uint32_t) Lg + (uint32_t) ch;
+    const WSlice* const lane_pre = (const WSlice*) pre + wsel * E;
+    auto slice_gu = [&](int t, int j) -> const WSlice& {   // slice(t, j, wsel) with the lane's part taken out
+        if (j >= a.k) return sel[wsel];
+        if (preload) return lane_pre[__builtin_amdgcn_readfirstlane(ri_s[t * 32 + j])];
+        return sel[3 + (t * kk + j) * 3 + wsel];
+    };
     {
         // The CU's tasks of a token go to whichever wave asks next: a wave whose records arrive late, or that shares its SIMD
         // with more waves, takes fewer.  A wave asks for its next task before it computes the current one, so that task's
@@ -291,9 +297,8 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         // before it computes the current one)
         auto fetch = [&](int t, int i) {
             const bool ok = t < T;
-            const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), v = (q - j * c.tpp) * c.rpw + lr;
-            const WSlice& w = slice(ok ? t : 0, j, v & 1);
-            return load_chunk<P>(w, (uint32_t) (v >> 1) * (uint32_t) Lg + (uint32_t) ch);
+            const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), r = (q - j * c.tpp) << c.lgV;   // the task's first SwiGLU row
+            return load_chunk<P>(slice_gu(ok ? t : 0, j), (uint32_t) r * (uint32_t) Lg + lane_unit);
         };
         int t, i;
         claim(t, i);
@@ -304,14 +309,15 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             int tn, inx;
             claim(tn, inx);
             const Chunk nxt = fetch(tn, inx);
-            const int q = q_lo + i, j = (int) ((uint32_t) q / c.by_tpp), v = (q - j * c.tpp) * c.rpw + lr;
+            const int q = q_lo + i, j = (int) ((uint32_t) q / c.by_tpp);
             float acc[1] = {0.0f};
-            chunk_dot<P, 1, true>(cur, slice(t, j, v & 1).eb, tab, xg + t * (Lg * XP) + ch * XP, 0, 1, acc);
+            chunk_dot<P, 1, true>(cur, slice_gu(t, j).eb, tab, xg + t * (Lg * XP) + ch * XP, 0, 1, acc);
             float s = acc[0];
             for (int o = Lg >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
             const float other = __shfl_xor(s, Lg);
             // (results leave after the loop: a store here would sit in front of the wait for the next task's records)
-            if (ch == 0 && !(v & 1)) avs[t * nav + (i << c.lgV) + (lr >> 1)] = bfr(silu_bf(bfr(s * NSLM_R32)) * bfr(other * NSLM_R32));
+            // (the two row sums; SwiGLU is left to the wave that stores the CU's values: one wave's instructions instead of every task's)
+            if (ch == 0 && !wsel) *(float2*) &avs[2 * (t * nav + (i << c.lgV) + (lr >> 1))] = make_float2(s, other);
             ++mine;
             if (tn != t) {   // The wave's last task of token t: it adds its tasks to the CU's count.  The wave that completes the
                              // count stores the CU's values of the token (as BF16 for the other CUs, as f32 for the caller), and once
@@ -325,7 +331,8 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                     for (int u = lane; u < (n_loc << c.lgV); u += 64) {
                         const int qq = q_lo + (u >> c.lgV), jj = (int) ((uint32_t) qq / c.by_tpp);
                         const size_t at = (size_t) (t * kk + jj) * a.ff + (size_t) (((qq - jj * c.tpp) << c.lgV) + (u & (c.vpt - 1)));
-                        const float av = avs[t * nav + u];
+                        const float2 gu = *(const float2*) &avs[2 * (t * nav + u)];
+                        const float av = bfr(silu_bf(bfr(gu.x * NSLM_R32)) * bfr(gu.y * NSLM_R32));
                         st_agent(xa16 + at, (uint16_t) (__float_as_uint(av) >> 16));
                         a.A[at] = av;
                     }
@@ -387,13 +394,13 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         }
         __syncthreads();
         // all pairs' A of the token, 16 bytes (a block of 8 values) a thread, staged as the down matvec reads it
+        // (block b of the token = block b % nbp of pair b / nbp: a pair's row is whole chunks, so the token's pairs lie in xd as one row)
         for (int b = tid; b < kk * c.nbp; b += NTHR) {
-            const int j = (int) ((uint32_t) b / c.by_nbp), bb = b - j * c.nbp;
-            const unsigned long long* src = (const unsigned long long*) (xa16 + ((size_t) t * kk + j) * a.ff + (size_t) bb * 8);
+            const unsigned long long* src = (const unsigned long long*) (xa16 + (size_t) t * kk * a.ff + (size_t) b * 8);
             const unsigned long long lo = ld_agent(src), hi = ld_agent(src + 1);
             const float v[8] = {bf((uint32_t) lo & 0xFFFFu), bf((uint32_t) (lo >> 16) & 0xFFFFu), bf((uint32_t) (lo >> 32) & 0xFFFFu), bf((uint32_t) (lo >> 48)),
                                 bf((uint32_t) hi & 0xFFFFu), bf((uint32_t) (hi >> 16) & 0xFFFFu), bf((uint32_t) (hi >> 32) & 0xFFFFu), bf((uint32_t) (hi >> 48))};
-            store_block<P>(xd + j * (Ld * XP), bb, v);
+            store_block<P>(xd, b, v);
         }
         __syncthreads();
         for (int it = 0; it < c.nit; ++it) {
@@ -533,7 +540,7 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     c.rw = take(a.T * 36);
     c.rn = take(MV_MAXT + 16);
     c.cnt = take(2 * MV_MAXT);
-    c.av = take(a.T * c.n_c * c.vpt);
+    c.av = take(2 * a.T * c.n_c * c.vpt);
     c.lgs = take(16);
     c.sel = take((3 + (a.E <= CU_PRE_MAXE ? 0 : a.T * a.kk * 3)) * ws);
     c.pre = take(a.E <= CU_PRE_MAXE ? 3 * a.E * ws : 0);
