@@ -28,7 +28,7 @@ using namespace nslm;
 
 namespace {
 
-#define CU_LDS_MAX (160 * 1024)
+#define CU_LDS_MAX (160 * 1024 - NSLM_TAB_WORDS * 4)   // dynamic LDS: what the kernel's own table leaves of a CU's 160 KB
 #define CU_LDS_MIN (82 * 1024)   // more than half a CU's LDS: two of these workgroups never share a CU
 #define CU_LG 4                  // router logits a CU forms
 #define CU_PRE_MAXE 256          // experts whose slice tables are copied to LDS while the logits are on their way
@@ -471,9 +471,16 @@ int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds
     static size_t lds_set = 0;   // the largest dynamic-LDS request this kernel has been prepared for
     static int resident = 0;
     if (lds > lds_set) {
-        if (hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return -1;
+        // (a refusal is this launcher's answer "not my shape", not an error of the step: the runtime's error state is cleared)
+        if (hipFuncSetAttribute((const void*) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) {
+            (void) hipGetLastError();
+            return -1;
+        }
         int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, NTHR, lds) != hipSuccess || per_cu < 1) return -1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, NTHR, lds) != hipSuccess || per_cu < 1) {
+            (void) hipGetLastError();
+            return -1;
+        }
         resident = per_cu;
         lds_set = lds;
     }

@@ -333,6 +333,41 @@ def test_steps_of_changing_size_share_the_barrier_words():
     st.close()
 
 
+@pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
+def test_both_step_kernels_give_the_separate_launches_bits(fmt):
+    """The library's two persistent step kernels (a workgroup per CU; a workgroup per (pair, row tile)), each forced in turn at 1
+    to 6 rows, against the separate launches: the same bits three ways, and no wait gives up."""
+    from nanoseedlm_amd import backend, moe
+    L = backend.hip()
+    rng = np.random.default_rng(600 + fmt)
+    E, k, d, ff = 32, 4, 512, 256
+    mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
+    st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=8)
+    st.set_layer(0, mk(rng, E, ff, d, eb=-21), mk(rng, E, ff, d, eb=-21), mk(rng, E, d, ff, eb=-20),
+                 packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
+    st.finalize()
+    try:
+        for T in range(1, 7):
+            dx = moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32)))
+            outs = {}
+            for which in (0, 1, 2):   # 0: the separate launches
+                st.set_fused(1 if which else 0)
+                L.kc_moe_decode_kernel(which)
+                before = st.fused_steps()
+                dio = moe.DevBuf.from_array(np.zeros((T, d), dtype=np.float32))
+                st.step(None, 0, dx.ptr, T, dio.ptr)
+                outs[which] = dio.to_array(np.float32, (T, d))
+                dio.free()
+                assert st.fused_error() == 0 and st.fused_steps() == before + (1 if which else 0), (T, which)
+            dx.free()
+            assert np.abs(outs[0]).max() > 0
+            for which in (1, 2):
+                assert np.array_equal(outs[which].view(np.uint32), outs[0].view(np.uint32)), (T, which)
+    finally:
+        L.kc_moe_decode_kernel(0)
+        st.close()
+
+
 def test_small_shape_then_long_rows_in_one_process():
     """The per-item step kernel's launcher keeps the number of workgroups a CU holds per kernel variant; the LDS a workgroup
     asks for grows with the longer of hidden and expert width (8192: 51,200 bytes, above the 48 KB a kernel may have without
