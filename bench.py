@@ -48,7 +48,8 @@ def counters_of(workload):
         e = {}
     return dict(traffic=e.get("hbm_bytes_per_launch"), traffic_source=COUNTERS if e.get("hbm_bytes_per_launch") else None,
                 valu_busy=e.get("valu_busy_pct") / 100.0 if e.get("valu_busy_pct") is not None else None,
-                valu_busy_source=COUNTERS if e.get("valu_busy_pct") is not None else None)
+                valu_busy_source=COUNTERS if e.get("valu_busy_pct") is not None else None,
+                valu_insts_per_block=e.get("valu_insts_per_block"))
 
 
 def fail_on_kernel_error(st=None):
