@@ -35,6 +35,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
 COUNTERS = "profiles/traffic.json"
+# Untimed steps before the W warmup steps: a fresh GPU reaches its steady clocks only after a few hundred milliseconds of work
+# (the same 400 timed steps: 23.8 us a step after 50 warmup steps, 22.9 after 4000), and a short run would measure the ramp.
+PREWARM_S = 0.3
 
 
 def counters_of(workload):
@@ -173,15 +176,31 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
             if q4:
                 q4.run(stream, l, xs[xi].ptr)
 
-    for i in range(warmup):
-        run(i)
+    # A step that is one launch is issued from the C host's own loop (nslm_moe_step_seq): with an interpreter between launches of
+    # ~23 us the timed region measured the interpreter, not the kernel.
+    seq = graphs is None and q4 is None
+
+    def run_many(first, n, before=None, after=None):
+        if seq:   # (the events recorded by the same call, directly around the steps)
+            idx = [combos[(first + i) % len(combos)] for i in range(n)]
+            st.step_seq(stream, [l for l, _ in idx], [xs[xi].ptr for _, xi in idx], T, out.ptr, before, after)
+        else:
+            if before:
+                before.record(stream)
+            for i in range(n):
+                run(first + i)
+            if after:
+                after.record(stream)
+
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < PREWARM_S:
+        run_many(0, 256)
+        moe.device_sync()
+    run_many(0, warmup)
     moe.device_sync()
     e0, e1 = moe.Event(), moe.Event()
     t0 = time.perf_counter()
-    e0.record(stream)
-    for i in range(steps):
-        run(warmup + i)
-    e1.record(stream)
+    run_many(warmup, steps, e0, e1)
     e1.sync()
     moe.device_sync()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -389,6 +408,11 @@ def dense_workload(name, steps, warmup, matrices=64):
         bytes_step, flops = R * K * 36 / 64.0, 2.0 * T * R * K
         desc, bound = "C1 seeded prefill GEMM: W 14336x4096 P=4, X bf16 [512 x 4096], bf16 MFMA, fp32 accumulate", "mfma"
         sample = dict(shapes=[(R, K)], reps=1, fmt=packs.MF_SEED4P4)
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < PREWARM_S:
+        for i in range(256):
+            run(i)
+        moe.device_sync()
     for i in range(warmup):
         run(i)
     moe.device_sync()
@@ -526,6 +550,7 @@ def main():
         "tokens_per_s": r["tokens"] / r["ms_per_step"] * 1e3, "bytes_per_step": r["bytes_per_step"],
         "tflops": r["flops_per_step"] / r["ms_per_step"] / 1e9, "host_ms_per_step": r["wall_ms_per_step"],
         "roofline": r["roofline"],
+        "prewarm_s": 0.0 if a.workload[:2] == "c4" else PREWARM_S,   # untimed steps of the same workload before the W warmup steps
     }
     line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(r["cpu_sample"])
     if a.calibrate_copy > 0:

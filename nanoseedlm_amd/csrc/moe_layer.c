@@ -404,6 +404,14 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
 
 void nslm_moe_set_fused(NslmMoe* m, int on) { m->fused = on; }
 int nslm_moe_fused_mode(const NslmMoe* m) { return m->fused; }
+int nslm_moe_step_seq(NslmMoe* m, kc_stream_t s, int n, const int* layers, const float* const* xn, int T, float* io, void* before,
+                      void* after) {
+    if (before && nh_event_record((nh_event_t) before, (nh_stream_t) s)) return -1;
+    for (int i = 0; i < n; ++i)
+        if (nslm_moe_step(m, s, layers[i], xn[i], T, io)) return -1;
+    if (after && nh_event_record((nh_event_t) after, (nh_stream_t) s)) return -1;
+    return 0;
+}
 int nslm_moe_fallbacks(const NslmMoe* m) { return m->fallbacks; }
 long nslm_moe_fused_steps(const NslmMoe* m) { return m->fused_steps; }
 void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }

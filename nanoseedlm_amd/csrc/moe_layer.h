@@ -50,6 +50,11 @@ int nslm_moe_fill_random(NslmMoe* m, uint64_t seed, int eb, float router_scale);
  * xn: the layer input [T][d] (device).  io [T][d] (device): softmax composition: receives sum_k wt_k y_k;
  * sigmoid composition: the residual stream, updated in place x = bf16(x + bf16(bf16(sum) + 0)). */
 int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, float* io);
+/* n steps one after the other on s from one call (step i: layer layers[i], input xn[i], all into io): what a C host's decode
+ * loop issues, without a caller's interpreter between the launches.  before / after (nh_event_t, or NULL): events recorded on s
+ * directly before the first and after the last step, for a caller that times the steps.  Stops at the first step that fails (-1). */
+int nslm_moe_step_seq(NslmMoe* m, kc_stream_t s, int n, const int* layers, const float* const* xn, int T, float* io, void* before,
+                      void* after);
 /* routed experts + a shared expert (3 host slices: gate, up, down of the routed experts' shape) + residual in the one persistent launch:
  * out = bf16(res + bf16(sum_j wt_j y_j + y_shared)).  0 done, 1 not available (nothing launched), -1 error. */
 int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out,

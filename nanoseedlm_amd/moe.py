@@ -117,6 +117,15 @@ class MoeStack:
         if self.L.nslm_moe_step(self.h, stream, layer, xn_ptr, T, io_ptr):
             raise RuntimeError("nslm_moe_step failed")
 
+    def step_seq(self, stream, layers, xn_ptrs, T, io_ptr, before=None, after=None):
+        """The steps (layers[i], xn_ptrs[i]) issued one after the other by one call into the C host (no interpreter between the
+        launches); before / after: Events recorded on the stream directly around them."""
+        n = len(layers)
+        la = (C.c_int * n)(*layers)
+        xa = (C.c_void_p * n)(*[p.value if isinstance(p, C.c_void_p) else p for p in xn_ptrs])
+        if self.L.nslm_moe_step_seq(self.h, stream, n, la, xa, T, io_ptr, before.e if before else None, after.e if after else None):
+            raise RuntimeError("nslm_moe_step_seq failed")
+
     def last_routing(self, T):
         ind = np.zeros((T, self.cfg.top_k), dtype=np.int32)
         wt = np.zeros((T, self.cfg.top_k), dtype=np.float32)
