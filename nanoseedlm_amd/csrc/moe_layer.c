@@ -412,6 +412,14 @@ int nslm_moe_step_seq(NslmMoe* m, kc_stream_t s, int n, const int* layers, const
     if (after && nh_event_record((nh_event_t) after, (nh_stream_t) s)) return -1;
     return 0;
 }
+int nslm_mv_seq(kc_stream_t s, int fmt, const WSlice* ws, int nw, int first, int n, int K, int R, const float* x, float* y, void* before,
+                void* after) {
+    if (nw < 1 || first < 0) return -1;
+    if (before && nh_event_record((nh_event_t) before, (nh_stream_t) s)) return -1;
+    for (int i = 0; i < n; ++i) kc_mv(s, fmt, ws[(first + i) % nw], K, R, x, K, y, R, 1, 0, NULL);
+    if (after && nh_event_record((nh_event_t) after, (nh_stream_t) s)) return -1;
+    return kc_last_error() ? -1 : 0;
+}
 int nslm_moe_fallbacks(const NslmMoe* m) { return m->fallbacks; }
 long nslm_moe_fused_steps(const NslmMoe* m) { return m->fused_steps; }
 void* nslm_moe_sync_ptr(NslmMoe* m) { return m->sync; }

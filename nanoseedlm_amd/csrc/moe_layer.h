@@ -55,6 +55,9 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
  * directly before the first and after the last step, for a caller that times the steps.  Stops at the first step that fails (-1). */
 int nslm_moe_step_seq(NslmMoe* m, kc_stream_t s, int n, const int* layers, const float* const* xn, int T, float* io, void* before,
                       void* after);
+/* The same for the dense one-row matvec: n launches of kc_mv(fmt, ws[(first + i) % nw], K, R, x -> y) on s, with the events around them. */
+int nslm_mv_seq(kc_stream_t s, int fmt, const WSlice* ws, int nw, int first, int n, int K, int R, const float* x, float* y, void* before,
+                void* after);
 /* routed experts + a shared expert (3 host slices: gate, up, down of the routed experts' shape) + residual in the one persistent launch:
  * out = bf16(res + bf16(sum_j wt_j y_j + y_shared)).  0 done, 1 not available (nothing launched), -1 error. */
 int nslm_moe_step_layer(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, const WSlice* shared, const float* res, float* out,
