@@ -309,7 +309,7 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
 /* kc_moe_decode without a workspace argument.  No counterpart in the reference: it is for callers that cannot allocate device
  * memory or carry a workspace around - code under stream capture, tight serving loops, harnesses that forbid hipMalloc.  What
  * kc_moe_decode's caller owns as scratch (logits, A, D, the sync words) lives in one array inside the library's code object
- * (4.9 MB of device memory on every GPU the library runs on, held until the process ends); the call allocates and frees nothing.
+ * (5.3 MB of device memory on every GPU the library runs on, held until the process ends); the call allocates and frees nothing.
  * ind / wt [T][top_k] (the routing) and out stay the caller's.  Results: kc_moe_decode's, bit for bit.
  * status (device, 4 bytes) or NULL: receives the error word after the step (non-zero: a wait between workgroups gave up, the
  * results are void) - one more one-thread launch.  clear != 0: the sync words are zeroed first (a fill kernel on s); needed
