@@ -937,7 +937,9 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
     // 2: 37.6 / 39.2, 3: 49.3 / 51.4, 4: 61.9 / 62.0, 5: 74.8 / 74.1, 6: 87 - 91 / 89.5 - 90.5; with the staged inputs and the
     // staged A in one LDS area 7 and 8 tokens fit too: 104 / 96 and 117 / 104); with an always-on expert up to three (the whole
     // model's step at 4 rows: 3.29 against 3.25 ms)
-    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (shared ? 3 : 4))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
+    // (rows whose chunks do not fill a wave, where that kernel's gate + up pass goes by iterations of the workgroup - C3's rows of 45
+    // chunks, us: 1 token 59.4 / 68.0, 2: 108.0 / 109.8, 3: 157.1 / 156.9, 4: 206.0 / 197.4 - up to two)
+    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (shared ? 3 : sg ? 4 : 2))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);

@@ -20,8 +20,11 @@
 //     when its down pass needs it, so only a one-token launch waits for the exchange.
 //   - Every instruction outside the row loops counts (a CU's waves all execute it at the same moment): what can be computed
 //     on the host arrives in the arguments, and no index is formed by an integer division.
-// Shapes: hidden width d = 64 * 2^n <= 2048 (a row's chunks fit a wave and the row sums are shuffles), T * pairs * ff <=
-// FUSED_XA_MAX, the workgroup's LDS <= 160 KB.  Other shapes stay with the kernel of nslm_fused.hip.
+//   - Rows whose chunks do not fit a wave as a power of two (45 chunks, say) take the gate + up pass by iterations of the whole
+//     workgroup instead - a thread a chunk of a virtual row, the row sums through LDS in chunk order, one barrier an
+//     iteration - with 22 of 22.7 possible rows an iteration where a 256-thread workgroup fills 4 of 5.7.
+// Shapes: a row of at most 256 chunks, T * pairs * ff <= FUSED_XA_MAX, the workgroup's LDS <= 160 KB less the table.  Other
+// shapes stay with the kernel of nslm_fused.hip.
 #include "nslm_fused_dev.h"
 
 using namespace nslm;
@@ -61,15 +64,16 @@ struct CuParams {
     int lgL;              // log2 of the chunks in a gate / up row (Lg)
     int rpw, tpp, Wt;     // gate + up: virtual rows a wave-task, tasks a pair, tasks a token
     int n_c, ncu_act;     // tasks a CU and token; CUs that have tasks
+    int rpi_g, nit_g;     // gate + up where a row's chunks do not fit a wave: virtual rows an iteration of the workgroup, iterations a token
     int rpc;              // down: output rows a CU owns
     int rpi, rows_t, nit; // down: (pair, row)s an iteration of the workgroup, (pair, row)s a token and CU, iterations a token
     int nbp;              // blocks of 8 in a row of A
     int vpt, lgV;         // SwiGLU outputs a task (rpw / 2) and its log2
     int E4, KP;           // E padded to 4; keys a token (E padded to 16)
-    FastDiv by_tpp, by_rpc, by_Ld, by_nbp, by_kk, by_E;
+    FastDiv by_tpp, by_rpc, by_Ld, by_Lg, by_nbp, by_kk, by_E;
 };
 
-template <int P, bool SHFL_D, int NTHR>
+template <int P, bool SHFL_G, bool SHFL_D, int NTHR>
 __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c) {
     constexpr int NW = NTHR / 64, XP = xpad<P>();
     extern __shared__ __attribute__((aligned(16))) float dyn[];
@@ -277,7 +281,34 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         if (preload) return lane_pre[__builtin_amdgcn_readfirstlane(ri_s[t * 32 + j])];
         return sel[3 + (t * kk + j) * 3 + wsel];
     };
-    {
+    const int nav = c.n_c << c.lgV;   // SwiGLU outputs a CU and token at most
+    // One wave stores the CU's values of a token - SwiGLU of the two row sums, as BF16 for the other CUs and as f32 for the caller -
+    // and, once the stores are acknowledged, arrives for the CU; the last CU of all raises the token's ready words.
+    auto publish = [&](int t) {
+        for (int u = lane; u < (n_loc << c.lgV); u += 64) {
+            const int qq = q_lo + (u >> c.lgV), jj = (int) ((uint32_t) qq / c.by_tpp);
+            const size_t at = (size_t) (t * kk + jj) * a.ff + (size_t) (((qq - jj * c.tpp) << c.lgV) + (u & (c.vpt - 1)));
+            const float2 gu = *(const float2*) &avs[2 * (t * nav + u)];
+            const float av = bfr(silu_bf(bfr(gu.x * NSLM_R32)) * bfr(gu.y * NSLM_R32));
+            st_agent(xa16 + at, (uint16_t) (__float_as_uint(av) >> 16));
+            a.A[at] = av;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (lane == 0) {
+            uint32_t* bar = a.sync + FUSED_CU_WORDS + t * FUSED_CU_TOKEN_WORDS;   // [32 group lines][root line][32 ready lines]
+            const uint32_t g = blockIdx.x % BAR_GROUPS, ncu = (uint32_t) c.ncu_act, ng = ncu < BAR_GROUPS ? ncu : BAR_GROUPS;
+            const uint32_t in_group = (ncu - g + BAR_GROUPS - 1) / BAR_GROUPS;
+            if (atomicAdd(bar + 32 * g, 1u) == in_group - 1) {
+                st_agent(bar + 32 * g, 0u);
+                if (atomicAdd(bar + 32 * BAR_GROUPS, 1u) == ng - 1) {
+                    st_agent(bar + 32 * BAR_GROUPS, 0u);
+#pragma unroll
+                    for (uint32_t r = 0; r < BAR_GROUPS; ++r) st_agent(bar + 32 * (BAR_GROUPS + 1 + r), tag);
+                }
+            }
+        }
+    };
+    if constexpr (SHFL_G) {
         // The CU's tasks of a token go to whichever wave asks next: a wave whose records arrive late, or that shares its SIMD
         // with more waves, takes fewer.  A wave asks for its next task before it computes the current one, so that task's
         // records travel meanwhile.  Task = (token, index in the CU's run); token T = none left.
@@ -304,7 +335,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         claim(t, i);
         Chunk cur = fetch(t, i);
         uint32_t mine = 0;   // tasks of the token in hand this wave has finished
-        const int nav = c.n_c << c.lgV;   // SwiGLU outputs a CU and token at most
         while (t < T) {
             int tn, inx;
             claim(tn, inx);
@@ -327,35 +357,62 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 if (lane == 0) before = atomicAdd(&cnt_s[MV_MAXT + t], mine);
                 before = __builtin_amdgcn_readfirstlane(before);
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                if (before + mine == (uint32_t) n_loc) {
-                    for (int u = lane; u < (n_loc << c.lgV); u += 64) {
-                        const int qq = q_lo + (u >> c.lgV), jj = (int) ((uint32_t) qq / c.by_tpp);
-                        const size_t at = (size_t) (t * kk + jj) * a.ff + (size_t) (((qq - jj * c.tpp) << c.lgV) + (u & (c.vpt - 1)));
-                        const float2 gu = *(const float2*) &avs[2 * (t * nav + u)];
-                        const float av = bfr(silu_bf(bfr(gu.x * NSLM_R32)) * bfr(gu.y * NSLM_R32));
-                        st_agent(xa16 + at, (uint16_t) (__float_as_uint(av) >> 16));
-                        a.A[at] = av;
-                    }
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                    if (lane == 0) {
-                        uint32_t* bar = a.sync + FUSED_CU_WORDS + t * FUSED_CU_TOKEN_WORDS;   // [32 group lines][root line][32 ready lines]
-                        const uint32_t g = blockIdx.x % BAR_GROUPS, ncu = (uint32_t) c.ncu_act, ng = ncu < BAR_GROUPS ? ncu : BAR_GROUPS;
-                        const uint32_t in_group = (ncu - g + BAR_GROUPS - 1) / BAR_GROUPS;
-                        if (atomicAdd(bar + 32 * g, 1u) == in_group - 1) {
-                            st_agent(bar + 32 * g, 0u);
-                            if (atomicAdd(bar + 32 * BAR_GROUPS, 1u) == ng - 1) {
-                                st_agent(bar + 32 * BAR_GROUPS, 0u);
-#pragma unroll
-                                for (uint32_t r = 0; r < BAR_GROUPS; ++r) st_agent(bar + 32 * (BAR_GROUPS + 1 + r), tag);
-                            }
-                        }
-                    }
-                }
+                if (before + mine == (uint32_t) n_loc) publish(t);
                 mine = 0;
             }
             cur = nxt;
             t = tn;
             i = inx;
+        }
+    }
+    else if (n_loc > 0) {
+        // Rows whose chunks do not fit a wave (a row of 45 chunks, say): the pass goes by iterations of the whole workgroup, a thread
+        // a chunk of a virtual row (2r = gate row r, 2r + 1 = up row r of the CU's run of SwiGLU rows, a "task" being one such
+        // row), the row sums through LDS in chunk order (the separate launches' order), one workgroup barrier an iteration
+        // (the partial sums are double-buffered by iteration parity).
+        const int gl = (int) ((uint32_t) tid / c.by_Lg), gch = tid - gl * Lg;
+        const bool gact = gl < c.rpi_g;
+        float* const partg = (float*) scr;   // [2][NTHR]
+        auto fetch_g = [&](int t, int it) {   // (unconditional: rows past the CU's last are clamped)
+            const int v = min(it * c.rpi_g + gl, 2 * n_loc - 1), q = q_lo + (v >> 1), j = (int) ((uint32_t) q / c.by_tpp);
+            return load_chunk<P>(slice(min(t, T - 1), j, v & 1), (uint32_t) (q - j * c.tpp) * (uint32_t) Lg + (uint32_t) gch);
+        };
+        Chunk cur = fetch_g(0, 0);
+        int par = 0;
+        for (int t = 0; t < T; ++t) {
+            for (int it = 0; it < c.nit_g; ++it, par ^= 1) {
+                const bool last = it + 1 == c.nit_g;
+                const Chunk nxt = fetch_g(last ? t + 1 : t, last ? 0 : it + 1);
+                const int v = it * c.rpi_g + gl, vc = min(v, 2 * n_loc - 1), q = q_lo + (vc >> 1), j = (int) ((uint32_t) q / c.by_tpp);
+                float acc[1] = {0.0f};
+                if (gact && v < 2 * n_loc) chunk_dot<P, 1, true>(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + gch * XP, 0, 1, acc);
+                partg[par * NTHR + tid] = acc[0];
+                __syncthreads();
+                const int nrow = min(c.rpi_g, 2 * n_loc - it * c.rpi_g);
+                if (tid < nrow / 2) {
+                    // the two rows' partial sums in chunk order; eight are read before the first is added (a chunk past the row's
+                    // last counts +0, which leaves the sum's bits alone)
+                    const float* pg = partg + par * NTHR + (2 * tid) * Lg;
+                    float gs = 0.0f, us = 0.0f;
+                    for (int c0 = 0; c0 < Lg; c0 += 8) {
+                        float pv[8], pu[8];
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) {
+                            pv[cc] = pg[min(c0 + cc, Lg - 1)];
+                            pu[cc] = pg[Lg + min(c0 + cc, Lg - 1)];
+                        }
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) {
+                            gs += c0 + cc < Lg ? pv[cc] : 0.0f;
+                            us += c0 + cc < Lg ? pu[cc] : 0.0f;
+                        }
+                    }
+                    *(float2*) &avs[2 * (t * nav + it * (c.rpi_g >> 1) + tid)] = make_float2(gs, us);
+                }
+                cur = nxt;
+            }
+            __syncthreads();   // the token's row sums are all in LDS
+            if (wv == NW - 1) publish(t);
         }
     }
     // Housekeeping, off the critical path: the lines of this kernel's logits table that this launch did not write, and the
@@ -465,9 +522,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     }
 }
 
-template <int P, bool SD, int NTHR>
+template <int P, bool SG, bool SD, int NTHR>
 int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds) {
-    void (*kern)(FusedArgs, CuParams) = k_moe_decode_cu<P, SD, NTHR>;
+    void (*kern)(FusedArgs, CuParams) = k_moe_decode_cu<P, SG, SD, NTHR>;
     static size_t lds_set = 0;   // the largest dynamic-LDS request this kernel has been prepared for
     static int resident = 0;
     if (lds > lds_set) {
@@ -503,16 +560,25 @@ namespace nslm {
 // 0 launched; -1 the shape is not this kernel's (nothing launched)
 int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     if (a.T < 1 || a.T > MV_MAXT) return -1;
-    if (a.Lg > 32 || (a.Lg & (a.Lg - 1))) return -1;                       // a row's chunks: a power of two inside a wave
+    const bool sg = a.Lg <= 32 && !(a.Lg & (a.Lg - 1));   // a gate / up row's chunks are a power of two inside a wave: row sums by shuffles
+    if (a.Lg > 256) return -1;
     if ((long) a.T * a.kk * a.ff > FUSED_XA_MAX || a.ff % 64 || a.kk > 33) return -1;
     const int G = fused_cu_count();
     if (G < 1 || a.E > 1024 || (long) a.T * a.E > (long) CU_LG * (G < FUSED_CULG_LINES ? G : FUSED_CULG_LINES)) return -1;   // (a CU forms CU_LG logits)
     a.grid = G;
     CuParams c = {};
     c.G = G;
-    c.lgL = log2_of(a.Lg);
-    c.rpw = 64 / a.Lg;
-    c.tpp = 2 * a.ff / c.rpw;
+    const int nthr = 1024;
+    if (sg) {
+        c.lgL = log2_of(a.Lg);
+        c.rpw = 64 / a.Lg;
+        c.tpp = 2 * a.ff / c.rpw;
+    } else {   // a task is one SwiGLU row (two virtual rows), dealt to the workgroup's threads by iterations
+        c.lgL = 0;
+        c.rpw = 2;
+        c.tpp = a.ff;
+        c.rpi_g = (nthr / a.Lg) & ~1;
+    }
     c.Wt = a.kk * c.tpp;
     c.n_c = (c.Wt + G - 1) / G;
     c.ncu_act = (c.Wt + c.n_c - 1) / c.n_c;
@@ -522,12 +588,13 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     c.E4 = (a.E + 3) & ~3;
     // 16 waves: four a SIMD get through a block's dependent instruction chains faster than three (C2, one token: 22.6 against
     // 23.3 us with 12 waves, whose tasks divide evenly among them; 4 tokens 62.5 against 64.2)
-    const int nthr = 1024;
     c.rpi = nthr / a.Ld;
     c.nit = (c.rows_t + c.rpi - 1) / c.rpi;
     c.KP = (a.E + 15) & ~15;
     c.vpt = c.rpw / 2;
     c.lgV = log2_of(c.vpt);
+    c.nit_g = sg ? 0 : (2 * c.n_c + c.rpi_g - 1) / c.rpi_g;
+    c.by_Lg = fastdiv_of((uint32_t) a.Lg);
     c.by_E = fastdiv_of((uint32_t) a.E);
     c.by_tpp = fastdiv_of((uint32_t) c.tpp);
     c.by_rpc = fastdiv_of((uint32_t) c.rpc);
@@ -539,7 +606,7 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     auto take = [&](int words) { const int at = o; o += (words + 3) & ~3; return at; };
     c.xg = take(a.T * a.Lg * xp);
     c.xd = take(a.kk * a.Ld * xp);
-    c.scr = take(nthr);
+    c.scr = take(2 * nthr);
     c.pk = take(a.T * c.KP);
     c.rv = take(a.T * c.E4);
     c.dsum = take(a.kk * c.rpc);
@@ -555,8 +622,12 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     size_t lds = (size_t) c.total * 4;
     if (lds > CU_LDS_MAX) return -1;
     if (lds < CU_LDS_MIN) lds = CU_LDS_MIN;
-    if (P == 4) return sd ? launch_one<4, true, 1024>(st, a, c, lds) : launch_one<4, false, 1024>(st, a, c, lds);
-    return sd ? launch_one<3, true, 1024>(st, a, c, lds) : launch_one<3, false, 1024>(st, a, c, lds);
+    if (P == 4) {
+        if (sg) return sd ? launch_one<4, true, true, 1024>(st, a, c, lds) : launch_one<4, true, false, 1024>(st, a, c, lds);
+        return sd ? launch_one<4, false, true, 1024>(st, a, c, lds) : launch_one<4, false, false, 1024>(st, a, c, lds);
+    }
+    if (sg) return sd ? launch_one<3, true, true, 1024>(st, a, c, lds) : launch_one<3, true, false, 1024>(st, a, c, lds);
+    return sd ? launch_one<3, false, true, 1024>(st, a, c, lds) : launch_one<3, false, false, 1024>(st, a, c, lds);
 }
 
 }   // namespace nslm
