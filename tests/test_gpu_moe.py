@@ -368,6 +368,50 @@ def test_both_step_kernels_give_the_separate_launches_bits(fmt):
         st.close()
 
 
+def test_steps_issued_by_one_call_equal_single_steps():
+    """nslm_moe_step_seq (n steps and the two timing events from one call into the C host) leaves what the same steps leave when
+    issued one by one, and its events bracket them; nslm_mv_seq does the same for the dense matvec."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    rng = np.random.default_rng(99)
+    st = _small_stack(rng)
+    d, T = 512, 2
+    xs = [moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))) for _ in range(3)]
+    out = moe.DevBuf(4 * T * d)
+    stream = moe.new_stream()
+    layers, xi = [0, 1, 1, 0, 1], [0, 1, 2, 2, 0]
+    for l, x in zip(layers, xi):
+        st.step(stream, l, xs[x].ptr, T, out.ptr)
+    moe.device_sync()
+    want = out.to_array(np.float32, (T, d)).copy()
+    backend.check(backend.hip().nh_memset(out.ptr, 0, C.c_size_t(out.nbytes)), "nh_memset")
+    e0, e1 = moe.Event(), moe.Event()
+    st.step_seq(stream, layers, [xs[x].ptr for x in xi], T, out.ptr, e0, e1)
+    e1.sync()
+    got = out.to_array(np.float32, (T, d))
+    assert st.fused_error() == 0 and np.abs(want).max() > 0
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert 0.0 < e1.ms_since(e0) < 50.0
+    # the dense matvec over two slices, the last launch's result
+    R = K = 256
+    p = packs.seed4p4(rng, 2, R, K, eb=-20)
+    ds, dc, de = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
+    sl = (backend.WSlice * 2)()
+    for i in range(2):
+        sl[i].p[0], sl[i].p[1], sl[i].p[3] = ds.ptr.value + i * R * K // 4, dc.ptr.value + i * R * K // 4, de.ptr.value + i * R * K // 16
+        sl[i].eb = -20
+    x = moe.DevBuf.from_array(rng.standard_normal(K).astype(np.float32))
+    y0, y1 = moe.DevBuf(4 * R), moe.DevBuf(4 * R)
+    backend.hip().kc_mv(stream, packs.MF_SEED4P4, sl[1], K, R, x.ptr, K, y0.ptr, R, 1, 0, None)
+    backend.check(backend.host().nslm_mv_seq(stream, packs.MF_SEED4P4, sl, 2, 0, 4, K, R, x.ptr, y1.ptr, None, None), "nslm_mv_seq")
+    moe.device_sync()
+    a, b = y0.to_array(np.float32, (R,)), y1.to_array(np.float32, (R,))
+    assert np.abs(a).max() > 0 and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    for buf in xs + [out, ds, dc, de, x, y0, y1]:
+        buf.free()
+    st.close()
+
+
 def test_small_shape_then_long_rows_in_one_process():
     """The per-item step kernel's launcher keeps the number of workgroups a CU holds per kernel variant; the LDS a workgroup
     asks for grows with the longer of hidden and expert width (8192: 51,200 bytes, above the 48 KB a kernel may have without
