@@ -242,7 +242,7 @@ def test_fused_step_rows_that_do_not_fill_a_workgroup(d, ff, fmt):
     gate, up, down = mk(rng, E, ff, d, eb=-23), mk(rng, E, ff, d, eb=-23), mk(rng, E, d, ff, eb=-22)
     st.set_layer(0, gate, up, down, packs.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.05).astype(np.float32)))
     st.finalize()
-    for T in (1, 3, 8):
+    for T in (1, 2, 3, 8):
         xn = packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))
         dx = moe.DevBuf.from_array(xn)
         outs = []
@@ -334,13 +334,15 @@ def test_steps_of_changing_size_share_the_barrier_words():
 
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
-def test_both_step_kernels_give_the_separate_launches_bits(fmt):
+@pytest.mark.parametrize("E,k,d,ff", [(32, 4, 512, 256), (6, 2, 2880, 2816), (5, 3, 1088, 704)])
+def test_both_step_kernels_give_the_separate_launches_bits(fmt, E, k, d, ff):
     """The library's two persistent step kernels (a workgroup per CU; a workgroup per (pair, row tile)), each forced in turn at 1
-    to 6 rows, against the separate launches: the same bits three ways, and no wait gives up."""
+    to 6 rows, against the separate launches: the same bits three ways, and no wait gives up.  Rows of 8 chunks (row sums by
+    shuffles in the CU kernel's gate + up pass) and of 45 and 17 chunks (that pass by iterations of the workgroup, sums through LDS;
+    2816 = 44 chunks and 704 = 11 chunks in the down pass)."""
     from nanoseedlm_amd import backend, moe
     L = backend.hip()
-    rng = np.random.default_rng(600 + fmt)
-    E, k, d, ff = 32, 4, 512, 256
+    rng = np.random.default_rng(600 + fmt + d)
     mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
     st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=8)
     st.set_layer(0, mk(rng, E, ff, d, eb=-21), mk(rng, E, ff, d, eb=-21), mk(rng, E, d, ff, eb=-20),
