@@ -44,7 +44,7 @@ __device__ __forceinline__ Chunk first_chunk(const WSlice& wA, const WSlice& wB,
 // is called by the thread that owns a finished row sum.
 template <int P, bool GATEUP, bool SHFL, typename Emit>
 __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1,
-                                          const uint32_t* tab, const float* xl, float (*part)[256], Emit emit) {
+                                          const uint32_t* tab, const float* xl, float (*part)[256], float2* gu, Emit emit) {
     const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
     auto fetch = [&](int vv) {   // (rows past the last: the last row's records once more)
@@ -65,8 +65,13 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
             float s = acc[0];
             for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
             if (GATEUP) {
+                // (the two row sums wait in LDS: what emit does with them - SwiGLU, a store - is then executed once behind the loop
+                // by the threads of a row each, not in every iteration by every wave that holds a row)
                 const float other = __shfl_xor(s, L);
-                if (active && ch == 0 && !(v & 1) && v < v1) emit(v >> 1, s * NSLM_R32, other * NSLM_R32);
+                if (active && ch == 0 && !(v & 1) && v < v1) {
+                    if (gu) gu[(v - v0) >> 1] = make_float2(s, other);
+                    else emit(v >> 1, s * NSLM_R32, other * NSLM_R32);
+                }
             } else if (active && ch == 0 && v < v1) emit(v, s * NSLM_R32, 0.0f);
         } else {
             part[par][tid] = acc[0];
@@ -88,6 +93,13 @@ __device__ __forceinline__ void rows_pass(Chunk cur, const WSlice& wA, const WSl
         cur = nxt;
     }
     if (!SHFL) __syncthreads();   // part may be reused by the next pass
+    if (GATEUP && SHFL && gu) {
+        __syncthreads();
+        for (int i = tid; i < (v1 - v0) >> 1; i += 256) {
+            const float2 q = gu[i];
+            emit((v0 >> 1) + i, q.x * NSLM_R32, q.y * NSLM_R32);
+        }
+    }
 }
 
 // n floats of a row staged into LDS in the form the format's matvec reads (store_block: chunk-padded, P = 4 as its 12 column
@@ -189,6 +201,7 @@ __device__ __forceinline__ void rank_logits(const float* rv, int E, int k, uint3
 template <int P, bool SHFL_G, bool SHFL_D, int WAVES>
 __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // WAVES waves a SIMD: five = at most 96 registers
     extern __shared__ float xl[];   // activations of the current pair: max(d, ff) floats, chunk-padded
+    float2* const gu_s = (float2*) (xl + a.gu_off);   // behind them: the gate and up row sums of the item in hand
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     __shared__ float part[2][256];
     __shared__ __attribute__((aligned(16))) float rv[1024];   // route: the token's logits
@@ -312,7 +325,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
             __syncthreads();
         }
         float* Ap = a.A + (size_t) p * a.ff;
-        rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part,
+        rows_pass<P, true, SHFL_G>(c0, sl_s[0][j], sl_s[1][j], a.Lg, a.rpig, v0, v1, tab, xl, part, gu_s,
                                    [&](int r, float gs, float us) { st_agent(Ap + r, bfr(silu_bf(bfr(gs)) * bfr(us))); });
         wg_release();   // this item's rows of A are written: one more of the pair's gate+up items is done
         __syncthreads();
@@ -362,7 +375,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         staged = -1;
         __syncthreads();
         float* Dp = a.D + (size_t) p * a.d;
-        rows_pass<P, false, SHFL_D>(d0, sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1, tab, xl, part,
+        rows_pass<P, false, SHFL_D>(d0, sl_s[2][j], sl_s[2][j], a.Ld, a.rpid, v0, v1, tab, xl, part, nullptr,
                                     [&](int r, float s, float) { st_agent(Dp + r, bfr(s)); });
         wg_release();
         __syncthreads();
@@ -659,7 +672,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             st_agent(a.A + (size_t) gm[g * NT + m] * a.ff + r, bfr(silu_bf(bfr(gs)) * bfr(us)));
         };
         if (nt == 1)   // a group of one: the one-token loop, no second row of multiply-adds
-            rows_pass<P, true, SHFL_G>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, (float (*)[256]) part,
+            rows_pass<P, true, SHFL_G>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, (float (*)[256]) part, nullptr,
                                        [&](int r, float gs, float us) { put_a(0, r, gs, us); });
         else
             rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part, put_a);
@@ -695,7 +708,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
         __syncthreads();
         auto put_d = [&](int m, int r, float sm, float) { st_agent(a.D + (size_t) gm[g * NT + m] * a.d + r, bfr(sm)); };
         if (nt == 1)
-            rows_pass<P, false, SHFL_D>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, (float (*)[256]) part,
+            rows_pass<P, false, SHFL_D>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, (float (*)[256]) part, nullptr,
                                         [&](int r, float sm, float) { put_d(0, r, sm, 0.0f); });
         else
             rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part, put_d);
@@ -773,8 +786,18 @@ int pick_by_cu_load(int units, int iters, int cus, int nmax) {
     return best;
 }
 
+#define GU_ROWS 128   // SwiGLU rows of an item whose two sums wait in LDS for the end of the item's row loop (per-item kernel)
+// the fewest items a pair at which an item's rows fit that area
+int gu_min_tiles(const FusedArgs& a) {
+    int n = 1;
+    while (n < FUSED_TILES && (long) ((a.it_g + n - 1) / n) * a.rpig / 2 > GU_ROWS) ++n;
+    return n;
+}
+
 template <int P>
 int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
+    a.gu_off = (int) (lds / sizeof(float));
+    lds += GU_ROWS * sizeof(float2);
     // One token is at most a few hundred items more than three workgroups a CU hold (C2: 784): that launch may use the
     // registers of four waves a SIMD instead of five (107 instead of 96, no spills: 35.0 -> 34.5 us).  With the P = 4 column form the
     // same holds up to four tokens (C2, four / five waves, us: 2 tokens 41.4 / 45.8, 3: 55.6 / 56.3, 4: 66.4 / 69.8, 5: 85.9 / 80.3,
@@ -809,6 +832,8 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
     a.ntile_g = few || !sg ? pick_one_round(P_, a.it_g, gmax, FUSED_TILES) : pick_by_cu_load(P_, a.it_g, cu_count(), FUSED_TILES);
     a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES);
+    if (a.ntile_g < gu_min_tiles(a)) a.ntile_g = gu_min_tiles(a);
+    if ((long) ((a.it_g + a.ntile_g - 1) / a.ntile_g) * a.rpig / 2 > GU_ROWS) return -1;
     const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
     int grid = items < gmax ? (int) items : gmax;
     if (grid < 1) grid = 1;
@@ -826,6 +851,7 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
     const int lmax = a.Lg > a.Ld ? a.Lg : a.Ld;
     size_t lds = (size_t) NT * lmax * xpad<P>() * sizeof(float);
     if (lds < FG_PRE_BYTES) lds = FG_PRE_BYTES;
+
     static int cached[2][2] = {{0, 0}, {0, 0}};   // resident workgroups per CU, by kernel variant, for the largest request seen
     static size_t cached_lds[2][2] = {{0, 0}, {0, 0}};
     int& per_cu = cached[sg][sd];
@@ -933,13 +959,13 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
-    // one workgroup per CU: ahead up to four tokens (C2, us, a workgroup per CU / per item, records from HBM: 1 token 22.5 / 25.9,
-    // 2: 37.6 / 39.2, 3: 49.3 / 51.4, 4: 61.9 / 62.0, 5: 74.8 / 74.1, 6: 87 - 91 / 89.5 - 90.5; with the staged inputs and the
-    // staged A in one LDS area 7 and 8 tokens fit too: 104 / 96 and 117 / 104); with an always-on expert up to three (the whole
-    // model's step at 4 rows: 3.29 against 3.25 ms)
+    // one workgroup per CU: ahead up to three tokens (C2, us, a workgroup per CU / per item, records from HBM: 1 token 22.8 / 25.6,
+    // 2: 37.2 / 38.0, 3: 48.9 / 49.7, 4: 61.6 / 60.1, 5: 74.4 / 71.7; with the staged inputs and the staged A in one LDS area
+    // 7 and 8 tokens fit too: 104 / 96 and 117 / 104); with an always-on expert the same three (the whole model's step at 4
+    // rows: 3.29 against 3.25 ms)
     // (rows whose chunks do not fill a wave, where that kernel's gate + up pass goes by iterations of the workgroup - C3's rows of 45
     // chunks, us: 1 token 59.4 / 68.0, 2: 108.0 / 109.8, 3: 157.1 / 156.9, 4: 206.0 / 197.4 - up to two)
-    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (shared ? 3 : sg ? 4 : 2))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
+    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (sg ? 3 : 2))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);

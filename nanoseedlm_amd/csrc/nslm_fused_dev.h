@@ -24,6 +24,7 @@ struct FusedArgs {
     int Lg, rpig, it_g, ntile_g;        // gate+up pass: chunks per row, virtual rows per iteration, iterations and items per pair
     int Ld, rpid, it_d, ntile_d;        // down pass (item i of a pair owns iterations i it / ntile .. (i + 1) it / ntile)
     int grid;
+    int gu_off;                         // per-item and grouped kernels: where, in floats of dynamic LDS, an item's gate / up row sums wait
     uint32_t spin;                      // polls a bounded wait makes before it gives up and sets the error word
 };
 
