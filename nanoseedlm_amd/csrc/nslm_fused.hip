@@ -419,7 +419,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
 
 template <int P, bool GATEUP, bool SHFL, int NT, typename Emit>
 __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const WSlice& wB, int L, int rpi, int v0, int v1,
-                                            const uint32_t* tab, const float* xl, int xstride, int nt, float* part, Emit emit) {
+                                            const uint32_t* tab, const float* xl, int xstride, int nt, float* part, float2* gu, Emit emit) {
     const int tid = threadIdx.x, lr = tid / L, ch = tid - lr * L;
     const bool active = lr < rpi;
     auto fetch = [&](int vv) {   // (rows past the last: the last row's records once more)
@@ -443,7 +443,10 @@ __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const W
                 for (int o = L >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
                 if (GATEUP) {
                     const float other = __shfl_xor(s, L);
-                    if (t < nt && active && ch == 0 && !(v & 1) && v < v1) emit(t, v >> 1, s * NSLM_R32, other * NSLM_R32);
+                    if (t < nt && active && ch == 0 && !(v & 1) && v < v1) {
+                        if (gu) gu[t * ((v1 - v0) >> 1) + ((v - v0) >> 1)] = make_float2(s, other);   // (as in rows_pass)
+                        else emit(t, v >> 1, s * NSLM_R32, other * NSLM_R32);
+                    }
                 } else if (t < nt && active && ch == 0 && v < v1) emit(t, v, s * NSLM_R32, 0.0f);
             }
         } else {
@@ -473,11 +476,22 @@ __device__ __forceinline__ void rows_pass_n(Chunk cur, const WSlice& wA, const W
         cur = nxt;
     }
     if (!SHFL) __syncthreads();   // part may be reused by the next pass
+    if (GATEUP && SHFL && gu) {
+        __syncthreads();
+        const int nr = (v1 - v0) >> 1;
+        for (int i = tid; i < nr * nt; i += 256) {
+            const int t = i / nr, r = i - t * nr;
+            const float2 q = gu[i];
+            emit(t, (v0 >> 1) + r, q.x * NSLM_R32, q.y * NSLM_R32);
+        }
+    }
 }
 
 template <int P, int NT, bool SHFL_G, bool SHFL_D>
 __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     extern __shared__ __attribute__((aligned(16))) float xl[];   // NT rows of max(d, ff) activations, chunk-padded, side by side
+    // behind them, where the launcher found room without giving up a resident workgroup: the gate and up row sums of the item in hand
+    float2* const gu_s = a.gu_off > 0 ? (float2*) (xl + a.gu_off) : nullptr;
     // What only the routing and the building of the groups need lives in the same area, which the passes overwrite (the launch
     // asks for FG_PRE_BYTES at least): a kilobyte of static LDS less is a resident workgroup more at some widths.
     float* const rv = xl;                                          // [1024] a token's logits
@@ -672,10 +686,10 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             st_agent(a.A + (size_t) gm[g * NT + m] * a.ff + r, bfr(silu_bf(bfr(gs)) * bfr(us)));
         };
         if (nt == 1)   // a group of one: the one-token loop, no second row of multiply-adds
-            rows_pass<P, true, SHFL_G>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, (float (*)[256]) part, nullptr,
+            rows_pass<P, true, SHFL_G>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, (float (*)[256]) part, gu_s,
                                        [&](int r, float gs, float us) { put_a(0, r, gs, us); });
         else
-            rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part, put_a);
+            rows_pass_n<P, true, SHFL_G, NT>(c0, sl_s[0], sl_s[1], a.Lg, a.rpig, v0, v1, tab, xl, xsg, nt, part, gu_s, put_a);
         wg_release();   // this item's rows of A are written: one more of the group's gate+up items is done
         __syncthreads();
         if (tid == 0 && atomicAdd(&grpc[g * 96], 1u) == (uint32_t) (a.ntile_g - 1)) st_agent(&grpc[g * 96 + 32], 1u);
@@ -711,7 +725,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
             rows_pass<P, false, SHFL_D>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, (float (*)[256]) part, nullptr,
                                         [&](int r, float sm, float) { put_d(0, r, sm, 0.0f); });
         else
-            rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part, put_d);
+            rows_pass_n<P, false, SHFL_D, NT>(d0, sl_s[2], sl_s[2], a.Ld, a.rpid, v0, v1, tab, xl, xsd, nt, part, nullptr, put_d);
         wg_release();
         for (int m = 0; m < nt; ++m) {   // one ticket per member's (token, row tile); the token's last arrival sums its experts
             const int t = gm[g * NT + m] / a.kk;
@@ -878,6 +892,25 @@ int launch_grouped(hipStream_t st, FusedArgs& a, bool sg, bool sd) {
     int grid = items < gmax ? (int) items : gmax;
     if (grid < a.T) grid = a.T < gmax ? a.T : gmax;
     a.grid = grid;
+    // Room behind the staged rows for the row sums of a gate + up item (so that SwiGLU and the store run once behind the item's
+    // row loop), taken only where it costs no resident workgroup: with 4 KB for it C2's 16-row step lost one of four and 6 %.
+    a.gu_off = 0;
+    if (sg) {
+        const size_t base = (lds + 15) & ~(size_t) 15;
+        const size_t want = base + (size_t) NT * ((a.it_g + a.ntile_g - 1) / a.ntile_g) * (a.rpig / 2) * sizeof(float2);
+        static size_t ok_lds[2] = {0, 0}, bad_lds[2] = {~(size_t) 0, ~(size_t) 0};   // by sd: the largest request known to keep per_cu, the smallest known not to
+        bool fits = want <= ok_lds[sd];
+        if (!fits && want < bad_lds[sd] && want <= 48 * 1024) {
+            int n = 0;
+            fits = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, 256, want) == hipSuccess && n >= per_cu;
+            if (fits) ok_lds[sd] = want;
+            else bad_lds[sd] = want;
+        }
+        if (fits) {
+            a.gu_off = (int) (base / sizeof(float));
+            lds = want;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned) grid), dim3(256), lds, st, a);
     host_note_launch();
     return 0;
