@@ -179,6 +179,19 @@ void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out)
 void kc_mm_grouped_packed_rows(kc_stream_t s, int fmt, const WSlice* ws, int K, int R, const uint16_t* x, int xs, float* y,
                                int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
                                int tile_rows);
+/* Two grouped GEMMs of one shape over the same tiles and activations in one launch (an expert's gate and up matrices: ya = the
+ * ws_a slices' product, yb = the ws_b slices'), each bit for bit what kc_mm_grouped_packed_rows gives alone: one launch's ramp
+ * and tail instead of two.  No counterpart in the reference (two launches, engine/mova_cuda.c:1308-1311). */
+void kc_mm_grouped_packed_pair(kc_stream_t s, int fmt, const WSlice* ws_a, const WSlice* ws_b, int K, int R, const uint16_t* x, int xs,
+                               float* ya, float* yb, int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt,
+                               int max_tiles, int tile_rows);
+/* The gate GEMM, the up GEMM and kc_swiglu_pack in one launch: a workgroup's 64 weight rows are 32 gate rows and the same 32 up
+ * rows of the tile's expert, so a lane holds both sums of a (pair, row) and stores a16[pair][row] = the BF16 bits kc_swiglu_pack
+ * would have stored from the two GEMMs' outputs (bit for bit).  R = the expert width, ys = a16's row stride.  -1 (nothing
+ * launched) where kc_mm_grouped_packed would not take its streamed kernel (K % 64, alignment) or kc_store_f32(1) is set.
+ * No counterpart in the reference (three launches, engine/mova_cuda.c:1308-1312). */
+int kc_mm_grouped_swiglu(kc_stream_t s, int fmt, const WSlice* gate, const WSlice* up, int K, int R, const uint16_t* x, int xs, uint16_t* a16,
+                         int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles, int tile_rows);
 /* 1: the matvec family stores unrounded f32 instead of BF16-rounded values (for comparison with CPU references that do
  * not round, nslm/lib_cpu_seed4.c).  Process-global like kc_seed_gemm_f32; default 0 = the reference's store. */
 void kc_store_f32(int on);

@@ -385,9 +385,11 @@ int nslm_moe_step(NslmMoe* m, kc_stream_t s, int layer, const float* xn, int T, 
         if (packed) {
             if (c->router != NSLM_ROUTE_SOFTMAX) kc_pack_input_bf16(s, xn, m->px, (size_t) T * d);   /* else: made for the router */
             /* a step of T rows chooses no expert more than T times: no tile holds more than T pairs */
-            kc_mm_grouped_packed_rows(s, c->fmt, gate, d, ff, m->px, d, m->G, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T);
-            kc_mm_grouped_packed_rows(s, c->fmt, up, d, ff, m->px, d, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T);
-            kc_swiglu_pack(s, m->G, m->U, (uint16_t*) m->A, (size_t) P * ff);
+            /* gate, up and SwiGLU in one launch (else: the two GEMMs in one launch, then SwiGLU) */
+            if (kc_mm_grouped_swiglu(s, c->fmt, gate, up, d, ff, m->px, d, (uint16_t*) m->A, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T)) {
+                kc_mm_grouped_packed_pair(s, c->fmt, gate, up, d, ff, m->px, d, m->G, m->U, ff, k, m->perm, m->tiles, m->ntiles, m->max_tiles, T);
+                kc_swiglu_pack(s, m->G, m->U, (uint16_t*) m->A, (size_t) P * ff);
+            }
             kc_mm_grouped_packed_rows(s, c->fmt, down, ff, d, (const uint16_t*) m->A, ff, m->D, d, 1, m->perm, m->tiles, m->ntiles,
                                       m->max_tiles, T);
         } else {

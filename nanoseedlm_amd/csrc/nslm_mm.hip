@@ -27,6 +27,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 struct MmArgs {
     int K, R, T, xs, ys, xdiv, add, f32out;
+    const WSlice* ws2;   // grouped launches of two matrices over the same tiles (grid.z = 2): the second slice table ..
+    float* y2;           // .. and its output
+    uint16_t* a16;       // non-null: a workgroup's 64 weight rows are 32 gate rows (ws) and the same 32 up rows (ws2), and what it
+                         // stores is their SwiGLU as BF16 bits [pair][ys] (the two GEMMs and the SwiGLU + pack pass in one launch)
 };
 
 // A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding global load of the
@@ -383,19 +387,30 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     const bool producer = wv >= NCW;
     const bool grouped = tiles != nullptr;
     if (grouped && ntiles && (int) blockIdx.y >= *ntiles) return;
-    const int r0 = (int) blockIdx.x * BM;
+    const bool gu = a.a16 != nullptr;   // (grouped launches only)
+    const int r0 = (int) blockIdx.x * (gu ? BM / 2 : BM);
     int start, count;
     WSlice wt;
     if (grouped) {
         const MmTile tl = tiles[blockIdx.y];
-        wt = ws[tl.slice];
+        if (blockIdx.z) {   // the launch's second matrix: same tiles and activations, its own slices and output
+            ws = a.ws2;
+            Y = a.y2;
+        }
+        // (gate / up tiles: the decoder waves of the tile's upper 32 rows read the up slice)
+        wt = gu && tid >= 64 * NCW + 128 ? a.ws2[tl.slice] : ws[tl.slice];
         start = tl.start;
         count = min(tl.count, BN);   // (a tile never holds more than the launch was told: see mm_grouped)
         if (BN < MMT_BN && tl.count > BN) {
             // a broken promise is made visible: the pairs this launch cannot reach are stored as NaN, not left stale
-            for (int i = BN * BM + tid; i < tl.count * BM; i += NTHR) {
-                const int orow = r0 + i % BM;
-                if (orow < a.R) Y[(size_t) perm[tl.start + i / BM] * a.ys + orow] = __uint_as_float(0x7FC00000u);
+            const int rows = gu ? BM / 2 : BM;
+            for (int i = BN * rows + tid; i < tl.count * rows; i += NTHR) {
+                const int orow = r0 + i % rows;
+                const size_t at = (size_t) perm[tl.start + i / rows] * a.ys + orow;
+                if (orow < a.R) {
+                    if (gu) a.a16[at] = 0x7FC0u;
+                    else Y[at] = __uint_as_float(0x7FC00000u);
+                }
             }
         }
     } else {
@@ -416,7 +431,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
 
     if (producer) {
         // rows past R decode row R - 1 again (never stored)
-        const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = min(r0 + rr, a.R - 1), nbk = a.K / 8;
+        const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = min(r0 + (gu ? rr & 31 : rr), a.R - 1), nbk = a.K / 8;
         // This thread's two blocks of step s.  Always the same loads - steps past the end request the last step again, and a
         // stream at any 2-byte boundary is read by the same instruction (the load is typed with that alignment) - so that the
         // compiler knows how many loads are in flight at every use: with the loads inside conditions it had waited, after
@@ -609,6 +624,20 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     wait_vm<0>();
     // accumulator element v of lane l: token row 8 * (v / 4) + 4 * (l / 32) + v % 4, weight column l % 32
     const bool plain = !a.add && !a.f32out;
+    if (gu) {   // n = 0: the gate rows, n = 1: the same rows of up, in the same lane: the values the two GEMMs would have stored
+                // (rounded to BF16), then SwiGLU and its rounding, stored as BF16 bits
+#pragma unroll
+        for (int m = 0; m < CT; ++m)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int tok = wtok + 32 * m + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int dst = drow[tok], orow = r0 + (lane & 31);
+                if (dst < 0 || orow >= a.R) continue;
+                const float av = bfr(silu_bf(bfr(acc[m][0][v])) * bfr(acc[m][1][v]));
+                a.a16[(size_t) dst * a.ys + orow] = (uint16_t) (__float_as_uint(av) >> 16);
+            }
+        return;
+    }
 #pragma unroll
     for (int m = 0; m < CT; ++m)
 #pragma unroll
@@ -657,7 +686,7 @@ void launch_mm_stream(hipStream_t st, int fmt, const MmArgs& a, WSlice wd, const
 template <bool PACKED>
 void mm_dense(hipStream_t st, int fmt, WSlice w, int K, int R, const void* x, int xs, float* y, int ys, int T, int add) {
     if (T < 1 || R < 1) return;
-    MmArgs a = {K, R, T, xs, ys, 1, add, host_store_f32()};
+    MmArgs a = {K, R, T, xs, ys, 1, add, host_store_f32(), nullptr, nullptr, nullptr};
     const unsigned gx = (unsigned) (R + BM - 1) / BM;
     if (PACKED && stream_ok(fmt, K, xs, x, T)) {
         if (T > 256) launch_mm_stream<2, 8, 4>(st, fmt, a, w, nullptr, x, y, nullptr, nullptr, nullptr, dim3(gx, (unsigned) (T + 511) / 512));
@@ -671,19 +700,25 @@ void mm_dense(hipStream_t st, int fmt, WSlice w, int K, int R, const void* x, in
 }
 template <bool PACKED>
 void mm_grouped(hipStream_t st, int fmt, const WSlice* ws, int K, int R, const void* x, int xs, float* y, int ys, int xdiv,
-                const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int grid_tiles, int tile_rows) {
+                const int32_t* perm, const MmTile* tiles, const int32_t* ntiles, int grid_tiles, int tile_rows,
+                const WSlice* ws2 = nullptr, float* y2 = nullptr) {
     if (grid_tiles < 1 || R < 1) return;
-    MmArgs a = {K, R, 0, xs, ys, xdiv, 0, host_store_f32()};
+    MmArgs a = {K, R, 0, xs, ys, xdiv, 0, host_store_f32(), ws2, y2, nullptr};
     WSlice none = {};
     if (PACKED && stream_ok(fmt, K, xs, x, 0)) {
         // grouped tiles are mostly a few pairs of one expert: decode-bound, so a short ring buys two workgroups a CU - and
         // where the caller knows that no tile holds more than 32 pairs, one multiplying wave instead of four buys four
-        const dim3 grid((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles);
+        const dim3 grid((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles, ws2 ? 2u : 1u);
         if (tile_rows <= 32) launch_mm_stream<1, 1, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
         else launch_mm_stream<1, 4, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
         return;
     }
     launch_mm<1, PACKED>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
+    if (ws2) {   // (the first-generation kernel takes one matrix a launch)
+        a.ws2 = nullptr;
+        a.y2 = nullptr;
+        launch_mm<1, PACKED>(st, fmt, a, none, ws2, x, y2, perm, tiles, ntiles, dim3((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles));
+    }
 }
 
 }   // namespace
@@ -723,6 +758,23 @@ void kc_mm_grouped_packed_rows(kc_stream_t s, int fmt, const WSlice* ws, int K, 
                                int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles,
                                int tile_rows) {
     mm_grouped<true>((hipStream_t) s, fmt, ws, K, R, x, xs, y, ys, xdiv, perm, tiles, nt, max_tiles, tile_rows < 1 ? MMT_BN : tile_rows);
+}
+int kc_mm_grouped_swiglu(kc_stream_t s, int fmt, const WSlice* gate, const WSlice* up, int K, int R, const uint16_t* x, int xs, uint16_t* a16,
+                         int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt, int max_tiles, int tile_rows) {
+    if (max_tiles < 1 || R < 1) return 0;
+    if (!stream_ok(fmt, K, xs, x, 0) || host_store_f32()) return -1;
+    MmArgs a = {K, R, 0, xs, ys, xdiv, 0, 0, up, nullptr, a16};
+    WSlice none = {};
+    const dim3 grid((unsigned) (R + BM / 2 - 1) / (BM / 2), (unsigned) max_tiles);
+    if (tile_rows >= 1 && tile_rows <= 32) launch_mm_stream<1, 1, 3>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);
+    else launch_mm_stream<1, 4, 3>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);
+    return 0;
+}
+void kc_mm_grouped_packed_pair(kc_stream_t s, int fmt, const WSlice* ws_a, const WSlice* ws_b, int K, int R, const uint16_t* x, int xs,
+                               float* ya, float* yb, int ys, int xdiv, const int32_t* perm, const MmTile* tiles, const int32_t* nt,
+                               int max_tiles, int tile_rows) {
+    mm_grouped<true>((hipStream_t) s, fmt, ws_a, K, R, x, xs, ya, ys, xdiv, perm, tiles, nt, max_tiles, tile_rows < 1 ? MMT_BN : tile_rows,
+                     ws_b, yb);
 }
 
 }   // extern "C"

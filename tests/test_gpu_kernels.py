@@ -717,6 +717,65 @@ def test_mm_grouped_packed_rows_equals_grouped_packed(fmt, T):
     assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("T", [5, 40])
+def test_mm_grouped_packed_pair_equals_two_launches(T):
+    """kc_mm_grouped_packed_pair (an expert's gate and up matrices over the same tiles in one launch) against two
+    kc_mm_grouped_packed_rows launches, and kc_mm_grouped_swiglu (the two and SwiGLU + pack in one launch) against
+    kc_swiglu_pack of their outputs, bit for bit; 5 rows take the narrow workgroups, 40 rows the wide ones; 72 weight rows:
+    not a multiple of a tile either way."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(4000 + T)
+    E, k, R, K, fmt = 9, 4, 72, 256, packs.MF_SEED4P4
+    tabs, keep = [], []
+    for _ in range(2):
+        p = make_pack(rng, fmt, E, R, K)
+        seeds, words, codes = moe.DevBuf.from_array(p["seeds"]), moe.DevBuf.from_array(p["coefs"]), moe.DevBuf.from_array(p["codes"])
+        arr = (backend.WSlice * E)()
+        for e in range(E):
+            arr[e].p[0] = seeds.ptr.value + e * R * K // 4
+            arr[e].p[1] = words.ptr.value + e * R * K // 4
+            arr[e].p[3] = codes.ptr.value + e * R * K // 16
+            arr[e].eb = int(p["eb"][e])
+        tab = moe.DevBuf(C.sizeof(arr))
+        backend.check(L.nh_memcpy_h2d(tab.ptr, arr, C.c_size_t(C.sizeof(arr))), "nh_memcpy_h2d")
+        tabs.append(tab)
+        keep += [seeds, words, codes, tab]
+    P = T * k
+    ind = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    di = moe.DevBuf.from_array(ind)
+    mt = P // 128 + E + 1
+    perm, tiles, work = moe.DevBuf(4 * P), moe.DevBuf(16 * mt), moe.DevBuf(4 * (2 * E + 4))
+    L.nh_memset(work.ptr, 0, C.c_size_t(work.nbytes))
+    L.nh_memset(tiles.ptr, 0, C.c_size_t(tiles.nbytes))
+    x = moe.DevBuf.from_array(packs.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32)))
+    ys = [moe.DevBuf(4 * P * R) for _ in range(4)]
+    for y in ys:
+        L.nh_memset(y.ptr, 0xFF, C.c_size_t(y.nbytes))
+    moe.device_sync()
+    L.kc_bucket(None, di.ptr, P, E, perm.ptr, tiles.ptr, work.ptr)
+    L.kc_mm_grouped_packed_rows(None, fmt, tabs[0].ptr, K, R, x.ptr, K, ys[0].ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T)
+    L.kc_mm_grouped_packed_rows(None, fmt, tabs[1].ptr, K, R, x.ptr, K, ys[1].ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T)
+    L.kc_mm_grouped_packed_pair(None, fmt, tabs[0].ptr, tabs[1].ptr, K, R, x.ptr, K, ys[2].ptr, ys[3].ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T)
+    # and with SwiGLU inside: the bits kc_swiglu_pack makes of the two outputs
+    pa, pb = moe.DevBuf(2 * P * R), moe.DevBuf(2 * P * R)
+    L.nh_memset(pa.ptr, 0xFF, C.c_size_t(pa.nbytes))
+    L.nh_memset(pb.ptr, 0xFF, C.c_size_t(pb.nbytes))
+    L.kc_swiglu_pack(None, ys[0].ptr, ys[1].ptr, pa.ptr, C.c_size_t(P * R))
+    assert L.kc_mm_grouped_swiglu(None, fmt, tabs[0].ptr, tabs[1].ptr, K, R, x.ptr, K, pb.ptr, R, k, perm.ptr, tiles.ptr, work.ptr, mt, T) == 0
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    a0, a1, b0, b1 = [y.to_array(np.uint32, (P, R)) for y in ys]
+    assert not (a0 == 0xFFFFFFFF).any() and not (a1 == 0xFFFFFFFF).any() and not np.array_equal(a0, a1)
+    assert np.array_equal(a0, b0) and np.array_equal(a1, b1)
+    sa, sb = pa.to_array(np.uint16, (P, R)), pb.to_array(np.uint16, (P, R))
+    assert not (sa == 0xFFFF).all() and np.array_equal(sa, sb)
+    for buf in keep + [di, perm, tiles, work, x, pa, pb] + ys:
+        buf.free()
+
+
 def test_mm_grouped_packed_rows_marks_a_broken_bound():
     """The bound is the caller's promise.  Indices that break it (10 rows that all name expert 2 four times: one tile of 40
     pairs under tile_rows = 10) leave the tile's first 32 pairs as kc_mm_grouped_packed computes them and the pairs beyond as
