@@ -268,6 +268,16 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         return sel[3 + (t * kk + j) * 3 + which];
     };
 
+    // (the down pass's threads and records, here already: a wave that has run out of gate + up tasks requests its first down records
+    // in the slot where its next task's records would have been requested, a whole task ahead of their use)
+    const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
+    const int dl = (int) ((uint32_t) tid / c.by_Ld), dch = tid - dl * Ld;
+    auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
+        const int g = min(it * c.rpi + dl, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
+        const WSlice& w = slice(min(t, T - 1), jj, 2);
+        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch);
+    };
+    Chunk dcur;
     // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
     const int q_lo = (int) blockIdx.x * c.n_c, n_loc = max(0, min(c.n_c, c.Wt - q_lo));   // this CU's tasks a token
     const int lr = lane >> c.lgL, ch = lane & (Lg - 1);
@@ -323,13 +333,16 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 ++ct;
             }
         };
-        // (the loads are unconditional - past the last task, the records of pair 0's first rows once more: a load under a
-        // condition keeps the compiler from counting the loads in flight, and it then waits for the next task's records
-        // before it computes the current one)
+        // (the loads are unconditional: a load under a condition keeps the compiler from counting the loads in flight, and it
+        // then waits for the next task's records before it computes the current one.  Past the last task the slot requests
+        // the thread's first down records instead.)
+        const int g_d = min(dl, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
+        const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) dch;
         auto fetch = [&](int t, int i) {
             const bool ok = t < T;
             const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), r = (q - j * c.tpp) << c.lgV;   // the task's first SwiGLU row
-            return load_chunk<P>(slice_gu(ok ? t : 0, j), (uint32_t) r * (uint32_t) Lg + lane_unit);
+            const WSlice& w = ok ? slice_gu(t, j) : slice(0, jj_d, 2);
+            return load_chunk<P>(w, ok ? (uint32_t) r * (uint32_t) Lg + lane_unit : unit_d);
         };
         int t, i;
         claim(t, i);
@@ -364,6 +377,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             t = tn;
             i = inx;
         }
+        dcur = cur;   // (the last request of the loop, or of the first claim: the down records)
     }
     else if (n_loc > 0) {
         // Rows whose chunks do not fit a wave (a row of 45 chunks, say): the pass goes by iterations of the whole workgroup, a thread
@@ -415,6 +429,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             if (wv == NW - 1) publish(t);
         }
     }
+    if constexpr (!SHFL_G) dcur = fetch_d(0, 0);
     // Housekeeping, off the critical path: the lines of this kernel's logits table that this launch did not write, and the
     // other step kernels' table (every launch of theirs rewrites all of it, the rows it does not use with zero: a word that
     // does not carry the current generation is then never older than one launch), are left at zero.
@@ -427,17 +442,11 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     if (tid == 0) arrive_finish(a.sync, (uint32_t) G, gen, arrived);
 
     // ---- down: CU c owns rows [c rpc, (c + 1) rpc) of every pair; a thread a chunk of a (pair, row); then the experts' sum --------
-    const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
-    const int dl = (int) ((uint32_t) tid / c.by_Ld), dch = tid - dl * Ld;
-    auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
-        const int g = min(it * c.rpi + dl, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
-        const WSlice& w = slice(min(t, T - 1), jj, 2);
-        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch);
-    };
-    Chunk dcur = fetch_d(0, 0);
     float* part = (float*) scr;
-    for (int t = 0; t < T; ++t) {
-        // the token's A is complete when the last CU has raised the ready words: lane 0 polls the word of this CU's group (bounded)
+    // the token's A is complete when the last CU has raised the ready words (lane 0 polls the word of this CU's group, bounded);
+    // then all pairs' A of the token, 16 bytes (a block of 8 values) a thread, staged as the down matvec reads it
+    // (block b of the token = block b % nbp of pair b / nbp: a pair's row is whole chunks, so the token's pairs lie in xd as one row)
+    auto wait_stage = [&](int t) {
         if (tid == 0) {
             const uint32_t* rdy = a.sync + FUSED_CU_WORDS + t * FUSED_CU_TOKEN_WORDS + 32 * (BAR_GROUPS + 1 + blockIdx.x % BAR_GROUPS);
             while (ld_agent(rdy) != tag) {
@@ -450,8 +459,6 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             }
         }
         __syncthreads();
-        // all pairs' A of the token, 16 bytes (a block of 8 values) a thread, staged as the down matvec reads it
-        // (block b of the token = block b % nbp of pair b / nbp: a pair's row is whole chunks, so the token's pairs lie in xd as one row)
         for (int b = tid; b < kk * c.nbp; b += NTHR) {
             const unsigned long long* src = (const unsigned long long*) (xa16 + (size_t) t * kk * a.ff + (size_t) b * 8);
             const unsigned long long lo = ld_agent(src), hi = ld_agent(src + 1);
@@ -460,46 +467,41 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             store_block<P>(xd, b, v);
         }
         __syncthreads();
-        for (int it = 0; it < c.nit; ++it) {
-            const bool last = it + 1 == c.nit;
-            const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
-            const int g = it * c.rpi + dl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
-            const bool ok = dl < c.rpi && g < c.rows_t && rr < nr;
-            float acc[1] = {0.0f};
-            if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + dch * XP, 0, 1, acc);
-            if (SHFL_D) {
-                float s = acc[0];
-                for (int o = Ld >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
-                if (ok && dch == 0) {
-                    const float dv = bfr(s * NSLM_R32);
-                    dsum[g] = dv;
-                    a.D[((size_t) t * kk + j) * a.d + r0 + rr] = dv;
-                }
-            } else {
-                part[tid] = acc[0];
-                __syncthreads();
-                const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
-                if (tid < c.rpi && gs < c.rows_t && rs < nr) {
-                    // the row's partial sums in chunk order; eight are read before the first is added (a chunk past the row's
-                    // last counts +0, which leaves the sum's bits alone)
-                    float s = 0.0f;
-                    for (int c0 = 0; c0 < Ld; c0 += 8) {
-                        float pv[8];
-#pragma unroll
-                        for (int cc = 0; cc < 8; ++cc) pv[cc] = part[tid * Ld + min(c0 + cc, Ld - 1)];
-#pragma unroll
-                        for (int cc = 0; cc < 8; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
-                    }
-                    const float dv = bfr(s * NSLM_R32);
-                    dsum[gs] = dv;
-                    a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
-                }
-                if (!last) __syncthreads();   // part is written again by the next iteration
+    };
+    // the rows' sums of one iteration from the threads' chunk sums, rounded as the separate launches round them
+    auto rows_out = [&](int t, int it, float acc0, bool ok, int g, int j, int rr, bool last) {
+        if (SHFL_D) {
+            float s = acc0;
+            for (int o = Ld >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            if (ok && dch == 0) {
+                const float dv = bfr(s * NSLM_R32);
+                dsum[g] = dv;
+                a.D[((size_t) t * kk + j) * a.d + r0 + rr] = dv;
             }
-            dcur = dnxt;
+        } else {
+            part[tid] = acc0;
+            __syncthreads();
+            const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
+            if (tid < c.rpi && gs < c.rows_t && rs < nr) {
+                // the row's partial sums in chunk order; eight are read before the first is added (a chunk past the row's
+                // last counts +0, which leaves the sum's bits alone)
+                float s = 0.0f;
+                for (int c0 = 0; c0 < Ld; c0 += 8) {
+                    float pv[8];
+#pragma unroll
+                    for (int cc = 0; cc < 8; ++cc) pv[cc] = part[tid * Ld + min(c0 + cc, Ld - 1)];
+#pragma unroll
+                    for (int cc = 0; cc < 8; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
+                }
+                const float dv = bfr(s * NSLM_R32);
+                dsum[gs] = dv;
+                a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
+            }
+            if (!last) __syncthreads();   // part is written again by the next iteration
         }
-        __syncthreads();
-        // out = sum_j wt_j D_j in j order (kq4_moe_combine's FMA chain), the shared expert's pair with weight 1 last
+    };
+    // out = sum_j wt_j D_j in j order (kq4_moe_combine's FMA chain), the shared expert's pair with weight 1 last
+    auto combine = [&](int t) {
         if (tid < nr) {
             const float* rw = rw_s + t * 36;
             float acc = 0.0f;
@@ -517,6 +519,39 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             const size_t at = (size_t) t * a.os + r0 + tid;
             a.out[at] = a.res ? bfr(a.res[at] + bfr(acc)) : acc;
         }
+    };
+    if (P == 4 && T == 1 && c.nit == 1) {
+        // One token whose down rows take one iteration: what the chunk can do without A - the streams, the byte transposition,
+        // the twelve exact column sums of every block - is done now, while A is still on its way between the CUs; what remains
+        // behind the exchange is a convert and a multiply-add a column (cols_pre / cols_post: chunk_dot's bits).
+        if constexpr (P == 4) {
+            const int g = dl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
+            const bool ok = dl < c.rpi && g < c.rows_t && rr < nr;
+            uint32_t zp[8][6];
+            if (ok) cols_pre(dcur, tab, zp);
+            wait_stage(0);
+            float acc0 = 0.0f;
+            if (ok) cols_post(zp, dcur.codes, slice(0, j, 2).eb, xd + j * (Ld * XP) + dch * XP, acc0);
+            rows_out(0, 0, acc0, ok, g, j, rr, true);
+            __syncthreads();
+            combine(0);
+        }
+        return;
+    }
+    for (int t = 0; t < T; ++t) {
+        wait_stage(t);
+        for (int it = 0; it < c.nit; ++it) {
+            const bool last = it + 1 == c.nit;
+            const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
+            const int g = it * c.rpi + dl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
+            const bool ok = dl < c.rpi && g < c.rows_t && rr < nr;
+            float acc[1] = {0.0f};
+            if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + dch * XP, 0, 1, acc);
+            rows_out(t, it, acc[0], ok, g, j, rr, last);
+            dcur = dnxt;
+        }
+        __syncthreads();
+        combine(t);
         // (the next token's staging writes xd, which every thread has finished reading before the barrier above; dsum and part
         // are next written behind the next token's first barrier)
     }

@@ -145,6 +145,44 @@ __device__ __forceinline__ void cols_dot(uint32_t up, uint32_t g, uint32_t be, f
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = fmaf(d[t], e2, acc[t]);
 }
+// The column form in two halves, for a caller that has a chunk's records before it has the activations: cols_pre forms the
+// twelve exact column sums Z'(0..10), Q of every block (|Z'| <= 256: two to a register as int16), cols_post multiplies them with the
+// staged values - the same converts, the same FMA chain in the same order as cols_dot, so the same bits.
+__device__ __forceinline__ void cols_pre(const Chunk& ck, const uint32_t* tab, uint32_t (&zp)[8][6]) {
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
+        const uint32_t g = stream_of(tab, (b & 1) ? ss >> 16 : ss & 0xFFFFu);
+        const uint32_t up = (b & 1) ? ss : ss << 16;
+        const uint32_t be = coef_bytes(cc, b & 1), bo = be << 4;
+        uint32_t G[6];
+        col_bytes_p4(up, g, G);
+#pragma unroll
+        for (int i = 0; i < 6; ++i) {
+            const int z0 = dot8z(G[i], be), z1 = i == 5 ? dot8ones(be) : dot8z(G[i], bo);
+            zp[b][i] = __builtin_amdgcn_perm((uint32_t) z1, (uint32_t) z0, 0x05040100u);   // { z0 as int16, z1 as int16 }
+        }
+        __builtin_amdgcn_sched_barrier(0);   // (a block at a time: 48 registers of results leave little room for eight blocks' temporaries)
+    }
+}
+__device__ __forceinline__ void cols_post(const uint32_t (&zp)[8][6], uint32_t codes, int eb, const float* xr, float& acc) {
+    const uint32_t ebase = (uint32_t) (eb + 127) << 23;
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const float* xb = xr + 12 * b;
+        const float4 x0 = *(const float4*) xb, x1 = *(const float4*) (xb + 4), x2 = *(const float4*) (xb + 8);
+        const float xs[12] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w, x2.x, x2.y, x2.z, x2.w};
+        const float e2 = __uint_as_float((((codes >> (4 * b)) & 15u) << 23) + ebase);
+        float d = 0.0f;
+#pragma unroll
+        for (int m = 0; m < 12; ++m) {
+            const uint32_t p = zp[b][m >> 1];
+            const float z = (m & 1) ? (float) ((int32_t) p >> 16) : (float) (int32_t) (int16_t) (p & 0xFFFFu);
+            d = m == 0 ? z * xs[0] : fmaf(z, xs[m], d);
+        }
+        acc = fmaf(d, e2, acc);
+    }
+}
 // PAIRED (P = 3 only): two blocks at a time in phase order (isum2_p3), as the GEMM's decoder waves decode: measured 1 % faster
 // in the persistent MoE kernel (three waves a SIMD), 6 % slower in the stand-alone matvec, which keeps the compiler's own order.
 template <int P, int NT, bool PAIRED = false, bool COLS = (P == 4)>
