@@ -312,6 +312,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
     };
 
     // ---- phase 2: gate + up + SwiGLU, items (pair, row tile) -------------------------------------------------------------
+    __builtin_amdgcn_s_setprio(2);   // (gate + up items go before the down items of the workgroups that share the CU: every down item waits for them)
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int p = item / a.ntile_g, tile = item - p * a.ntile_g, t = p / a.kk, j = p - t * a.kk;
         route(t);
@@ -340,6 +341,7 @@ __global__ void __launch_bounds__(256, WAVES) k_moe_decode(FusedArgs a) {   // W
         route_weights(t);
     }
     if (tid == 0) arrive_finish(a.sync, G, my_gen, arrived);   // here most workgroups are about to wait for their pair anyway
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- phase 3: down, then the last workgroup of a (token, row tile) sums the k experts --------------------------------
     // the first down item's records do not depend on phase 2: they are requested before the wait for the pair
@@ -667,6 +669,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
 
     // ---- gate + up + SwiGLU: items (group, row tile) ---------------------------------------------------------------------------
     int staged_g = -1;
+    __builtin_amdgcn_s_setprio(2);   // (as in k_moe_decode: gate + up items before the down items that wait for them)
     for (int item = (int) blockIdx.x; item < items_g; item += (int) G) {
         const int g = item / a.ntile_g, tile = item - g * a.ntile_g, nt = gn[g], e = pe[gm[g * NT]];
         const int v0 = tile * a.it_g / a.ntile_g * a.rpig, v1 = min((tile + 1) * a.it_g / a.ntile_g * a.rpig, 2 * a.ff);
@@ -696,6 +699,7 @@ __global__ void __launch_bounds__(256) k_moe_decode_grouped(FusedArgs a) {
     }
 
     if (tid == 0) arrive_finish(a.sync, G, my_gen, arrived);
+    __builtin_amdgcn_s_setprio(0);
 
     // ---- down, then the last workgroup of a (token, row tile) sums the token's experts ------------------------------------
     for (int item = (int) blockIdx.x; item < items_d; item += (int) G) {

@@ -347,6 +347,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         int t, i;
         claim(t, i);
         Chunk cur = fetch(t, i);
+        __builtin_amdgcn_s_setprio(2);   // (tasks, and the store of the CU's values, go before the waves that have run out of tasks)
         uint32_t mine = 0;   // tasks of the token in hand this wave has finished
         while (t < T) {
             int tn, inx;
@@ -378,6 +379,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             i = inx;
         }
         dcur = cur;   // (the last request of the loop, or of the first claim: the down records)
+        __builtin_amdgcn_s_setprio(0);
     }
     else if (n_loc > 0) {
         // Rows whose chunks do not fit a wave (a row of 45 chunks, say): the pass goes by iterations of the whole workgroup, a thread
