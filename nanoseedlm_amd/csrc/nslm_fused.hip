@@ -996,13 +996,11 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
-    // one workgroup per CU: ahead up to three tokens (C2, us, a workgroup per CU / per item, records from HBM: 1 token 22.8 / 25.6,
-    // 2: 37.2 / 38.0, 3: 48.9 / 49.7, 4: 61.6 / 60.1, 5: 74.4 / 71.7; with the staged inputs and the staged A in one LDS area
-    // 7 and 8 tokens fit too: 104 / 96 and 117 / 104); with an always-on expert the same three (the whole model's step at 4
-    // rows: 3.29 against 3.25 ms)
-    // (rows whose chunks do not fill a wave, where that kernel's gate + up pass goes by iterations of the workgroup - C3's rows of 45
-    // chunks, us: 1 token 59.4 / 68.0, 2: 108.0 / 109.8, 3: 157.1 / 156.9, 4: 206.0 / 197.4 - up to two)
-    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (sg ? 3 : 2))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
+    // one workgroup per CU: ahead at one token everywhere and at two where a row's chunks fill a wave (us, a workgroup per CU / per
+    // item, records from HBM.  C2: 1 token 20.4 / 25.2, 2: 36.6 / 35.5, 3: 48.4 / 45.5; C2's shape in P = 3: 24.6 / 26.3, 39.4 / 43.5,
+    // 54.7 / 50.9, 4: 70.0 / 63.8; 256 experts of 4096 x 1024: 45.8 / 54.9, 80.7 / 90.6, 168.8 / 168.9; C3, whose rows of 45 chunks
+    // make that kernel's gate + up pass go by iterations of the workgroup: 59.7 / 67.3, 108.7 / 105.0, 158.3 / 148.4)
+    if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (sg ? 2 : 1))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);
     return fmt == MF_SEED4P4 ? launch_fused<4>((hipStream_t) s, a, sg, sd, lds) : launch_fused<3>((hipStream_t) s, a, sg, sd, lds);

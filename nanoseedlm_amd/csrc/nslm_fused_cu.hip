@@ -319,11 +319,22 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         }
     };
     if constexpr (SHFL_G) {
-        // The CU's tasks of a token go to whichever wave asks next: a wave whose records arrive late, or that shares its SIMD
-        // with more waves, takes fewer.  A wave asks for its next task before it computes the current one, so that task's
-        // records travel meanwhile.  Task = (token, index in the CU's run); token T = none left.
-        int ct = 0;   // the token this wave draws from
+        // One token: wave w takes the CU's tasks w, w + 16, ..  Waves w, w + 4, w + 8, w + 12 share a SIMD, so the SIMDs' task counts
+        // differ by one at most, and the first records are requested without a counter's round trip.  (Handed out in the order
+        // of asking, the second round's tasks went to the waves that happened to finish first - on 28 % of the CUs three of them
+        // on one SIMD, whose last task then ended 0.8 us after the other CUs' - and some such CU is always the step's last.)
+        // More tokens: a token's tasks go to whichever wave asks next, because the wave that stores a token's values is busy for
+        // most of a task's time and falls behind a fixed schedule (3 tokens: 51.5 against 48.7 us).
+        // A wave asks for its next task before it computes the current one, so that task's records travel meanwhile.
+        // Task = (token, index in the CU's run); token T = none left.
+        int ct = 0, ci = wv - NW;   // the token this wave draws from; one token: the wave's last task
         auto claim = [&](int& t, int& i) {
+            if (T == 1) {
+                ci += NW;
+                if (ci < n_loc) { t = 0; i = ci; }
+                else { t = T; i = 0; }
+                return;
+            }
             for (;;) {
                 if (ct >= T || n_loc == 0) { t = T; i = 0; return; }
                 uint32_t got = 0;
