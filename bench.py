@@ -252,7 +252,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         # queued back to back, so there is no gap between them unless the step is wrapped in a graph).
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
                                frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
-                               kernel=("k_moe_decode_cu" if T <= (2 if name[:2] == "c2" else 1) else "k_moe_decode") + " (one launch per step)",
+                               kernel=("k_moe_decode_cu" if T == 1 else "k_moe_decode") + " (one launch per step)",
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, gate_up_alone=part, **counters_of(name))
         ind.free(); A.free()
     else:
