@@ -392,7 +392,14 @@ __device__ __forceinline__ float wide_dot(const float (&w)[8], const float* xb) 
     d = fmaf(w[6], x1.z, d);
     return fmaf(w[7], x1.w, d);
 }
-template <int FMT, int MODE>
+// ONE: a launch whose workgroups stage one row of activations for the rows of one matrix (gather launches; dense launches of one
+// token that do not also write the BF16 view).  Its waves request their pieces of work - 256 blocks of a row, four a lane - one
+// piece ahead: the first before the activations are staged, every later one before the piece in hand is multiplied, a row's
+// last before its sums are formed and stored.  So a wave's round trips to memory overlap with its other work (a launch of one row
+// a wave, 2880 x 2880 in Q4, was two latencies long: 5.9 us for 4.7 MB), and a wave that walks many rows waits for one piece while
+// it computes another.  (Launches of several tokens keep the plain loop: their accumulators, carried around the pipelined
+// loop, cost 70 registers and half the resident waves.)
+template <int FMT, int MODE, bool ONE>
 __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
     extern __shared__ __attribute__((aligned(16))) float xw[];   // [nt][K]
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -414,6 +421,81 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
     if (MODE == MULTI) {
         total = 0;
         for (int j = 0; j < a.nj; ++j) total += a.Rj[j];
+    }
+    if constexpr (ONE) {
+        // a wave's row rr: the matrix it belongs to (MULTI: the rows of the matrices follow each other) and its number there
+        auto row_of = [&](int rr, int& r, int& job) {
+            r = rr;
+            job = 0;
+            if (MODE == MULTI) {
+                while (job + 1 < a.nj && r >= a.Rj[job]) r -= a.Rj[job++];
+                wA = a.wj[job];
+                alA = ((uintptr_t) wA.p[0] & 15u) == 0;
+            }
+        };
+        auto request = [&](WideRaw<FMT> (&ra)[4], WideRaw<FMT> (&rb)[4], int r, int j0) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = j0 + 64 * u;
+                if (j < nbk) {
+                    ra[u] = wide_load<FMT>(wA, r, a.K, j, alA);
+                    if (MODE == GATEUP) rb[u] = wide_load<FMT>(wB, r, a.K, j, alB);
+                }
+            }
+        };
+        const int rstep = (int) gridDim.x * 4;
+        int rr = (int) blockIdx.x * 4 + wv, j0 = lane, r = 0, job = 0;
+        WideRaw<FMT> na[4], nb[4];
+        if (rr < total) {
+            row_of(rr, r, job);
+            request(na, nb, r, j0);
+        }
+        for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[i] = ((const float4*) xrow)[i];
+        __syncthreads();
+        float acc = 0.0f, accu = 0.0f;
+        while (rr < total) {
+            WideRaw<FMT> ca[4], cb[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                ca[u] = na[u];
+                cb[u] = nb[u];
+            }
+            const int r_now = r, job_now = job, j_now = j0;
+            j0 += 256;
+            const bool row_done = j0 >= nbk;
+            if (row_done) {
+                rr += rstep;
+                j0 = lane;
+                if (rr < total) row_of(rr, r, job);
+            }
+            if (rr < total) request(na, nb, r, j0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {   // the piece's arithmetic, in block order
+                const int j = j_now + 64 * u;
+                if (j >= nbk) break;
+                float w[8];
+                wide_weights<FMT>(ca[u], w);
+                acc = fmaf(wide_dot(w, xw + (size_t) j * 8), 1.0f, acc);
+                if (MODE == GATEUP) {
+                    wide_weights<FMT>(cb[u], w);
+                    accu = fmaf(wide_dot(w, xw + (size_t) j * 8), 1.0f, accu);
+                }
+            }
+            if (!row_done) continue;
+            float s = acc;
+            for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+            if (MODE == GATEUP) {
+                float u = accu;
+                for (int o = 32; o > 0; o >>= 1) u += __shfl_xor(u, o);
+                if (lane == 0) a.y[(size_t) pair * a.ys + r_now] = a.f32out ? (s / (1.0f + expf(-s))) * u : bfr(silu_bf(bfr(s)) * bfr(u));
+            } else if (lane == 0) {
+                if (MODE == MULTI) store_y(a.yj[job_now] + r_now, s, a.addj[job_now], a.f32out);
+                else store_y(a.y + (size_t) (MODE == DENSE ? tg0 : pair) * a.ys + r_now, s, a.add, a.f32out);
+            }
+            acc = 0.0f;
+            accu = 0.0f;
+        }
+        return;
     }
     // staging: with several rows a piece of every row is requested before the first is stored (a loop over the rows with a load
     // and a store each is one memory round trip a row: 8 us of a 14 us launch at 8 rows of 2048)
@@ -604,10 +686,20 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
     const int cap = (8 * cu_count() + ny - 1) / ny;
     if (gx > cap) gx = cap < 1 ? 1 : cap;
     const dim3 grid((unsigned) gx, (unsigned) ny);
+    // (one staged row of one matrix: the pipelined variant.  2880 x 2880 in Q4, one token: 5.9 -> 5.0 us; the multi-matrix launch of
+    // three such took 11.1 instead of 9.6 us with it and the gate + up launch the same 7.3, so those keep the plain loop)
+    const bool one = MODE == GATHER || (MODE == DENSE && (a.ttot > 0 ? a.ttot : a.nt) == 1 && !a.px);
 #define NSLM_WIDE(F)                                                                         \
     do {                                                                                     \
-        if (lds > 48 * 1024) allow_big_lds<k_mv_wide<F, MODE>>();                              \
-        hipLaunchKernelGGL((k_mv_wide<F, MODE>), grid, dim3(256), lds, st, a);               \
+        if (one) {                                                                           \
+            if constexpr (MODE == DENSE || MODE == GATHER) {                                 \
+                if (lds > 48 * 1024) allow_big_lds<k_mv_wide<F, MODE, true>>();                \
+                hipLaunchKernelGGL((k_mv_wide<F, MODE, true>), grid, dim3(256), lds, st, a); \
+            }                                                                                \
+        } else if constexpr (MODE != GATHER) {                                               \
+            if (lds > 48 * 1024) allow_big_lds<k_mv_wide<F, MODE, false>>();                   \
+            hipLaunchKernelGGL((k_mv_wide<F, MODE, false>), grid, dim3(256), lds, st, a);    \
+        }                                                                                    \
     } while (0)
     if (fmt == MF_BF16) NSLM_WIDE(MF_BF16);
     else if (fmt == MF_Q8) NSLM_WIDE(MF_Q8);
