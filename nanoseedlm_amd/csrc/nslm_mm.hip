@@ -383,6 +383,14 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     WTile* Wsm = (WTile*) (smem + NCW * XCH * XCHUNK);          // [2]
     __shared__ int srow[BN], drow[BN];
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    // FSYNC (one consumer wave: the grouped launches of a batched step, whose time is the decoders'): the weight tiles change hands
+    // by counters in LDS instead of a workgroup barrier a step.  A decoder waits only for the consumer to have read the tile it
+    // is about to overwrite (two steps back - it has, when the decode is what takes the time), never for the other decoders: with
+    // the barrier every step cost each decoder wave the wait for the slowest of the four (C2 at 32 rows: 271.2 -> 263.5 us, C3 at 16:
+    // 627 -> 609; with no hand-over at all and garbage computed: 247 and 540).  The dense 512-token GEMM with its eight consumer
+    // waves is indifferent to the barrier and keeps it.
+    constexpr bool FSYNC = NCW == 1;
+    __shared__ __attribute__((aligned(16))) uint32_t flg[8];
     const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool producer = wv >= NCW;
     const bool grouped = tiles != nullptr;
@@ -420,6 +428,56 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     }
     if (count < 1) return;
     if (seedf) load_tables(tab);
+    if (FSYNC && tid < 8) flg[tid] = 0u;
+    // flg[w], w < 4: weight steps decoder wave w has written; flg[4]: steps the consumer has read.  (One word a decoder, not a sum:
+    // with two tiles a decoder may be a step ahead of another, and three waves a step ahead would make up for one a step behind.)
+    // The polls and the posts are a few instructions of inline code with registers of their own: written in the language (volatile
+    // reads in a loop, s_setprio builtins around it) they cost 20 registers and with them the fifth wave a SIMD, i.e. a resident
+    // workgroup - a quarter more time instead of less.  A poll is bounded; a waiting wave drops to priority 0, so its polls take
+    // only the issue slots nobody else wants.
+    auto wait_written = [&](uint32_t need) {   // all four decoders have written `need` steps; back at priority 3
+        uint32_t g0, g1, g2, g3, spins = 1u << 24;
+        asm volatile("s_setprio 0\n\t"
+                     "1:\n\t"
+                     "ds_read_b32 %0, %5\n\t"
+                     "ds_read_b32 %1, %5 offset:4\n\t"
+                     "ds_read_b32 %2, %5 offset:8\n\t"
+                     "ds_read_b32 %3, %5 offset:12\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_min3_u32 %0, %0, %1, %2\n\t"
+                     "v_min_u32 %0, %0, %3\n\t"
+                     "v_cmp_ge_u32 vcc, %0, %6\n\t"
+                     "s_cbranch_vccnz 2f\n\t"
+                     "s_sub_u32 %4, %4, 1\n\t"
+                     "s_cmp_lg_u32 %4, 0\n\t"
+                     "s_cbranch_scc1 1b\n\t"
+                     "2:\n\t"
+                     "s_setprio 3"
+                     : "=&v"(g0), "=&v"(g1), "=&v"(g2), "=&v"(g3), "+s"(spins)
+                     : "v"((uint32_t) (uintptr_t) &flg[0]), "v"(need)
+                     : "vcc", "scc", "memory");
+    };
+    auto wait_read = [&](uint32_t need) {   // the consumer has read `need` steps; back at priority 2
+        uint32_t got, spins = 1u << 24;
+        asm volatile("s_setprio 0\n\t"
+                     "1:\n\t"
+                     "ds_read_b32 %0, %2\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_cmp_ge_u32 vcc, %0, %3\n\t"
+                     "s_cbranch_vccnz 2f\n\t"
+                     "s_sub_u32 %1, %1, 1\n\t"
+                     "s_cmp_lg_u32 %1, 0\n\t"
+                     "s_cbranch_scc1 1b\n\t"
+                     "2:\n\t"
+                     "s_setprio 2"
+                     : "=&v"(got), "+s"(spins)
+                     : "v"((uint32_t) (uintptr_t) &flg[4]), "v"(need)
+                     : "vcc", "scc", "memory");
+    };
+    // (every lane stores the same word; the wave's LDS accesses before it are complete)
+    auto post = [&](int which, uint32_t v) {
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_write_b32 %0, %1" ::"v"((uint32_t) (uintptr_t) &flg[which]), "v"(v) : "memory");
+    };
     for (int i = tid; i < BN; i += NTHR) {
         const bool ok = i < count;
         const int j = start + (ok ? i : 0);   // padding rows load the tile's first row; their results are never stored
@@ -430,6 +488,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     const int nsteps = a.K / WK;
 
     if (producer) {
+        if (FSYNC) __builtin_amdgcn_s_setprio(2);
         // rows past R decode row R - 1 again (never stored)
         const int ptid = tid - 64 * NCW, rr = ptid >> 2, jb = ptid & 3, row = min(r0 + (gu ? rr & 31 : rr), a.R - 1), nbk = a.K / 8;
         // This thread's two blocks of step s.  Always the same loads - steps past the end request the last step again, and a
@@ -513,6 +572,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
                     }
                 }
             }
+            if (FSYNC && s >= 2) wait_read((uint32_t) s - 1u);
 #pragma unroll
             for (int h = 0; h < 2; ++h)
                 *(uint4*) &Wsm[s & 1][rr][16 * jb + 8 * h] = make_uint4(cvt_pk_bf16(f[h][0], f[h][1]), cvt_pk_bf16(f[h][2], f[h][3]),
@@ -528,7 +588,8 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
             lookup(rec[(u + 1) % RECD], look[(u + 1) & 1]);   // the next step's table reads travel under this step's decode
             produce(s, rec[u], look[u & 1]);
             load_rec(s + RECD, rec[u]);
-            lds_barrier();
+            if (FSYNC) post(wv - NCW, (uint32_t) s + 1u);
+            else lds_barrier();
         };
         // whole rounds of the record ring in a loop with one way out (a conditional exit per step costs the loop a
         // register move per record word and step), the steps left over after it
@@ -549,10 +610,11 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     // ---- consumer side ---------------------------------------------------------------------------------------------------
     const int wtok = wv * 32 * CT;          // this wave's first token of the tile
     if (wtok >= count) {                    // a wave whose tokens are all padding has nothing to multiply
-        for (int s = 0; s < nsteps; ++s) lds_barrier();
+        if (FSYNC) post(4, 0x7FFFFFFFu);
+        else for (int s = 0; s < nsteps; ++s) lds_barrier();
         return;
     }
-    __builtin_amdgcn_s_setprio(2);   // the matrix pipeline's instruction stream goes first when both roles are ready
+    __builtin_amdgcn_s_setprio(FSYNC ? 3 : 2);   // the matrix pipeline's instruction stream goes first when both roles are ready
     f32x16 acc[CT][2];
 #pragma unroll
     for (int m = 0; m < CT; ++m)
@@ -589,12 +651,14 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     // One weight step: chunk m multiplies out of fragment set (m even ? fa : fb) while the next chunk's fragments travel
     // into the other set; with MT odd the sets have swapped roles when the step ends.
     auto step = [&](int s, bf16x8 (&fa)[4], bf16x8 (&fb)[4]) {
-        lds_barrier();   // weight step s is in tile s & 1
+        if (FSYNC) wait_written((uint32_t) s + 1u);
+        else lds_barrier();   // weight step s is in tile s & 1
         bf16x8 bq[4][2];
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
             for (int n = 0; n < 2; ++n) bq[kk][n] = *(const bf16x8*) &Wsm[s & 1][32 * n + frow][16 * kk + 8 * fhi];
+        if (FSYNC) post(4, (uint32_t) s + 1u);
 #pragma unroll
         for (int m = 0; m < CT; ++m) {
             const int c = s * CT + m;

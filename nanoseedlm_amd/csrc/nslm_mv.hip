@@ -444,11 +444,11 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
             }
         };
         const int rstep = (int) gridDim.x * 4;
-        int rr = (int) blockIdx.x * 4 + wv, j0 = lane, r = 0, job = 0;
+        int rr = (int) blockIdx.x * 4 + wv, jb = 0, r = 0, job = 0;   // the piece in hand: row, first block (the same for all lanes)
         WideRaw<FMT> na[4], nb[4];
         if (rr < total) {
             row_of(rr, r, job);
-            request(na, nb, r, j0);
+            request(na, nb, r, lane);
         }
         for (int i = tid; i < a.K / 4; i += 256) ((float4*) xw)[i] = ((const float4*) xrow)[i];
         __syncthreads();
@@ -460,15 +460,15 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
                 ca[u] = na[u];
                 cb[u] = nb[u];
             }
-            const int r_now = r, job_now = job, j_now = j0;
-            j0 += 256;
-            const bool row_done = j0 >= nbk;
+            const int r_now = r, job_now = job, j_now = jb + lane;
+            jb += 256;
+            const bool row_done = jb >= nbk;   // (for the wave, not the lane: the sums below are the whole wave's)
             if (row_done) {
                 rr += rstep;
-                j0 = lane;
+                jb = 0;
                 if (rr < total) row_of(rr, r, job);
             }
-            if (rr < total) request(na, nb, r, j0);
+            if (rr < total) request(na, nb, r, jb + lane);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {   // the piece's arithmetic, in block order
                 const int j = j_now + 64 * u;

@@ -131,8 +131,9 @@ def test_heads_deq(be, oracle):
 # ---- matvec family ------------------------------------------------------------------------------------------------------------
 
 # K: 256 / 512 the reference's cases (tests/test_mova_kernels.c:161); 768 and 2880 rows whose chunk count is not a power
-# of two (LDS row sums); 2048 / 4096 the benchmark shapes; 136 not a multiple of 64 (generic path)
-@pytest.mark.parametrize("K", [256, 512, 768, 2880, 2048, 4096, 136])
+# of two (LDS row sums); 2048 / 4096 the benchmark shapes; 136 not a multiple of 64 (generic path); 4480 = 560 blocks, whose third
+# piece of 256 ends inside a wave (the wide matvec's row ends for the wave, not for a lane)
+@pytest.mark.parametrize("K", [256, 512, 768, 2880, 2048, 4096, 136, 4480])
 @pytest.mark.parametrize("fmt", ALL_FMT)
 def test_mv_dense_gather_gateup(be, oracle, fmt, K):
     if fmt in (packs.MF_Q4, packs.MF_Q8) and K % 64:
