@@ -390,6 +390,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
     // 627 -> 609; with no hand-over at all and garbage computed: 247 and 540).  The dense 512-token GEMM with its eight consumer
     // waves is indifferent to the barrier and keeps it.
     constexpr bool FSYNC = NCW == 1;
+    constexpr int NWT = FSYNC && XCH == 2 ? 3 : 2;   // weight tiles in LDS: a third one where the activation ring leaves room for it
     __shared__ __attribute__((aligned(16))) uint32_t flg[8];
     const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool producer = wv >= NCW;
@@ -572,10 +573,10 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
                     }
                 }
             }
-            if (FSYNC && s >= 2) wait_read((uint32_t) s - 1u);
+            if (FSYNC && s >= NWT) wait_read((uint32_t) (s - NWT + 1));
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                *(uint4*) &Wsm[s & 1][rr][16 * jb + 8 * h] = make_uint4(cvt_pk_bf16(f[h][0], f[h][1]), cvt_pk_bf16(f[h][2], f[h][3]),
+                *(uint4*) &Wsm[NWT == 2 ? s & 1 : s % NWT][rr][16 * jb + 8 * h] = make_uint4(cvt_pk_bf16(f[h][0], f[h][1]), cvt_pk_bf16(f[h][2], f[h][3]),
                                                                        cvt_pk_bf16(f[h][4], f[h][5]), cvt_pk_bf16(f[h][6], f[h][7]));
         };
         MmRec2 rec[RECD] = {};
@@ -657,7 +658,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-            for (int n = 0; n < 2; ++n) bq[kk][n] = *(const bf16x8*) &Wsm[s & 1][32 * n + frow][16 * kk + 8 * fhi];
+            for (int n = 0; n < 2; ++n) bq[kk][n] = *(const bf16x8*) &Wsm[NWT == 2 ? s & 1 : s % NWT][32 * n + frow][16 * kk + 8 * fhi];
         if (FSYNC) post(4, (uint32_t) s + 1u);
 #pragma unroll
         for (int m = 0; m < CT; ++m) {
@@ -720,7 +721,7 @@ __global__ void __launch_bounds__(64 * (NCW + 4)) k_mm_stream(MmArgs a, WSlice w
         }
 }
 template <int NCW, int XCH>
-constexpr size_t mm_stream_lds() { return (size_t) (NCW * XCH * XCHUNK + 2 * BM * LDW2) * sizeof(uint16_t); }
+constexpr size_t mm_stream_lds() { return (size_t) (NCW * XCH * XCHUNK + (NCW == 1 && XCH == 2 ? 3 : 2) * BM * LDW2) * sizeof(uint16_t); }
 // the streamed kernel takes BF16 activations in 16-byte aligned rows, one BF16 term per weight, K in whole weight steps
 // (xrows > 0: the row count, for the variants that address rows by 32-bit byte offsets)
 bool stream_ok(int fmt, int K, int xs, const void* x, long long xrows) {
@@ -773,7 +774,11 @@ void mm_grouped(hipStream_t st, int fmt, const WSlice* ws, int K, int R, const v
         // grouped tiles are mostly a few pairs of one expert: decode-bound, so a short ring buys two workgroups a CU - and
         // where the caller knows that no tile holds more than 32 pairs, one multiplying wave instead of four buys four
         const dim3 grid((unsigned) (R + BM - 1) / BM, (unsigned) grid_tiles, ws2 ? 2u : 1u);
-        if (tile_rows <= 32) launch_mm_stream<1, 1, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
+        // (one multiplying wave: four workgroups a CU fit either three weight tiles and a ring of two activation chunks or two and
+        // three.  C2 at 32 rows, P = 4: 260.3 against 263.5 us; C3 at 16 rows, P = 3, whose steps are shorter than an activation
+        // chunk's way from memory: 620 against 609; three and three, three workgroups a CU: 265.2 and 615.6)
+        if (tile_rows <= 32 && fmt == MF_SEED4P4) launch_mm_stream<1, 1, 2>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
+        else if (tile_rows <= 32) launch_mm_stream<1, 1, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
         else launch_mm_stream<1, 4, 3>(st, fmt, a, none, ws, x, y, perm, tiles, ntiles, grid);
         return;
     }
