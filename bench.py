@@ -262,7 +262,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
                                frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
                                kernel=("k_moe_decode_grouped (one launch per step)" if T <= 24 and name[:2] == "c2" else
-                                       "k_mm_stream<1, %d, 3> grouped (two launches of the step: gate + up + SwiGLU, down; with its glue kernels)" % (1 if T <= 32 else 4)),
+                                       "k_mm_stream<1, %d, %d> grouped (two launches of the step: gate + up + SwiGLU, down; with its glue kernels)" % (1 if T <= 32 else 4, 2 if T <= 32 and name[:2] == "c2" else 3)),
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, **counters_of(name))
     desc = {"c2": "C2 MoE decode layer step: 128 experts seeded P=4, top-8 softmax, hidden 2048, intermediate 768",
             "c3": "C3 mixed-format layer step: 64 experts seeded P=3, top-4, hidden 2880, intermediate 2880, plus seven 2880 x 2880 Q4-g64 projections (q, k, v, o, shared gate / up / down)"}[name[:2]]

@@ -835,7 +835,8 @@ int kc_mm_grouped_swiglu(kc_stream_t s, int fmt, const WSlice* gate, const WSlic
     MmArgs a = {K, R, 0, xs, ys, xdiv, 0, 0, up, nullptr, a16};
     WSlice none = {};
     const dim3 grid((unsigned) (R + BM / 2 - 1) / (BM / 2), (unsigned) max_tiles);
-    if (tile_rows >= 1 && tile_rows <= 32) launch_mm_stream<1, 1, 3>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);
+    if (tile_rows >= 1 && tile_rows <= 32 && fmt == MF_SEED4P4) launch_mm_stream<1, 1, 2>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);   // (as in mm_grouped)
+    else if (tile_rows >= 1 && tile_rows <= 32) launch_mm_stream<1, 1, 3>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);
     else launch_mm_stream<1, 4, 3>((hipStream_t) s, fmt, a, none, gate, x, nullptr, perm, tiles, nt, grid);
     return 0;
 }
