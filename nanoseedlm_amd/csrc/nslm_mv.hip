@@ -41,6 +41,7 @@ struct MvArgs {
     const float* nw;      // non-null (dense modes): x is normalised first, xn_k = x_k r (1 + nw_k), r = rsqrt(mean(x^2) + neps)
     float neps;
     int ttot;             // dense modes with NT > 1: tokens of the launch; workgroup row blockIdx.y takes tokens NT y .. (nt = NT)
+    int trun;             // k_mv_wide, dense, ttot > 0: tokens a workgroup row takes (0: MV_MAXT)
                           // (last, so that the one-token kernels read their arguments where they always did: a field
                           // added in the middle cost them a second round of argument loads, 0.3 us a launch)
     uint16_t* px;         // k_mv_wide, dense: non-null = the staged rows also leave as BF16 bits [token][K] (the batched GEMMs' view)
@@ -412,9 +413,10 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
         if (MODE == GATEUP) wB = a.wu[sl];
     }
     // dense launches of more than MV_MAXT tokens (ttot > 0): the tokens are dealt to grid.y in runs of MV_MAXT
-    const int tg0 = (MODE == DENSE && a.ttot > 0) ? (int) blockIdx.y * MV_MAXT : 0;
+    const int trun = a.trun ? a.trun : MV_MAXT;
+    const int tg0 = (MODE == DENSE && a.ttot > 0) ? (int) blockIdx.y * trun : 0;
     const float* xrow = a.x + (size_t) (DNW ? tg0 : pair / a.xdiv) * a.xs;
-    const int nbk = a.K / 8, nt = !DNW ? 1 : (MODE == DENSE && a.ttot > 0) ? min(MV_MAXT, a.ttot - tg0) : a.nt;
+    const int nbk = a.K / 8, nt = !DNW ? 1 : (MODE == DENSE && a.ttot > 0) ? min(trun, a.ttot - tg0) : a.nt;
     bool alA = ((uintptr_t) wA.p[0] & 15u) == 0;
     const bool alB = ((uintptr_t) wB.p[0] & 15u) == 0;
     int total = a.R;
@@ -709,6 +711,14 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
 
 void note_launch() { nslm::host_note_launch(); }
 
+// Tokens a workgroup row of a wave-a-row dense launch takes: MV_MAXT, fewer while the rows alone do not fill the chip twice (a router's
+// 128 rows at 32 tokens: 128 workgroups that each stage 64 KB of activations took 9.3 us; a token's result does not depend on its run)
+int wide_run(int R, int T) {
+    int run = MV_MAXT;
+    while (run > 2 && (long) ((R + 3) / 4) * ((T + run - 1) / run) < 2L * cu_count()) run /= 2;
+    return run;
+}
+
 #define MV_TG 4   // tokens a workgroup of the multi-token fast path stages in LDS
 #define MV_MULTI_MAXT 64
 
@@ -775,9 +785,10 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
     // not depend on the run it is in): for the wave-a-row kernel the runs of one launch, dealt to grid.y.
     if (T > MV_MAXT && wide_ok(fmt, K, x, xs, MV_MAXT)) {
         MvArgs b = a;
-        b.nt = MV_MAXT;   // (sizes the staging)
+        b.trun = wide_run(R, T);
+        b.nt = b.trun;   // (sizes the staging)
         b.ttot = T;
-        launch_wide<DENSE>(st, fmt, b, (T + MV_MAXT - 1) / MV_MAXT);
+        launch_wide<DENSE>(st, fmt, b, (T + b.trun - 1) / b.trun);
         note_launch();
         return;
     }
@@ -796,10 +807,11 @@ int kc_mv_pack(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, i
     if (T < 1 || T > MV_MULTI_MAXT || R < 1 || !wide_ok(fmt, K, x, xs, T < MV_MAXT ? T : MV_MAXT) || !aligned16(px)) return -1;
     MvArgs a = {};
     a.wd = w; a.x = x; a.y = y; a.K = K; a.R = R; a.xdiv = 1; a.xs = xs; a.ys = ys; a.f32out = g_store_f32;
-    a.nt = T < MV_MAXT ? T : MV_MAXT;
+    a.trun = wide_run(R, T);
+    a.nt = T < a.trun ? T : a.trun;
     a.ttot = T;
     a.px = px;
-    launch_wide<DENSE>((hipStream_t) s, fmt, a, (T + MV_MAXT - 1) / MV_MAXT);
+    launch_wide<DENSE>((hipStream_t) s, fmt, a, (T + a.trun - 1) / a.trun);
     note_launch();
     return 0;
 }
