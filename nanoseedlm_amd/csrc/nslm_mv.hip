@@ -124,6 +124,11 @@ __global__ void __launch_bounds__(NTHR) k_mv_seed(MvArgs a) {
         const WSlice& w = (MODE == GATEUP && (vc & 1)) ? wB : wA;
         return load_chunk<P>(w, (uint32_t) r * (uint32_t) L + (uint32_t) ch);
     };
+    // (Half the waves ask a moment later.  With all 9.4 MB of a 4096 x 4096 matrix requested in the same instant - one workgroup of 16
+    // waves a CU, every wave one chunk of records - the launch took 8.5 us; with the requests in two waves of arrivals, 64 clocks
+    // apart (any split of the waves does, longer pauses do less), the first records are back sooner and the launch takes 7.8.  The
+    // smaller workgroups of the other shapes gain a few tenths of a percent.)
+    if ((tid >> 6) >= NTHR / 128) __builtin_amdgcn_s_sleep(1);
     Chunk cur = fetch(v);
     loads_issued();
     if (NT == 1) {
