@@ -68,8 +68,8 @@ def fail_on_kernel_error(st=None):
 class Q4Projections:
     """Config 3's affine-int4 side of the layer: q / k / v / o and the shared expert's gate / up / down, each d x d, Q4
     group 64 (BF16 scale ~U(0.005, 0.02), zero point uniform [0, 15] stored as bias = -z * scale).  The benchmark definition gives no
-    shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs up to 8 tokens, the packed
-    MFMA GEMM above (as the reference's enc_dense / enc_dense_packed choose, engine/mova_cuda.c:1020-1028)."""
+    shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs up to 16 tokens, the packed
+    MFMA GEMM above (the reference's enc_dense / enc_dense_packed change over at 8, engine/mova_cuda.c:1020-1028)."""
 
     def __init__(self, rng, n_layers, d, T):
         from nanoseedlm_amd import backend, moe, packs
@@ -103,7 +103,7 @@ class Q4Projections:
         from nanoseedlm_amd import packs
         L, d, T, Q4 = self.L, self.d, self.T, packs.MF_Q4
         arr, tab = self.layers[layer]
-        if T <= 8:
+        if T <= 16:   # (up to 16 rows the matvecs are ahead of the GEMMs on these 2880 x 2880 matrices: 19 against 23 us a projection at 16)
             # q, k, v over the same input: one launch (kc_mv_multi; the same bits as one kc_mv each), else the three launches
             if L.kc_mv_multi(stream, Q4, 3, arr, self.R3, self.y3, self.R3, self.add3, d, x_ptr, d, T, None, C.c_float(0.0)):
                 for i, y in enumerate((self.q, self.kk, self.v)):

@@ -327,6 +327,7 @@ __global__ void __launch_bounds__(256) k_mv_any(int fmt, MvArgs a) {
 // xor-shuffle sum), hence the same bits - but the activations are staged once per workgroup in LDS instead of being
 // re-read from global memory for every row, a block's weights arrive as one 16 / 8 / 4-byte load, a wave walks its rows
 // with a grid stride and keeps the loads of four blocks in flight, and many small workgroups share a CU.
+#define WIDE_RB 2   // rows a wave of a several-token dense launch takes at a time
 template <int FMT>
 struct WideRaw {
     uint4 q;         // BF16: 8 weights; Q8: q.xy; Q4: q.x
@@ -529,6 +530,65 @@ __global__ void __launch_bounds__(256) k_mv_wide(MvArgs a) {
             ((uint4*) (a.px + (size_t) (tg0 + t) * a.K))[j] = make_uint4(pack_bf2(q0.x, q0.y), pack_bf2(q0.z, q0.w), pack_bf2(q1.x, q1.y), pack_bf2(q1.z, q1.w));
         }
     }
+    if (MODE == DENSE && nt > 1) {
+        // Several tokens: a wave takes WIDE_RB rows at a time, so a block's activations are read from LDS once for the four rows'
+        // multiply-adds.  (A row at a time, 16 tokens on 2880 x 2880 in Q4 read 0.5 GB from LDS and took 24 us; the LM head at 8
+        // tokens was bound by those reads, not by HBM.)  Per (row, token) the blocks still add up in the one-row order.
+        for (int rg = ((int) blockIdx.x * 4 + wv) * WIDE_RB; rg < total; rg += (int) gridDim.x * 4 * WIDE_RB) {
+            float acc[WIDE_RB][MV_MAXT];
+#pragma unroll
+            for (int rb = 0; rb < WIDE_RB; ++rb)
+#pragma unroll
+                for (int t = 0; t < MV_MAXT; ++t) acc[rb][t] = 0.0f;
+            for (int j0 = lane; j0 < nbk; j0 += 128) {   // two blocks of each row in flight, then their arithmetic in block order
+                WideRaw<FMT> ra[WIDE_RB][2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int j = j0 + 64 * u;
+                    if (j < nbk) {
+#pragma unroll
+                        for (int rb = 0; rb < WIDE_RB; ++rb) ra[rb][u] = wide_load<FMT>(wA, min(rg + rb, total - 1), a.K, j, alA);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const int j = j0 + 64 * u;
+                    if (j >= nbk) break;
+                    float w[WIDE_RB][8];
+#pragma unroll
+                    for (int rb = 0; rb < WIDE_RB; ++rb) wide_weights<FMT>(ra[rb][u], w[rb]);
+#pragma unroll
+                    for (int t = 0; t < MV_MAXT; ++t) {
+                        if (t >= nt) break;
+                        const float* xb = xw + (size_t) t * a.K + (size_t) j * 8;
+                        const float4 x0 = *(const float4*) xb, x1 = *(const float4*) (xb + 4);
+#pragma unroll
+                        for (int rb = 0; rb < WIDE_RB; ++rb) {   // (wide_dot's chain of operations)
+                            float d = w[rb][0] * x0.x;
+                            d = fmaf(w[rb][1], x0.y, d);
+                            d = fmaf(w[rb][2], x0.z, d);
+                            d = fmaf(w[rb][3], x0.w, d);
+                            d = fmaf(w[rb][4], x1.x, d);
+                            d = fmaf(w[rb][5], x1.y, d);
+                            d = fmaf(w[rb][6], x1.z, d);
+                            d = fmaf(w[rb][7], x1.w, d);
+                            acc[rb][t] = fmaf(d, 1.0f, acc[rb][t]);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int rb = 0; rb < WIDE_RB; ++rb)
+#pragma unroll
+                for (int t = 0; t < MV_MAXT; ++t) {
+                    if (t >= nt) break;
+                    float sum = acc[rb][t];
+                    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+                    if (lane == 0 && rg + rb < total) store_y(a.y + (size_t) (tg0 + t) * a.ys + rg + rb, sum, a.add, a.f32out);
+                }
+        }
+        return;
+    }
     for (int rr = (int) blockIdx.x * 4 + wv; rr < total; rr += (int) gridDim.x * 4) {
         int r = rr, job = 0;
         if (MODE == MULTI) {   // the matrix this row belongs to (the rows of the matrices follow each other)
@@ -689,7 +749,8 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
         rows = 0;
         for (int j = 0; j < a.nj; ++j) rows += a.Rj[j];
     }
-    int gx = (rows + 3) / 4;
+    const int per_wg = MODE == DENSE && a.nt > 1 ? 4 * WIDE_RB : 4;   // (several tokens: a wave takes WIDE_RB rows at a time)
+    int gx = (rows + per_wg - 1) / per_wg;
     const int cap = (8 * cu_count() + ny - 1) / ny;
     if (gx > cap) gx = cap < 1 ? 1 : cap;
     const dim3 grid((unsigned) gx, (unsigned) ny);
@@ -716,11 +777,18 @@ void launch_wide(hipStream_t st, int fmt, const MvArgs& a, int ny) {
 
 void note_launch() { nslm::host_note_launch(); }
 
-// Tokens a workgroup row of a wave-a-row dense launch takes: MV_MAXT, fewer while the rows alone do not fill the chip twice (a router's
-// 128 rows at 32 tokens: 128 workgroups that each stage 64 KB of activations took 9.3 us; a token's result does not depend on its run)
-int wide_run(int R, int T) {
-    int run = MV_MAXT;
-    while (run > 2 && (long) ((R + 3) / 4) * ((T + run - 1) / run) < 2L * cu_count()) run /= 2;
+// Tokens a workgroup row of a wave-a-row dense launch takes (a token's result does not depend on its run): MV_MAXT at most; fewer
+// while the rows alone do not fill the chip twice (a router's 128 rows at 32 tokens: 128 workgroups that each stage 64 KB of
+// activations took 9.3 us); and, for a matrix small enough to be re-read from the caches by every run, few enough that several
+// workgroups share a CU's LDS (eight rows of 2880 are 92 KB: one workgroup a CU).
+int wide_run(int fmt, int K, int R, int T) {
+    int run = T < MV_MAXT ? T : MV_MAXT;
+    // (workgroups of a launch: four waves of WIDE_RB rows each, of one row where the run is a single token)
+    auto wgs = [&](int run_) { const int per = run_ > 1 ? 4 * WIDE_RB : 4; return (long) ((R + per - 1) / per) * ((T + run_ - 1) / run_); };
+    while (run > 1 && wgs(run) < 2L * cu_count()) run /= 2;
+    const double bytes = (double) R * K * (fmt == MF_BF16 ? 2.0 : fmt == MF_Q8 ? 1.0625 : 0.5625);
+    if (bytes <= 16e6)
+        while (run > 1 && (size_t) run * K * sizeof(float) > 48 * 1024) run = (run + 1) / 2;
     return run;
 }
 
@@ -786,11 +854,11 @@ void kc_mv(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, int x
         note_launch();
         return;
     }
-    // Every other shape: the kernels' token loops hold MV_MAXT tokens, so more rows go in runs of MV_MAXT (a token's result does
-    // not depend on the run it is in): for the wave-a-row kernel the runs of one launch, dealt to grid.y.
-    if (T > MV_MAXT && wide_ok(fmt, K, x, xs, MV_MAXT)) {
+    // Every other shape: the kernels' token loops hold MV_MAXT tokens, so more rows go in runs (a token's result does not depend on
+    // the run it is in): for the wave-a-row kernel the runs of one launch, dealt to grid.y.
+    if (T > 1 && wide_ok(fmt, K, x, xs, T < MV_MAXT ? T : MV_MAXT)) {
         MvArgs b = a;
-        b.trun = wide_run(R, T);
+        b.trun = wide_run(fmt, K, R, T);
         b.nt = b.trun;   // (sizes the staging)
         b.ttot = T;
         launch_wide<DENSE>(st, fmt, b, (T + b.trun - 1) / b.trun);
@@ -812,7 +880,7 @@ int kc_mv_pack(kc_stream_t s, int fmt, WSlice w, int K, int R, const float* x, i
     if (T < 1 || T > MV_MULTI_MAXT || R < 1 || !wide_ok(fmt, K, x, xs, T < MV_MAXT ? T : MV_MAXT) || !aligned16(px)) return -1;
     MvArgs a = {};
     a.wd = w; a.x = x; a.y = y; a.K = K; a.R = R; a.xdiv = 1; a.xs = xs; a.ys = ys; a.f32out = g_store_f32;
-    a.trun = wide_run(R, T);
+    a.trun = wide_run(fmt, K, R, T);
     a.nt = T < a.trun ? T : a.trun;
     a.ttot = T;
     a.px = px;
@@ -825,6 +893,16 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
                 const float* x, int xs, int T, const float* norm_w, float norm_eps) {
     if (n >= 1 && n <= MV_MAXJ && T >= 1 && T <= MV_MAXT && !norm_w && wide_ok(fmt, K, x, xs, T)) {
         // BF16 / Q8 / Q4: a wave a row, the rows of the n matrices one after the other (the same row sums as kc_mv's)
+        if (T > 1 && (size_t) T * K * sizeof(float) > 48 * 1024) {
+            // several tokens of long rows: one dense launch a matrix, whose token runs keep several workgroups on a CU (eight tokens
+            // of 2880 are 92 KB of staged activations - one workgroup a CU, and 91 us for three 2880 x 2880 matrices in Q4
+            // against 11 us a dense launch)
+            for (int j = 0; j < n; ++j) {
+                if (R[j] < 1) return -1;
+                kc_mv(s, fmt, w[j], K, R[j], x, xs, y[j], ys[j], T, add[j], nullptr);
+            }
+            return 0;
+        }
         MvArgs a = {};
         a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.nj = n; a.nt = T;
         for (int j = 0; j < n; ++j) {
