@@ -454,7 +454,7 @@ def dense_workload(name, steps, warmup, matrices=64):
         resident = dict(launch_us=rms * 1e3, achieved=bytes_step / rms / 1e6, frac=bytes_step / rms / 1e6 / HBM_PEAK_GBS, matrices=1)
     if bound == "hbm":
         res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s",
-                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_mv_seed<dense>" if name == "c0" else "k_deq",
+                               frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS, kernel="k_mv_seed<dense>" if name == "c0" else "k_deq_seed",
                                launch_us=ms * 1e3, algorithmic_bytes=bytes_step, cache_resident=resident, **counters_of(name))
     else:
         res["roofline"] = dict(bound="mfma", achieved=flops / ms / 1e9, peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s",

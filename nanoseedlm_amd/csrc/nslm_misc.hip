@@ -454,6 +454,46 @@ __global__ void __launch_bounds__(512) k_slots_copy(CachePool p) {
 
 // ---- weights to BF16 bits: one thread per 8-weight block ---------------------------------------------------------------
 // heads: W.p[2] holds an int32 exponent bias per head (SEED4P4 per-head maps); otherwise the slice's own eb.
+#define DEQ_NB 8   // blocks a thread of the seed formats' path takes
+__device__ __forceinline__ uint32_t deq_pk_bf16(float lo, float hi) {   // v_cvt_pk_bf16_f32: both round to nearest even
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+// The seed formats, 16-byte aligned output: a thread takes DEQ_NB blocks (block wg * 256 * DEQ_NB + k * 256 + tid, so a wave's
+// accesses are consecutive), all their records requested before the first is expanded, a block's eight BF16 values leaving as one
+// 16-byte store.  (A block a thread with the tables loaded for every 256 blocks and eight 2-byte stores: 164 instructions a block.)
+template <int P>
+__global__ void __launch_bounds__(256) k_deq_seed(WSlice W, int rows_per_head, int K, int nblocks, int heads, uint16_t* out) {
+    __shared__ uint32_t tab[NSLM_TAB_WORDS];
+    load_tables(tab);
+    const int nbk = K / 8, b0 = (int) blockIdx.x * 256 * DEQ_NB + (int) threadIdx.x;
+    uint32_t seed[DEQ_NB], word[DEQ_NB], cb[DEQ_NB];
+    int eb[DEQ_NB];
+#pragma unroll
+    for (int k = 0; k < DEQ_NB; ++k) {   // (clamped: the loads stay unconditional)
+        const int b = min(b0 + 256 * k, nblocks - 1);
+        seed[k] = gp<uint16_t>(W.p[0])[b];
+        word[k] = gp<uint16_t>(W.p[1])[b];
+        cb[k] = P == 4 ? gp<uint8_t>(W.p[3])[b >> 1] : 0u;
+        eb[k] = heads ? gp<int32_t>(W.p[2])[(b / nbk) / rows_per_head] : W.eb;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < DEQ_NB; ++k) {
+        const int b = b0 + 256 * k;
+        if (b >= nblocks) break;
+        int is[8];
+        block_isum<P>(tab, seed[k], word[k], is);
+        const int code = P == 4 ? (int) ((cb[k] >> ((b & 1) * 4)) & 15u) : (int) (word[k] & 15u);
+        const float sc = pow2f(eb[k] + code) * NSLM_R32;   // exact: a power-of-two scaling of R32
+        float o[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o[c] = (float) is[c] * sc;
+        *(uint4*) (out + (size_t) b * 8) = make_uint4(deq_pk_bf16(o[0], o[1]), deq_pk_bf16(o[2], o[3]), deq_pk_bf16(o[4], o[5]), deq_pk_bf16(o[6], o[7]));
+    }
+}
 __global__ void __launch_bounds__(256) k_deq(int fmt, WSlice W, int rows_per_head, int K, int nblocks, int heads, uint16_t* out) {
     __shared__ uint32_t tab[NSLM_TAB_WORDS];
     load_tables(tab);
@@ -492,6 +532,17 @@ __global__ void __launch_bounds__(256) k_deq(int fmt, WSlice W, int rows_per_hea
     uint16_t* dst = out + (size_t) b * 8;
 #pragma unroll
     for (int c = 0; c < 8; ++c) dst[c] = (uint16_t) tobf(o[c]);
+}
+
+void launch_deq(hipStream_t st, int fmt, WSlice W, int rows_per_head, int K, int nb, int heads, uint16_t* out) {
+    const bool seed = fmt == MF_SEED4P4 || fmt == MF_SEED4;
+    if (seed && ((uintptr_t) out & 15u) == 0) {
+        const dim3 grid((unsigned) ((nb + 256 * DEQ_NB - 1) / (256 * DEQ_NB)));
+        if (fmt == MF_SEED4P4) hipLaunchKernelGGL(k_deq_seed<4>, grid, dim3(256), 0, st, W, rows_per_head, K, nb, heads, out);
+        else hipLaunchKernelGGL(k_deq_seed<3>, grid, dim3(256), 0, st, W, rows_per_head, K, nb, heads, out);
+        return;
+    }
+    hipLaunchKernelGGL(k_deq, dim3((unsigned) (nb + 255) / 256), dim3(256), 0, st, fmt, W, rows_per_head, K, nb, heads, out);
 }
 
 }   // namespace
@@ -574,13 +625,12 @@ void kc_heads_deq(kc_stream_t s, int fmt, WSlice W, const uint32_t* G, int H, in
     (void) G;
     const int nb = H * O * (I / 8);
     if (nb < 1) return;
-    hipLaunchKernelGGL(k_deq, dim3((unsigned) (nb + 255) / 256), dim3(256), 0, (hipStream_t) s, fmt, W, O, I, nb,
-                       fmt == MF_SEED4P4 ? 1 : 0, out);
+    launch_deq((hipStream_t) s, fmt, W, O, I, nb, fmt == MF_SEED4P4 ? 1 : 0, out);
 }
 void kc_slice_deq(kc_stream_t s, int fmt, WSlice w, int K, int R, uint16_t* out) {
     const int nb = R * (K / 8);
     if (nb < 1) return;
-    hipLaunchKernelGGL(k_deq, dim3((unsigned) (nb + 255) / 256), dim3(256), 0, (hipStream_t) s, fmt, w, R, K, nb, 0, out);
+    launch_deq((hipStream_t) s, fmt, w, R, K, nb, 0, out);
 }
 
 }   // extern "C"
