@@ -36,8 +36,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 COUNTERS = "profiles/traffic.json"
 # Untimed steps before the W warmup steps: a fresh GPU reaches its steady clocks only after a few hundred milliseconds of work
-# (the same 400 timed steps: 23.8 us a step after 50 warmup steps, 22.9 after 4000), and a short run would measure the ramp.
-PREWARM_S = 0.3
+# (the same 400 timed steps: 23.8 us a step after 50 warmup steps, 22.9 after 4000; a box that had just been handed out once
+# read 22.5 us behind 0.3 s of it where the next runs read 19.9), and a short run would measure the ramp.
+PREWARM_S = 1.0
 
 
 def counters_of(workload):
