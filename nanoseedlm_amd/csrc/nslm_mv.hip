@@ -923,7 +923,10 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     a.x = x; a.K = K; a.xdiv = 1; a.xs = xs; a.f32out = g_store_f32; a.L = L; a.rpi = rpi; a.nj = n; a.nw = norm_w; a.neps = norm_eps;
     int total = 0;
     for (int j = 0; j < n; ++j) total += R[j];
-    a.rows_per_wg = pick_rows_per_wg(total, rpi, 1);
+    // (one token: the workgroup size kc_mv's one-token launches take for as many rows)
+    const int nthr = T == 1 ? pick_threads(total, L, shfl) : 256;
+    if (T == 1) a.rpi = nthr / L;
+    a.rows_per_wg = pick_rows_per_wg(total, a.rpi, 1, nthr);
     for (int j = 0; j < n; ++j) {
         if (R[j] < 1) return -1;
         a.wj[j] = w[j]; a.Rj[j] = R[j]; a.ysj[j] = ys[j]; a.addj[j] = add[j];
@@ -934,7 +937,7 @@ int kc_mv_multi(kc_stream_t s, int fmt, int n, const WSlice* w, const int* R, fl
     if (T == 1) {
         a.nt = 1;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
-        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, (size_t) L * xpad_of(fmt) * sizeof(float));
+        launch_seed_fmt<MULTI, 1>(st, fmt, a, shfl, grid, (size_t) L * xpad_of(fmt) * sizeof(float), nthr);
     } else {   // runs of MV_TG tokens over grid.y, as kc_mv's
         a.ttot = T;
         for (int j = 0; j < n; ++j) a.yj[j] = y[j];
