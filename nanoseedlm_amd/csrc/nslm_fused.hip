@@ -779,12 +779,12 @@ bool shape_of(int K, bool gateup, int* L, int* rpi, bool* shfl) {
 // other (an item's set-up priced at a third of an iteration, unequal items at half an iteration: workgroups i, i + 256, ...
 // share a CU, so the long items of a regular pattern meet on the same CUs); up to `slack` items more than the workgroups still
 // count as one round.
-int pick_one_round(int units, int iters, int gmax, int nmax, int slack = 0) {
+int pick_one_round(int units, int iters, int gmax, int nmax, int slack = 0, int setup = 2) {
     int best = 1;
     long best_cost = -1;
     for (int n = 1; n <= iters && n <= nmax; ++n) {
         const long over = (long) units * n - slack, rounds = over <= gmax ? 1 : (over + gmax - 1) / gmax, per = (iters + n - 1) / n;
-        const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + 2);
+        const long cost = rounds * (6 * per + (iters % n ? 3 : 0) + setup);
         if (best_cost < 0 || cost <= best_cost) { best = n; best_cost = cost; }   // ties: more, shorter items
     }
     return best;
@@ -849,7 +849,9 @@ int launch_fused(hipStream_t st, FusedArgs& a, bool sg, bool sd, size_t lds) {
     // through LDS (C3) one round stayed ahead.
     const int gmax = (per_cu < 5 ? per_cu : 5) * cu_count(), P_ = a.T * a.kk;
     a.ntile_g = few || !sg ? pick_one_round(P_, a.it_g, gmax, FUSED_TILES) : pick_by_cu_load(P_, a.it_g, cu_count(), FUSED_TILES);
-    a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES);
+    // (a down item's set-up - the wait for its pair, the staging of A - priced at two thirds of an iteration: at a third, six
+    // tokens of C2 took two rounds of 49 two-iteration items a pair, 81.6 us, where one round of 26 takes 76.5)
+    a.ntile_d = pick_one_round(P_, a.it_d, gmax, FUSED_TILES, 0, 4);
     if (a.ntile_g < gu_min_tiles(a)) a.ntile_g = gu_min_tiles(a);
     if ((long) ((a.it_g + a.ntile_g - 1) / a.ntile_g) * a.rpig / 2 > GU_ROWS) return -1;
     const long items = (long) P_ * (a.ntile_g > a.ntile_d ? a.ntile_g : a.ntile_d);
