@@ -73,7 +73,8 @@ struct CuParams {
     FastDiv by_tpp, by_rpc, by_Ld, by_Lg, by_nbp, by_kk, by_E;
 };
 
-template <int P, bool SHFL_G, bool SHFL_D, int NTHR>
+// NORM: the launch normalises its input (a.nw); launches that do not are compiled without what that path adds.
+template <int P, bool SHFL_G, bool SHFL_D, int NTHR, bool NORM>
 __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c) {
     constexpr int NW = NTHR / 64, XP = xpad<P>();
     extern __shared__ __attribute__((aligned(16))) float dyn[];
@@ -106,6 +107,16 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     const int piece = min(tid, per - 1);
     const uint4 pw0 = ((const uint4*) a.gate)[piece], pw1 = ((const uint4*) a.up)[piece], pw2 = ((const uint4*) a.down)[piece];
     loads_issued();
+    // With a norm, this CU's router rows - the operand of a logit that comes from HBM - are requested before the rows' scales are
+    // formed, not behind their two barriers (the inputs and the norm weights, which the CU has read by then, follow there).
+    const int lg0 = CU_LG * (int) blockIdx.x, lgn = max(0, min(CU_LG, T * E - lg0));
+    const int nb_x = a.d >> 3;
+    const bool early = NORM && nb_x <= 256;   // (a logit's operands in one request a lane)
+    RouterRegs rr;
+    if (early && wv >= NW - lgn) {
+        const int item = lg0 + NW - 1 - wv, e = item - (int) ((uint32_t) item / c.by_E) * E;
+        router_fetch_row(rr, a.rw + (size_t) e * a.d, nb_x, lane);
+    }
     if (a.nw) {   // the rows' scales, as the norm kernel sums them: 256 threads, thread i takes x[i], x[i + 256], ..
         for (int t = 0; t < T; ++t) {
             float ss = 0.0f;
@@ -135,10 +146,11 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     // line (item i at word 16 (i / CU_LG) + i % CU_LG), which is written once, by one instruction.  (A line that 16 CUs each
     // wrote a word of, while every CU polled it, took 1.7 us from the last store to the first CU that saw all of it; a line
     // written once is seen 0.4 us later.  Few items a CU: a CU's vector-memory path takes 1.5 us to load twelve router rows.)
-    const int lg0 = CU_LG * (int) blockIdx.x, lgn = max(0, min(CU_LG, T * E - lg0));
     if (wv >= NW - lgn) {
         const int u = NW - 1 - wv, item = lg0 + u, t = (int) ((uint32_t) item / c.by_E), e = item - t * E;
-        const float lv = router_logit(a.rw + (size_t) e * a.d, a.x + (size_t) t * a.xs, a.d, a.nw, a.nw ? rn_s[t] : 1.0f);
+        if (early) router_fetch_input(rr, a.x + (size_t) t * a.xs, nb_x, a.nw, lane);
+        const float lv = early ? router_sum(router_add(rr, nb_x, true, rn_s[t], lane, 0.0f))
+                               : router_logit(a.rw + (size_t) e * a.d, a.x + (size_t) t * a.xs, a.d, a.nw, a.nw ? rn_s[t] : 1.0f);
         if (lane == 0) lgs[u] = lv;
     }
     tables_store<NTHR>(tab, tw);
@@ -570,9 +582,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     }
 }
 
-template <int P, bool SG, bool SD, int NTHR>
-int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds) {
-    void (*kern)(FusedArgs, CuParams) = k_moe_decode_cu<P, SG, SD, NTHR>;
+template <int P, bool SG, bool SD, int NTHR, bool NORM>
+int launch_one_n(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds) {
+    void (*kern)(FusedArgs, CuParams) = k_moe_decode_cu<P, SG, SD, NTHR, NORM>;
     static size_t lds_set = 0;   // the largest dynamic-LDS request this kernel has been prepared for
     static int resident = 0;
     if (lds > lds_set) {
@@ -604,6 +616,11 @@ int log2_of(int v) {
 }   // namespace
 
 namespace nslm {
+
+template <int P, bool SG, bool SD, int NTHR>
+int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds) {
+    return a.nw ? launch_one_n<P, SG, SD, NTHR, true>(st, a, c, lds) : launch_one_n<P, SG, SD, NTHR, false>(st, a, c, lds);
+}
 
 // 0 launched; -1 the shape is not this kernel's (nothing launched)
 int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {

@@ -125,6 +125,60 @@ __device__ __forceinline__ void arrive_finish(uint32_t* sync, uint32_t G, uint32
 // load of the round requested before the first use; an 8-term FMA chain a block, the blocks added in order, the lanes by
 // xor-shuffles) on the input - normalised on the way as kq4_norm1p would have stored it when nw is given (rn: the row's scale) -
 // rounded to BF16.  Every lane returns the value.
+// router_logit in pieces (the same loads, the same chain of operations), for a kernel that requests a logit's router row before it
+// knows the row's scale: router_fetch_row / router_fetch_input ask for the lane's four blocks from j0 on, router_add adds their
+// dot products to acc in block order, router_sum is the wave's sum and its rounding.  (router_logit itself stays as it is: built
+// from these pieces it was 0.6 us slower inside the step kernels.)
+struct RouterRegs {
+    uint4 q[4];
+    float4 x0[4], x1[4], w0[4], w1[4];
+};
+// (the router's row alone - the operand that comes from HBM; the input and the norm weights, which the CU has just read, follow)
+__device__ __forceinline__ void router_fetch_row(RouterRegs& r, const uint16_t* wr, int nb, int j0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r.q[u] = *(const uint4*) (wr + (size_t) min(j0 + 64 * u, nb - 1) * 8);   // clamped: the loads stay unconditional
+}
+__device__ __forceinline__ void router_fetch_input(RouterRegs& r, const float* xr, int nb, const float* nw, int j0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const size_t j = (size_t) min(j0 + 64 * u, nb - 1);
+        r.x0[u] = *(const float4*) (xr + j * 8);
+        r.x1[u] = *(const float4*) (xr + j * 8 + 4);
+        if (nw) {
+            r.w0[u] = *(const float4*) (nw + j * 8);
+            r.w1[u] = *(const float4*) (nw + j * 8 + 4);
+        }
+    }
+}
+__device__ __forceinline__ void router_fetch(RouterRegs& r, const uint16_t* wr, const float* xr, int nb, const float* nw, int j0) {
+    router_fetch_row(r, wr, nb, j0);
+    router_fetch_input(r, xr, nb, nw, j0);
+}
+__device__ __forceinline__ float router_add(const RouterRegs& r, int nb, bool normed, float rn, int j0, float acc) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        if (j0 + 64 * u >= nb) break;
+        float4 y0 = r.x0[u], y1 = r.x1[u];
+        if (normed) {
+            y0.x = y0.x * rn * (1.0f + r.w0[u].x); y0.y = y0.y * rn * (1.0f + r.w0[u].y); y0.z = y0.z * rn * (1.0f + r.w0[u].z); y0.w = y0.w * rn * (1.0f + r.w0[u].w);
+            y1.x = y1.x * rn * (1.0f + r.w1[u].x); y1.y = y1.y * rn * (1.0f + r.w1[u].y); y1.z = y1.z * rn * (1.0f + r.w1[u].z); y1.w = y1.w * rn * (1.0f + r.w1[u].w);
+        }
+        float dd = bf(r.q[u].x & 0xFFFFu) * y0.x;
+        dd = fmaf(bf(r.q[u].x >> 16), y0.y, dd);
+        dd = fmaf(bf(r.q[u].y & 0xFFFFu), y0.z, dd);
+        dd = fmaf(bf(r.q[u].y >> 16), y0.w, dd);
+        dd = fmaf(bf(r.q[u].z & 0xFFFFu), y1.x, dd);
+        dd = fmaf(bf(r.q[u].z >> 16), y1.y, dd);
+        dd = fmaf(bf(r.q[u].w & 0xFFFFu), y1.z, dd);
+        dd = fmaf(bf(r.q[u].w >> 16), y1.w, dd);
+        acc = fmaf(dd, 1.0f, acc);
+    }
+    return acc;
+}
+__device__ __forceinline__ float router_sum(float acc) {
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    return bfr(acc);
+}
 __device__ __forceinline__ float router_logit(const uint16_t* wr, const float* xr, int d, const float* nw, float rn) {
     const int lane = threadIdx.x & 63, nb = d / 8;
     float acc = 0.0f;
