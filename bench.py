@@ -335,8 +335,8 @@ def model_workload(name, steps, warmup, no_graph, branches=False, splits=32):
     flops = 2.0 * T * (m.step_bytes() - 2 * cfg["vocab"] * cfg["d"]) / 4.5 * 8 + 2.0 * T * cfg["vocab"] * cfg["d"]
     res = dict(ms_per_step=ms, wall_ms_per_step=wall_ms / steps, bytes_per_step=bytes_step, tokens=T, flops_per_step=flops)
     res["roofline"] = dict(bound="hbm", achieved=bytes_step / ms / 1e6, peak=HBM_PEAK_GBS, unit="GB/s", frac=bytes_step / ms / 1e6 / HBM_PEAK_GBS,
-                           traffic=None, traffic_source=None, kernel="whole decode step (k_moe_decode x 24 is the largest share)" if T <= 8 else
-                           "whole decode step (grouped k_mm_stream launches are the largest share)",
+                           traffic=None, traffic_source=None, kernel="whole decode step (%s x 24 is the largest share)" % ("k_moe_decode_cu" if T == 1 else "k_moe_decode" if T <= 8 else "k_moe_decode_grouped")
+                           if T <= 24 else "whole decode step (grouped k_mm_stream launches are the largest share)",
                            launch_us=ms * 1e3, algorithmic_bytes=bytes_step)
     res["config"] = {"workload": f"C4 full synthetic model greedy decode: 24 layers, hidden 2048, MLA 16 heads (latent 512 + rope 64, FP8 cache), "
                                  f"128 seeded P=4 experts top-8 (intermediate 768) + shared expert, vocab 151936 BF16 LM head, batch {T}, "
