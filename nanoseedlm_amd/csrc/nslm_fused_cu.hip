@@ -65,6 +65,7 @@ struct CuParams {
     int rpw, tpp, Wt;     // gate + up: virtual rows a wave-task, tasks a pair, tasks a token
     int n_c, ncu_act;     // tasks a CU and token; CUs that have tasks
     int rpi_g, nit_g;     // gate + up where a row's chunks do not fit a wave: virtual rows an iteration of the workgroup, iterations a token
+    int ltail_g, ltail_d; // P = 3, passes by iterations: log2 of the lanes that share a chunk in the pass's last iteration (0: a thread a chunk there too)
     int rpc;              // down: output rows a CU owns
     int rpi, rows_t, nit; // down: (pair, row)s an iteration of the workgroup, (pair, row)s a token and CU, iterations a token
     int nbp;              // blocks of 8 in a row of A
@@ -284,10 +285,17 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     // in the slot where its next task's records would have been requested, a whole task ahead of their use)
     const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
     const int dl = (int) ((uint32_t) tid / c.by_Ld), dch = tid - dl * Ld;
+    // A pass's last iteration seldom fills the workgroup (C3: 2 of 22 virtual rows, 4 of 22 down rows), and a thread a chunk makes
+    // it as long as a full one.  Where its chunks fit the workgroup 2, 4 or 8 times over, as many adjacent lanes share a chunk there
+    // (chunk_dot_split: the same bits): thread = (chunk of the iteration, lane of the chunk's group).
+    const int ltg = P == 3 ? c.ltail_g : 0, ltd = P == 3 ? c.ltail_d : 0;
+    const int tgx = tid >> ltg, tgl = (int) ((uint32_t) tgx / c.by_Lg), tgch = tgx - tgl * Lg, tgs = tid & ((1 << ltg) - 1);
+    const int tdx = tid >> ltd, tdl = (int) ((uint32_t) tdx / c.by_Ld), tdch = tdx - tdl * Ld, tds = tid & ((1 << ltd) - 1);
     auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
-        const int g = min(it * c.rpi + dl, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
+        const bool tl = ltd && it == c.nit - 1;
+        const int g = min(it * c.rpi + (tl ? tdl : dl), c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
         const WSlice& w = slice(min(t, T - 1), jj, 2);
-        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) dch);
+        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) (tl ? tdch : dch));
     };
     Chunk dcur;
     // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
@@ -359,8 +367,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         // (the loads are unconditional: a load under a condition keeps the compiler from counting the loads in flight, and it
         // then waits for the next task's records before it computes the current one.  Past the last task the slot requests
         // the thread's first down records instead.)
-        const int g_d = min(dl, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
-        const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) dch;
+        const bool tl_d = ltd && c.nit == 1;   // (fetch_d(0, 0)'s records)
+        const int g_d = min(tl_d ? tdl : dl, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
+        const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) (tl_d ? tdch : dch);
         auto fetch = [&](int t, int i) {
             const bool ok = t < T;
             const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), r = (q - j * c.tpp) << c.lgV;   // the task's first SwiGLU row
@@ -413,8 +422,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         const bool gact = gl < c.rpi_g;
         float* const partg = (float*) scr;   // [2][NTHR]
         auto fetch_g = [&](int t, int it) {   // (unconditional: rows past the CU's last are clamped)
-            const int v = min(it * c.rpi_g + gl, 2 * n_loc - 1), q = q_lo + (v >> 1), j = (int) ((uint32_t) q / c.by_tpp);
-            return load_chunk<P>(slice(min(t, T - 1), j, v & 1), (uint32_t) (q - j * c.tpp) * (uint32_t) Lg + (uint32_t) gch);
+            const bool tl = ltg && it == c.nit_g - 1;
+            const int v = min(it * c.rpi_g + (tl ? tgl : gl), 2 * n_loc - 1), q = q_lo + (v >> 1), j = (int) ((uint32_t) q / c.by_tpp);
+            return load_chunk<P>(slice(min(t, T - 1), j, v & 1), (uint32_t) (q - j * c.tpp) * (uint32_t) Lg + (uint32_t) (tl ? tgch : gch));
         };
         Chunk cur = fetch_g(0, 0);
         int par = 0;
@@ -422,26 +432,35 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             for (int it = 0; it < c.nit_g; ++it, par ^= 1) {
                 const bool last = it + 1 == c.nit_g;
                 const Chunk nxt = fetch_g(last ? t + 1 : t, last ? 0 : it + 1);
-                const int v = it * c.rpi_g + gl, vc = min(v, 2 * n_loc - 1), q = q_lo + (vc >> 1), j = (int) ((uint32_t) q / c.by_tpp);
-                float acc[1] = {0.0f};
-                if (gact && v < 2 * n_loc) chunk_dot<P, 1, true>(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + gch * XP, 0, 1, acc);
-                partg[par * NTHR + tid] = acc[0];
+                const bool tl = ltg && last;
+                const int rl = tl ? tgl : gl, rch = tl ? tgch : gch;
+                const int v = it * c.rpi_g + rl, vc = min(v, 2 * n_loc - 1), q = q_lo + (vc >> 1), j = (int) ((uint32_t) q / c.by_tpp);
+                if (!tl) {
+                    float acc[1] = {0.0f};
+                    if (gact && v < 2 * n_loc) chunk_dot<P, 1, true>(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + rch * XP, 0, 1, acc);
+                    partg[par * NTHR + tid] = acc[0];
+                } else if constexpr (P == 3) {
+                    if (rl < c.rpi_g && v < 2 * n_loc) {   // (the lanes of a chunk's group take this branch together)
+                        const float sum = chunk_dot_split(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + rch * XP, tgs, ltg);
+                        if (tgs == (1 << ltg) - 1) partg[par * NTHR + tgx] = sum;
+                    }
+                }
                 __syncthreads();
                 const int nrow = min(c.rpi_g, 2 * n_loc - it * c.rpi_g);
                 if (tid < nrow / 2) {
-                    // the two rows' partial sums in chunk order; eight are read before the first is added (a chunk past the row's
+                    // the two rows' partial sums in chunk order; sixteen of each are read before the first is added (a chunk past the row's
                     // last counts +0, which leaves the sum's bits alone)
                     const float* pg = partg + par * NTHR + (2 * tid) * Lg;
                     float gs = 0.0f, us = 0.0f;
-                    for (int c0 = 0; c0 < Lg; c0 += 8) {
-                        float pv[8], pu[8];
+                    for (int c0 = 0; c0 < Lg; c0 += 16) {
+                        float pv[16], pu[16];
 #pragma unroll
-                        for (int cc = 0; cc < 8; ++cc) {
+                        for (int cc = 0; cc < 16; ++cc) {
                             pv[cc] = pg[min(c0 + cc, Lg - 1)];
                             pu[cc] = pg[Lg + min(c0 + cc, Lg - 1)];
                         }
 #pragma unroll
-                        for (int cc = 0; cc < 8; ++cc) {
+                        for (int cc = 0; cc < 16; ++cc) {
                             gs += c0 + cc < Lg ? pv[cc] : 0.0f;
                             us += c0 + cc < Lg ? pu[cc] : 0.0f;
                         }
@@ -494,7 +513,8 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         __syncthreads();
     };
     // the rows' sums of one iteration from the threads' chunk sums, rounded as the separate launches round them
-    auto rows_out = [&](int t, int it, float acc0, bool ok, int g, int j, int rr, bool last) {
+    int dpar = 0;
+    auto rows_out = [&](int t, int it, float acc0, bool ok, int g, int j, int rr, bool last, int slot) {   // slot: where the thread's chunk sum goes (< 0: it has none)
         if (SHFL_D) {
             float s = acc0;
             for (int o = Ld >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -504,25 +524,29 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 a.D[((size_t) t * kk + j) * a.d + r0 + rr] = dv;
             }
         } else {
-            part[tid] = acc0;
+            // (the chunk sums are double-buffered by iteration parity, as the gate + up pass's: the next iteration's chunks are
+            // decoded while this one's rows are summed, and the buffer is written again only behind the next iteration's barrier)
+            float* const pb = part + dpar * NTHR;
+            dpar ^= 1;
+            if (slot >= 0) pb[slot] = acc0;
             __syncthreads();
             const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
             if (tid < c.rpi && gs < c.rows_t && rs < nr) {
-                // the row's partial sums in chunk order; eight are read before the first is added (a chunk past the row's
+                // the row's partial sums in chunk order; sixteen are read before the first is added (a chunk past the row's
                 // last counts +0, which leaves the sum's bits alone)
                 float s = 0.0f;
-                for (int c0 = 0; c0 < Ld; c0 += 8) {
-                    float pv[8];
+                for (int c0 = 0; c0 < Ld; c0 += 16) {
+                    float pv[16];
 #pragma unroll
-                    for (int cc = 0; cc < 8; ++cc) pv[cc] = part[tid * Ld + min(c0 + cc, Ld - 1)];
+                    for (int cc = 0; cc < 16; ++cc) pv[cc] = pb[tid * Ld + min(c0 + cc, Ld - 1)];
 #pragma unroll
-                    for (int cc = 0; cc < 8; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
+                    for (int cc = 0; cc < 16; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
                 }
                 const float dv = bfr(s * NSLM_R32);
                 dsum[gs] = dv;
                 a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
             }
-            if (!last) __syncthreads();   // part is written again by the next iteration
+            (void) last;
         }
     };
     // out = sum_j wt_j D_j in j order (kq4_moe_combine's FMA chain), the shared expert's pair with weight 1 last
@@ -557,7 +581,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             wait_stage(0);
             float acc0 = 0.0f;
             if (ok) cols_post(zp, dcur.codes, slice(0, j, 2).eb, xd + j * (Ld * XP) + dch * XP, acc0);
-            rows_out(0, 0, acc0, ok, g, j, rr, true);
+            rows_out(0, 0, acc0, ok, g, j, rr, true, tid);
             __syncthreads();
             combine(0);
         }
@@ -568,11 +592,19 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         for (int it = 0; it < c.nit; ++it) {
             const bool last = it + 1 == c.nit;
             const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
-            const int g = it * c.rpi + dl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
-            const bool ok = dl < c.rpi && g < c.rows_t && rr < nr;
+            const bool tl = ltd && last;
+            const int rl = tl ? tdl : dl, rch = tl ? tdch : dch;
+            const int g = it * c.rpi + rl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
+            const bool ok = rl < c.rpi && g < c.rows_t && rr < nr;
             float acc[1] = {0.0f};
-            if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + dch * XP, 0, 1, acc);
-            rows_out(t, it, acc[0], ok, g, j, rr, last);
+            int slot = tid;
+            if (!tl) {
+                if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + rch * XP, 0, 1, acc);
+            } else if constexpr (P == 3) {
+                if (ok) acc[0] = chunk_dot_split(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + rch * XP, tds, ltd);   // (a chunk's lanes together)
+                slot = ok && tds == (1 << ltd) - 1 ? tdx : -1;
+            }
+            rows_out(t, it, acc[0], ok, g, j, rr, last, slot);
             dcur = dnxt;
         }
         __syncthreads();
@@ -659,6 +691,15 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     c.vpt = c.rpw / 2;
     c.lgV = log2_of(c.vpt);
     c.nit_g = sg ? 0 : (2 * c.n_c + c.rpi_g - 1) / c.rpi_g;
+    if (P == 3) {   // the last iteration's chunks over 2, 4 or 8 lanes each where they fit
+        auto lanes_log2 = [&](int rows, int L) {
+            for (int l = 3; l >= 1; --l)
+                if (((long) rows * L << l) <= nthr) return l;
+            return 0;
+        };
+        if (!sg) c.ltail_g = lanes_log2(2 * c.n_c - (c.nit_g - 1) * c.rpi_g, a.Lg);
+        if (!sd) c.ltail_d = lanes_log2(c.rows_t - (c.nit - 1) * c.rpi, a.Ld);
+    }
     c.by_Lg = fastdiv_of((uint32_t) a.Lg);
     c.by_E = fastdiv_of((uint32_t) a.E);
     c.by_tpp = fastdiv_of((uint32_t) c.tpp);

@@ -232,6 +232,44 @@ __device__ __forceinline__ void chunk_dot(const Chunk& ck, int eb, const uint32_
     }
 }
 
+// A P = 3 chunk's sum by 2^ls adjacent lanes (ls = 1 .. 3), lane s of the group taking blocks [s nb, (s + 1) nb), nb = 8 >> ls: each
+// block's product with the activations as block_dot forms it, then block_dot's chain of multiply-adds over the blocks in block
+// order, handed from lane to lane (lane s holds its final value after step s).  The group's last lane returns chunk_dot's bits.
+__device__ __forceinline__ float chunk_dot_split(const Chunk& ck, int eb, const uint32_t* tab, const float* xr, int s, int ls) {
+    const int nb = 8 >> ls, b0 = s * nb;
+    float d[4] = {0.0f, 0.0f, 0.0f, 0.0f}, e2[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (i < nb) {
+            const int b = b0 + i;
+            const uint32_t ss = word_of(ck.sd, b >> 1), cc = word_of(ck.cw, b >> 1);
+            const uint32_t seed16 = (b & 1) ? ss >> 16 : ss & 0xFFFFu, word16 = (b & 1) ? cc >> 16 : cc & 0xFFFFu;
+            int is[8];
+            isum_p3((b & 1) ? ss : ss << 16, stream_of(tab, seed16), tab[512 + ((word16 >> 4) & 0xFFu)], tab[512 + (word16 >> 12)], is);
+            const float* xb = xr + 8 * b;
+            float w[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) w[c] = (float) is[c];
+            float dd = w[0] * xb[0];
+#pragma unroll
+            for (int c = 1; c < 8; ++c) dd = fmaf(w[c], xb[c], dd);
+            d[i] = dd;
+            e2[i] = pow2f(eb + (int) (word16 & 15u));
+        }
+    }
+    float acc = 0.0f;
+    for (int step = 0; step < (1 << ls); ++step) {
+        // (the lane below, by a row shift of the wave's data path: the groups lie inside rows of 16 lanes)
+        const float in = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x111, 0xF, 0xF, false));
+        float v = s == 0 ? 0.0f : in;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (i < nb) v = fmaf(d[i], e2[i], v);
+        acc = v;
+    }
+    return acc;
+}
+
 // The 8 weights of block j of row r as f32: seeds unscaled integers with *sc = 2^e R32; BF16 / Q8 as BF16 values; Q4 in
 // MLX's matvec form s * q + b unrounded (reference engine/kernels_moe.cu:91-107, 171-189).
 __device__ __forceinline__ void block_weights(int fmt, const WSlice& w, const uint32_t* tab, int r, int K, int j, float (&o)[8],

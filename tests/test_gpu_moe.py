@@ -229,14 +229,15 @@ def test_fused_step_equal_logits(oracle, case, E):
 
 
 @pytest.mark.parametrize("fmt", [packs.MF_SEED4P4, packs.MF_SEED4])
-@pytest.mark.parametrize("d,ff", [(2880, 2880), (2816, 2880), (4480, 5760)])
-def test_fused_step_rows_that_do_not_fill_a_workgroup(d, ff, fmt):
+@pytest.mark.parametrize("d,ff,k", [(2880, 2880, 2), (2880, 2880, 4), (2816, 2880, 2), (4480, 5760, 2)])
+def test_fused_step_rows_that_do_not_fill_a_workgroup(d, ff, k, fmt):
     """Rows of 44, 45, 70 or 90 chunks (hidden 2880 = the mixed-format configuration): whole rows do not fill a workgroup's
     256 threads, the row sums go through LDS in both passes, and 2816 rows are 563.2 iterations of 5, so the last item
-    ends inside an iteration.  Same bits as the separate launches, at 1, 3 and 8 rows."""
+    ends inside an iteration.  Same bits as the separate launches, at 1, 3 and 8 rows.  With a workgroup a CU (1 and 2 rows) a
+    pass's last iteration holds 2, 3, 4 or 6 rows, whose chunks 8, 4 or 2 lanes share (top-4 of 2880 x 2880: 4 lanes in the down pass)."""
     from nanoseedlm_amd import moe
-    rng = np.random.default_rng(d + ff + fmt)
-    E, k = 6, 2
+    rng = np.random.default_rng(d + ff + fmt + k)
+    E = 6
     mk = packs.seed4p4 if fmt == packs.MF_SEED4P4 else packs.seed4
     st = moe.MoeStack(1, E, k, d, ff, fmt=fmt, router=moe.ROUTE_SOFTMAX, max_rows=8)
     gate, up, down = mk(rng, E, ff, d, eb=-23), mk(rng, E, ff, d, eb=-23), mk(rng, E, d, ff, eb=-22)
