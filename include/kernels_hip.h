@@ -299,7 +299,7 @@ int kc_moe_decode_error_word(void);
  * between streams may want a shorter bound; tests set a tiny one to drive the error path while every kernel still exits. */
 void kc_moe_decode_spin_limit(unsigned polls);
 /* Which of the library's two persistent kernels a step of up to MV_MAXT tokens takes (the same bits either way): 0 (default) the
- * one with a workgroup per CU at 1 token, and at 2 where it measured faster (the 64-weight chunks of a hidden row a power of two <= 32, and the format P = 3 or top_k * d * ff >= 24 Mi) where the shape fits it (T * pairs * ff <= 65536, T * n_exp <= 1024, the tokens' staged inputs within
+ * one with a workgroup per CU at 1 token, and at 2 where it measured faster (the format P = 3, or the 64-weight chunks of a hidden row a power of two <= 32 and top_k * d * ff >= 24 Mi) where the shape fits it (T * pairs * ff <= 65536, T * n_exp <= 1024, the tokens' staged inputs within
  * a CU's LDS), else the one with a workgroup per (pair, row tile); 1 always the latter; 2 the former wherever the shape fits
  * it.  Process-global, for comparisons. */
 void kc_moe_decode_kernel(int which);

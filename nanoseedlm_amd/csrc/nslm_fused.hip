@@ -998,12 +998,12 @@ int kc_moe_decode_layer(kc_stream_t s, int fmt, const uint16_t* router_w, const 
         if (!sg) return -1;
         return fmt == MF_SEED4P4 ? launch_grouped<4, 2>((hipStream_t) s, a, sg, sd) : launch_grouped<3, 2>((hipStream_t) s, a, sg, sd);
     }
-    // one workgroup per CU: ahead at one token everywhere, at two where a row's chunks fill a wave and the step is large or P = 3 (us,
-    // a workgroup per CU / per item, records from HBM.  C2: 1 token 19.9 / 25.2, 2: 36.6 / 35.5, 3: 48.4 / 45.5; C2's shape in P = 3:
-    // 24.6 / 26.3, 39.4 / 43.5, 54.7 / 50.9, 4: 70.0 / 63.8; 256 experts of 4096 x 1024: 45.8 / 54.9, 80.7 / 90.6, 168.8 / 168.9; C3,
-    // whose rows of 45 chunks make that kernel's gate + up pass go by iterations of the workgroup: 59.7 / 67.3, 108.7 / 105.0,
-    // 158.3 / 148.4)
-    const bool cu_two = sg && (fmt != MF_SEED4P4 || (long) top_k * d * ff >= 24L << 20);
+    // one workgroup per CU: ahead at one token everywhere, at two where the step is large or P = 3 (us, a workgroup per CU / per
+    // item, records from HBM.  C2: 1 token 19.9 / 25.2, 2: 36.6 / 35.5, 3: 48.4 / 45.5; C2's shape in P = 3: 24.6 / 26.3,
+    // 39.4 / 43.5, 54.7 / 50.9, 4: 70.0 / 63.8; 256 experts of 4096 x 1024: 45.8 / 54.9, 80.7 / 90.6, 168.8 / 168.9; C3, whose rows
+    // of 45 chunks make that kernel's passes go by iterations of the workgroup: 55.0 / 67.3, 100.9 / 104.7, 146.9 / 147.6,
+    // 192.6 / 186.2)
+    const bool cu_two = fmt != MF_SEED4P4 || (sg && (long) top_k * d * ff >= 24L << 20);
     if ((g_kernel_choice == 2 || (g_kernel_choice == 0 && T <= (cu_two ? 2 : 1))) && launch_moe_decode_cu((hipStream_t) s, a, fmt == MF_SEED4P4 ? 4 : 3, sd) == 0) return 0;
     const int kmax = d > ff ? d : ff;
     size_t lds = (size_t) (kmax / 64) * (fmt == MF_SEED4P4 ? xpad<4>() : xpad<3>()) * sizeof(float);

@@ -20,9 +20,9 @@
 //     when its down pass needs it, so only a one-token launch waits for the exchange.
 //   - Every instruction outside the row loops counts (a CU's waves all execute it at the same moment): what can be computed
 //     on the host arrives in the arguments, and no index is formed by an integer division.
-//   - Rows whose chunks do not fit a wave as a power of two (45 chunks, say) take the gate + up pass by iterations of the whole
-//     workgroup instead - a thread a chunk of a virtual row, the row sums through LDS in chunk order, one barrier an
-//     iteration - with 22 of 22.7 possible rows an iteration where a 256-thread workgroup fills 4 of 5.7.
+//   - Rows whose chunks do not fit a wave as a power of two (45 chunks, say) take both passes by iterations of the whole
+//     workgroup instead - the token's chunks dealt to the threads as one list, the row sums through LDS in chunk order, one barrier
+//     an iteration - with 1012 of 1024 threads busy where a 256-thread workgroup fills 4 of 5.7 possible rows.
 // Shapes: a row of at most 256 chunks, T * pairs * ff <= FUSED_XA_MAX, the workgroup's LDS <= 160 KB less the table.  Other
 // shapes stay with the kernel of nslm_fused.hip.
 #include "nslm_fused_dev.h"
@@ -47,7 +47,7 @@ __device__ __forceinline__ uint32_t operator/(uint32_t x, FastDiv f) { return f.
 struct CuParams {
     int xg;      // [T][Lg * xpad] the tokens' inputs in the form the gate + up matvec reads
     int xd;      // [kk][Ld * xpad] one token's A, all pairs, in the form the down matvec reads
-    int scr;     // [NTHR] down pass: the threads' partial sums (rows that do not fit a shuffle)
+    int scr;     // [4 NTHR] passes by iterations: the chunks' sums of three iterations, the first iteration's slots twice
     int pk;      // [T][KP] ranking: the logits' keys
     int rv;      // [T][E4] the logits
     int dsum;    // [kk][rpc] the down rows of the token in hand, rounded to BF16
@@ -64,14 +64,14 @@ struct CuParams {
     int lgL;              // log2 of the chunks in a gate / up row (Lg)
     int rpw, tpp, Wt;     // gate + up: virtual rows a wave-task, tasks a pair, tasks a token
     int n_c, ncu_act;     // tasks a CU and token; CUs that have tasks
-    int rpi_g, nit_g;     // gate + up where a row's chunks do not fit a wave: virtual rows an iteration of the workgroup, iterations a token
+    int nit_g;            // gate + up where a row's chunks do not fit a wave: iterations of the workgroup a token
     int ltail_g, ltail_d; // P = 3, passes by iterations: log2 of the lanes that share a chunk in the pass's last iteration (0: a thread a chunk there too)
     int rpc;              // down: output rows a CU owns
     int rpi, rows_t, nit; // down: (pair, row)s an iteration of the workgroup, (pair, row)s a token and CU, iterations a token
     int nbp;              // blocks of 8 in a row of A
     int vpt, lgV;         // SwiGLU outputs a task (rpw / 2) and its log2
     int E4, KP;           // E padded to 4; keys a token (E padded to 16)
-    FastDiv by_tpp, by_rpc, by_Ld, by_Lg, by_nbp, by_kk, by_E;
+    FastDiv by_tpp, by_rpc, by_Ld, by_Lg, by_nbp, by_kk, by_E, by_ring;
 };
 
 // NORM: the launch normalises its input (a.nw); launches that do not are compiled without what that path adds.
@@ -285,17 +285,38 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     // in the slot where its next task's records would have been requested, a whole task ahead of their use)
     const int r0 = (int) blockIdx.x * rpc, nr = max(0, min(rpc, a.d - r0));
     const int dl = (int) ((uint32_t) tid / c.by_Ld), dch = tid - dl * Ld;
-    // A pass's last iteration seldom fills the workgroup (C3: 2 of 22 virtual rows, 4 of 22 down rows), and a thread a chunk makes
-    // it as long as a full one.  Where its chunks fit the workgroup 2, 4 or 8 times over, as many adjacent lanes share a chunk there
-    // (chunk_dot_split: the same bits): thread = (chunk of the iteration, lane of the chunk's group).
+    // Passes by iterations (rows whose chunks are no power of two inside a wave) deal a token's chunks to the threads as one
+    // list - thread i of iteration it takes chunk it NTHR + i, rows end where they end - so only the pass's last iteration can
+    // be short.  A thread a chunk would make that one as long as a full one; where its chunks fit the workgroup 2, 4 or 8 times
+    // over (P = 3), as many adjacent lanes share a chunk there (chunk_dot_split: the same bits).  The chunk sums wait for their
+    // row's last in a ring of three iterations: a row's chunks lie in at most two, and the third is being written.  The ring's first
+    // NTHR slots are kept twice, the copy behind its end, so that a row's sums are read from consecutive words wherever it starts.
+    constexpr int RING = 3 * NTHR;
     const int ltg = P == 3 ? c.ltail_g : 0, ltd = P == 3 ? c.ltail_d : 0;
-    const int tgx = tid >> ltg, tgl = (int) ((uint32_t) tgx / c.by_Lg), tgch = tgx - tgl * Lg, tgs = tid & ((1 << ltg) - 1);
-    const int tdx = tid >> ltd, tdl = (int) ((uint32_t) tdx / c.by_Ld), tdch = tdx - tdl * Ld, tds = tid & ((1 << ltd) - 1);
+    struct Deal {
+        int f, row, ch, sub;   // chunk of the token's list, its row and place in the row, the thread's place among the chunk's lanes
+        bool tail;
+    };
+    auto deal = [&](int it, int nit, int lt, int L, FastDiv by_L) {
+        Deal q;
+        q.tail = lt && it == nit - 1;
+        q.f = it * NTHR + (q.tail ? tid >> lt : tid);
+        q.row = (int) ((uint32_t) q.f / by_L);
+        q.ch = q.f - q.row * L;
+        q.sub = q.tail ? tid & ((1 << lt) - 1) : 0;
+        return q;
+    };
+    auto ring_slot = [&](int f) { return f - (int) ((uint32_t) f / c.by_ring) * RING; };
+    auto ring_put = [&](float* ring, int f, float v) {
+        const int sl = ring_slot(f);
+        ring[sl] = v;
+        if (sl < NTHR) ring[sl + RING] = v;
+    };
     auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
-        const bool tl = ltd && it == c.nit - 1;
-        const int g = min(it * c.rpi + (tl ? tdl : dl), c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
+        const Deal q = deal(it, c.nit, ltd, Ld, c.by_Ld);
+        const int g = min(q.row, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
         const WSlice& w = slice(min(t, T - 1), jj, 2);
-        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) (tl ? tdch : dch));
+        return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) q.ch);
     };
     Chunk dcur;
     // ---- gate + up + SwiGLU: a wave a task = 64 / Lg virtual rows (2r = gate row r, 2r + 1 = up row r) of one pair -------------
@@ -367,9 +388,9 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         // (the loads are unconditional: a load under a condition keeps the compiler from counting the loads in flight, and it
         // then waits for the next task's records before it computes the current one.  Past the last task the slot requests
         // the thread's first down records instead.)
-        const bool tl_d = ltd && c.nit == 1;   // (fetch_d(0, 0)'s records)
-        const int g_d = min(tl_d ? tdl : dl, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
-        const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) (tl_d ? tdch : dch);
+        const Deal q_d = deal(0, c.nit, ltd, Ld, c.by_Ld);   // (fetch_d(0, 0)'s records)
+        const int g_d = min(q_d.row, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
+        const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) q_d.ch;
         auto fetch = [&](int t, int i) {
             const bool ok = t < T;
             const int q = ok ? q_lo + i : 0, j = (int) ((uint32_t) q / c.by_tpp), r = (q - j * c.tpp) << c.lgV;   // the task's first SwiGLU row
@@ -414,50 +435,50 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         __builtin_amdgcn_s_setprio(0);
     }
     else if (n_loc > 0) {
-        // Rows whose chunks do not fit a wave (a row of 45 chunks, say): the pass goes by iterations of the whole workgroup, a thread
-        // a chunk of a virtual row (2r = gate row r, 2r + 1 = up row r of the CU's run of SwiGLU rows, a "task" being one such
-        // row), the row sums through LDS in chunk order (the separate launches' order), one workgroup barrier an iteration
-        // (the partial sums are double-buffered by iteration parity).
-        const int gl = (int) ((uint32_t) tid / c.by_Lg), gch = tid - gl * Lg;
-        const bool gact = gl < c.rpi_g;
-        float* const partg = (float*) scr;   // [2][NTHR]
+        // Rows whose chunks do not fit a wave (a row of 45 chunks, say): the pass goes by iterations of the whole workgroup over the
+        // chunks of the CU's virtual rows (2r = gate row r, 2r + 1 = up row r of its run of SwiGLU rows, a "task" being one such
+        // pair of rows), the row sums through LDS in chunk order (the separate launches' order), one workgroup barrier an iteration.
+        float* const partg = (float*) scr;   // [RING + NTHR]
+        const int nch = 2 * n_loc * Lg;      // this CU's chunks a token
         auto fetch_g = [&](int t, int it) {   // (unconditional: rows past the CU's last are clamped)
-            const bool tl = ltg && it == c.nit_g - 1;
-            const int v = min(it * c.rpi_g + (tl ? tgl : gl), 2 * n_loc - 1), q = q_lo + (v >> 1), j = (int) ((uint32_t) q / c.by_tpp);
-            return load_chunk<P>(slice(min(t, T - 1), j, v & 1), (uint32_t) (q - j * c.tpp) * (uint32_t) Lg + (uint32_t) (tl ? tgch : gch));
+            const Deal q = deal(it, c.nit_g, ltg, Lg, c.by_Lg);
+            const int v = min(q.row, 2 * n_loc - 1), u = q_lo + (v >> 1), j = (int) ((uint32_t) u / c.by_tpp);
+            return load_chunk<P>(slice(min(t, T - 1), j, v & 1), (uint32_t) (u - j * c.tpp) * (uint32_t) Lg + (uint32_t) q.ch);
         };
         Chunk cur = fetch_g(0, 0);
-        int par = 0;
         for (int t = 0; t < T; ++t) {
-            for (int it = 0; it < c.nit_g; ++it, par ^= 1) {
+            int pd = 0;   // SwiGLU rows of the token whose two sums are formed
+            for (int it = 0; it < c.nit_g; ++it) {
                 const bool last = it + 1 == c.nit_g;
                 const Chunk nxt = fetch_g(last ? t + 1 : t, last ? 0 : it + 1);
-                const bool tl = ltg && last;
-                const int rl = tl ? tgl : gl, rch = tl ? tgch : gch;
-                const int v = it * c.rpi_g + rl, vc = min(v, 2 * n_loc - 1), q = q_lo + (vc >> 1), j = (int) ((uint32_t) q / c.by_tpp);
-                if (!tl) {
+                const Deal q = deal(it, c.nit_g, ltg, Lg, c.by_Lg);
+                const int vc = min(q.row, 2 * n_loc - 1), u = q_lo + (vc >> 1), j = (int) ((uint32_t) u / c.by_tpp);
+                const float* xq = xg + t * (Lg * XP) + q.ch * XP;
+                if (!q.tail) {
                     float acc[1] = {0.0f};
-                    if (gact && v < 2 * n_loc) chunk_dot<P, 1, true>(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + rch * XP, 0, 1, acc);
-                    partg[par * NTHR + tid] = acc[0];
+                    if (q.f < nch) chunk_dot<P, 1, true>(cur, slice(t, j, vc & 1).eb, tab, xq, 0, 1, acc);
+                    ring_put(partg, q.f, acc[0]);
                 } else if constexpr (P == 3) {
-                    if (rl < c.rpi_g && v < 2 * n_loc) {   // (the lanes of a chunk's group take this branch together)
-                        const float sum = chunk_dot_split(cur, slice(t, j, vc & 1).eb, tab, xg + t * (Lg * XP) + rch * XP, tgs, ltg);
-                        if (tgs == (1 << ltg) - 1) partg[par * NTHR + tgx] = sum;
+                    if (q.f < nch) {   // (the lanes of a shared chunk take this branch together)
+                        const float sum = chunk_dot_split(cur, slice(t, j, vc & 1).eb, tab, xq, q.sub, ltg);
+                        if (q.sub == (1 << ltg) - 1) ring_put(partg, q.f, sum);
                     }
                 }
                 __syncthreads();
-                const int nrow = min(c.rpi_g, 2 * n_loc - it * c.rpi_g);
-                if (tid < nrow / 2) {
+                // the SwiGLU rows whose last chunk this iteration held, a thread each
+                const int pe = last ? n_loc : min(n_loc, (int) ((uint32_t) ((it + 1) * NTHR) / c.by_Lg) >> 1);
+                if (tid < pe - pd) {
                     // the two rows' partial sums in chunk order; sixteen of each are read before the first is added (a chunk past the row's
                     // last counts +0, which leaves the sum's bits alone)
-                    const float* pg = partg + par * NTHR + (2 * tid) * Lg;
+                    const float* const pg = partg + ring_slot(2 * (pd + tid) * Lg);   // (2 Lg <= NTHR: the copy covers the two rows)
+                    auto at = [&](int o) { return pg[o]; };
                     float gs = 0.0f, us = 0.0f;
                     for (int c0 = 0; c0 < Lg; c0 += 16) {
                         float pv[16], pu[16];
 #pragma unroll
                         for (int cc = 0; cc < 16; ++cc) {
-                            pv[cc] = pg[min(c0 + cc, Lg - 1)];
-                            pu[cc] = pg[Lg + min(c0 + cc, Lg - 1)];
+                            pv[cc] = at(min(c0 + cc, Lg - 1));
+                            pu[cc] = at(Lg + min(c0 + cc, Lg - 1));
                         }
 #pragma unroll
                         for (int cc = 0; cc < 16; ++cc) {
@@ -465,11 +486,12 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                             us += c0 + cc < Lg ? pu[cc] : 0.0f;
                         }
                     }
-                    *(float2*) &avs[2 * (t * nav + it * (c.rpi_g >> 1) + tid)] = make_float2(gs, us);
+                    *(float2*) &avs[2 * (t * nav + pd + tid)] = make_float2(gs, us);
                 }
+                pd = pe;
                 cur = nxt;
             }
-            __syncthreads();   // the token's row sums are all in LDS
+            __syncthreads();   // the token's row sums are all in LDS (and the ring is free for the next token's chunks)
             if (wv == NW - 1) publish(t);
         }
     }
@@ -513,8 +535,8 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         __syncthreads();
     };
     // the rows' sums of one iteration from the threads' chunk sums, rounded as the separate launches round them
-    int dpar = 0;
-    auto rows_out = [&](int t, int it, float acc0, bool ok, int g, int j, int rr, bool last, int slot) {   // slot: where the thread's chunk sum goes (< 0: it has none)
+    int ud = 0;   // (pair, row)s of the token in hand whose sums are formed
+    auto rows_out = [&](int t, int it, float acc0, bool ok, int g, int j, int rr, bool last, int slot) {   // slot: the thread's chunk in the token's list (< 0: it has none to store)
         if (SHFL_D) {
             float s = acc0;
             for (int o = Ld >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o);
@@ -524,21 +546,22 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 a.D[((size_t) t * kk + j) * a.d + r0 + rr] = dv;
             }
         } else {
-            // (the chunk sums are double-buffered by iteration parity, as the gate + up pass's: the next iteration's chunks are
-            // decoded while this one's rows are summed, and the buffer is written again only behind the next iteration's barrier)
-            float* const pb = part + dpar * NTHR;
-            dpar ^= 1;
-            if (slot >= 0) pb[slot] = acc0;
+            // (the chunk sums wait in the ring, as the gate + up pass's: the next iteration's chunks are decoded while this one's
+            // rows are summed)
+            if (slot >= 0) ring_put(part, slot, acc0);
             __syncthreads();
-            const int gs = it * c.rpi + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
-            if (tid < c.rpi && gs < c.rows_t && rs < nr) {
+            // the (pair, row)s whose last chunk this iteration held, a thread each
+            const int ue = last ? c.rows_t : min(c.rows_t, (int) ((uint32_t) ((it + 1) * NTHR) / c.by_Ld));
+            const int gs = ud + tid, js = min((int) ((uint32_t) gs / c.by_rpc), kk - 1), rs = gs - (int) ((uint32_t) gs / c.by_rpc) * rpc;
+            if (tid < ue - ud && rs < nr) {
                 // the row's partial sums in chunk order; sixteen are read before the first is added (a chunk past the row's
                 // last counts +0, which leaves the sum's bits alone)
+                const float* const pg = part + ring_slot(gs * Ld);   // (Ld <= NTHR: the copy covers the row)
                 float s = 0.0f;
                 for (int c0 = 0; c0 < Ld; c0 += 16) {
                     float pv[16];
 #pragma unroll
-                    for (int cc = 0; cc < 16; ++cc) pv[cc] = pb[tid * Ld + min(c0 + cc, Ld - 1)];
+                    for (int cc = 0; cc < 16; ++cc) pv[cc] = pg[min(c0 + cc, Ld - 1)];
 #pragma unroll
                     for (int cc = 0; cc < 16; ++cc) s += c0 + cc < Ld ? pv[cc] : 0.0f;
                 }
@@ -546,7 +569,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
                 dsum[gs] = dv;
                 a.D[((size_t) t * kk + js) * a.d + r0 + rs] = dv;
             }
-            (void) last;
+            ud = ue;
         }
     };
     // out = sum_j wt_j D_j in j order (kq4_moe_combine's FMA chain), the shared expert's pair with weight 1 last
@@ -589,20 +612,20 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
     }
     for (int t = 0; t < T; ++t) {
         wait_stage(t);
+        ud = 0;
         for (int it = 0; it < c.nit; ++it) {
             const bool last = it + 1 == c.nit;
             const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
-            const bool tl = ltd && last;
-            const int rl = tl ? tdl : dl, rch = tl ? tdch : dch;
-            const int g = it * c.rpi + rl, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
-            const bool ok = rl < c.rpi && g < c.rows_t && rr < nr;
+            const Deal q = deal(it, c.nit, ltd, Ld, c.by_Ld);
+            const int g = q.row, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
+            const bool ok = g < c.rows_t && rr < nr;
             float acc[1] = {0.0f};
-            int slot = tid;
-            if (!tl) {
-                if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + rch * XP, 0, 1, acc);
+            int slot = ok ? q.f : -1;
+            if (!q.tail) {
+                if (ok) chunk_dot<P, 1, false>(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + q.ch * XP, 0, 1, acc);
             } else if constexpr (P == 3) {
-                if (ok) acc[0] = chunk_dot_split(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + rch * XP, tds, ltd);   // (a chunk's lanes together)
-                slot = ok && tds == (1 << ltd) - 1 ? tdx : -1;
+                if (ok) acc[0] = chunk_dot_split(dcur, slice(t, j, 2).eb, tab, xd + j * (Ld * XP) + q.ch * XP, q.sub, ltd);   // (a chunk's lanes together)
+                if (q.sub != (1 << ltd) - 1) slot = -1;
             }
             rows_out(t, it, acc[0], ok, g, j, rr, last, slot);
             dcur = dnxt;
@@ -658,7 +681,7 @@ int launch_one(hipStream_t st, const FusedArgs& a, const CuParams& c, size_t lds
 int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     if (a.T < 1 || a.T > MV_MAXT) return -1;
     const bool sg = a.Lg <= 32 && !(a.Lg & (a.Lg - 1));   // a gate / up row's chunks are a power of two inside a wave: row sums by shuffles
-    if (a.Lg > 256) return -1;
+    if (a.Lg > 256 || a.Ld > 1024) return -1;   // (a SwiGLU row's two rows of chunks, a down row's chunks: inside one iteration's threads)
     if ((long) a.T * a.kk * a.ff > FUSED_XA_MAX || a.ff % 64 || a.kk > 33) return -1;
     const int G = fused_cu_count();
     if (G < 1 || a.E > 1024 || (long) a.T * a.E > (long) CU_LG * (G < FUSED_CULG_LINES ? G : FUSED_CULG_LINES)) return -1;   // (a CU forms CU_LG logits)
@@ -674,7 +697,6 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
         c.lgL = 0;
         c.rpw = 2;
         c.tpp = a.ff;
-        c.rpi_g = (nthr / a.Lg) & ~1;
     }
     c.Wt = a.kk * c.tpp;
     c.n_c = (c.Wt + G - 1) / G;
@@ -686,20 +708,21 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     // 16 waves: four a SIMD get through a block's dependent instruction chains faster than three (C2, one token: 22.6 against
     // 23.3 us with 12 waves, whose tasks divide evenly among them; 4 tokens 62.5 against 64.2)
     c.rpi = nthr / a.Ld;
-    c.nit = (c.rows_t + c.rpi - 1) / c.rpi;
+    c.nit = (c.rows_t * a.Ld + nthr - 1) / nthr;   // (rows whose chunks are a power of two inside a wave: whole rows an iteration)
     c.KP = (a.E + 15) & ~15;
     c.vpt = c.rpw / 2;
     c.lgV = log2_of(c.vpt);
-    c.nit_g = sg ? 0 : (2 * c.n_c + c.rpi_g - 1) / c.rpi_g;
+    c.nit_g = sg ? 0 : (2 * c.n_c * a.Lg + nthr - 1) / nthr;
     if (P == 3) {   // the last iteration's chunks over 2, 4 or 8 lanes each where they fit
-        auto lanes_log2 = [&](int rows, int L) {
+        auto lanes_log2 = [&](int chunks) {
             for (int l = 3; l >= 1; --l)
-                if (((long) rows * L << l) <= nthr) return l;
+                if (((long) chunks << l) <= nthr) return l;
             return 0;
         };
-        if (!sg) c.ltail_g = lanes_log2(2 * c.n_c - (c.nit_g - 1) * c.rpi_g, a.Lg);
-        if (!sd) c.ltail_d = lanes_log2(c.rows_t - (c.nit - 1) * c.rpi, a.Ld);
+        if (!sg) c.ltail_g = lanes_log2(2 * c.n_c * a.Lg - (c.nit_g - 1) * nthr);
+        if (!sd) c.ltail_d = lanes_log2(c.rows_t * a.Ld - (c.nit - 1) * nthr);
     }
+    c.by_ring = fastdiv_of((uint32_t) (3 * nthr));
     c.by_Lg = fastdiv_of((uint32_t) a.Lg);
     c.by_E = fastdiv_of((uint32_t) a.E);
     c.by_tpp = fastdiv_of((uint32_t) c.tpp);
@@ -712,7 +735,7 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     auto take = [&](int words) { const int at = o; o += (words + 3) & ~3; return at; };
     c.xg = take(a.T * a.Lg * xp);
     c.xd = take(a.kk * a.Ld * xp);
-    c.scr = take(2 * nthr);
+    c.scr = take(4 * nthr);
     c.pk = take(a.T * c.KP);
     c.rv = take(a.T * c.E4);
     c.dsum = take(a.kk * c.rpc);
