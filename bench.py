@@ -69,10 +69,13 @@ def fail_on_kernel_error(st=None):
 class Q4Projections:
     """Config 3's affine-int4 side of the layer: q / k / v / o and the shared expert's gate / up / down, each d x d, Q4
     group 64 (BF16 scale ~U(0.005, 0.02), zero point uniform [0, 15] stored as bias = -z * scale).  The benchmark definition gives no
-    shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs up to 16 tokens, the packed
-    MFMA GEMM above (the reference's enc_dense / enc_dense_packed change over at 8, engine/mova_cuda.c:1020-1028)."""
+    shapes for them; these are fixed here.  run() is the launch sequence of one step: matvecs for few tokens, the packed
+    MFMA GEMMs above (the reference's enc_dense / enc_dense_packed change over at 8, engine/mova_cuda.c:1020-1028).  From
+    gemm_from to 32 tokens the matrices that share an input go through the grouped GEMM's entry points as "experts" that every
+    token chose - q, k and v as one launch of three tiles, the shared expert's gate and up with SwiGLU as one launch - so that a
+    launch has 135 and 90 workgroups where a 2880-row matrix alone has 45."""
 
-    def __init__(self, rng, n_layers, d, T):
+    def __init__(self, rng, n_layers, d, T, gemm_from=9):
         from nanoseedlm_amd import backend, moe, packs
         self.L, self.d, self.T, self.keep = backend.hip(), d, T, []
         self.layers = []
@@ -95,6 +98,14 @@ class Q4Projections:
         self.q, self.kk, self.v, self.o, self.a, self.g, self.u, self.sh = (f(T * d) for _ in range(8))
         self.px, self.pa = moe.DevBuf(2 * T * d), moe.DevBuf(2 * T * d)
         self.sel0 = moe.DevBuf.from_array(np.zeros(max(T, 1), dtype=np.int32))
+        self.gemm_from = gemm_from
+        # grouped launches: pair (matrix e, token t) reads row perm / n = t of the input and writes row perm = t n + e of the output
+        self.y3g, self.p3g = moe.DevBuf(4 * T * 3 * d), moe.DevBuf(2 * T * 3 * d)
+        self.perm3 = moe.DevBuf.from_array(np.array([t * 3 + e for e in range(3) for t in range(T)], dtype=np.int32))
+        self.tiles3 = moe.DevBuf.from_array(np.array([[e, e * T, T, 0] for e in range(3)], dtype=np.int32))
+        self.perm1 = moe.DevBuf.from_array(np.arange(T, dtype=np.int32))
+        self.tiles1 = moe.DevBuf.from_array(np.array([[0, 0, T, 0]], dtype=np.int32))
+        self.nt3, self.nt1 = moe.DevBuf.from_array(np.array([3], dtype=np.int32)), moe.DevBuf.from_array(np.array([1], dtype=np.int32))
         self.R3, self.add3 = (C.c_int * 3)(d, d, d), (C.c_int * 3)(0, 0, 0)
         self.y3 = (C.c_void_p * 3)(self.q.ptr.value, self.kk.ptr.value, self.v.ptr.value)
         self.L.kc_mv_multi.argtypes = [C.c_void_p, C.c_int, C.c_int, C.POINTER(backend.WSlice), C.POINTER(C.c_int), C.POINTER(C.c_void_p),
@@ -104,7 +115,18 @@ class Q4Projections:
         from nanoseedlm_amd import packs
         L, d, T, Q4 = self.L, self.d, self.T, packs.MF_Q4
         arr, tab = self.layers[layer]
-        if T <= 16:   # (up to 16 rows the matvecs are ahead of the GEMMs on these 2880 x 2880 matrices: 19 against 23 us a projection at 16)
+        if self.gemm_from <= T <= 32:
+            ws = C.sizeof(arr[0])
+            L.kc_pack_input_bf16(stream, x_ptr, self.px.ptr, C.c_size_t(T * d))
+            L.kc_mm_grouped_packed_rows(stream, Q4, tab.ptr, d, d, self.px.ptr, d, self.y3g.ptr, d, 3, self.perm3.ptr, self.tiles3.ptr,
+                                        self.nt3.ptr, 3, T)                                  # [T][q | k | v]
+            L.kc_pack_input_bf16(stream, self.y3g.ptr, self.p3g.ptr, C.c_size_t(T * 3 * d))
+            L.kc_mm_packed(stream, Q4, arr[3], d, d, self.p3g.ptr, 3 * d, self.o.ptr, d, T, 0, None)   # o over the q columns
+            if L.kc_mm_grouped_swiglu(stream, Q4, tab.at(4 * ws), tab.at(5 * ws), d, d, self.px.ptr, d, self.pa.ptr, d, 1, self.perm1.ptr,
+                                      self.tiles1.ptr, self.nt1.ptr, 1, T):
+                raise RuntimeError("kc_mm_grouped_swiglu refused the shared expert's shape")
+            L.kc_mm_packed(stream, Q4, arr[6], d, d, self.pa.ptr, d, self.sh.ptr, d, T, 0, None)
+        elif T <= 16:   # (matvecs: ahead of the one-matrix GEMMs on these 2880 x 2880 matrices, 19 against 23 us a projection at 16 rows)
             # q, k, v over the same input: one launch (kc_mv_multi; the same bits as one kc_mv each), else the three launches
             if L.kc_mv_multi(stream, Q4, 3, arr, self.R3, self.y3, self.R3, self.add3, d, x_ptr, d, T, None, C.c_float(0.0)):
                 for i, y in enumerate((self.q, self.kk, self.v)):
@@ -127,7 +149,7 @@ class Q4Projections:
             L.kc_mm_packed(stream, Q4, arr[6], d, d, self.pa.ptr, d, self.sh.ptr, d, T, 0, None)
 
 
-def moe_workload(name, steps, warmup, n_layers, no_graph):
+def moe_workload(name, steps, warmup, n_layers, no_graph, q4_gemm_from=9):
     from nanoseedlm_amd import backend, moe, packs
     cfgs = {"c2": dict(E=128, k=8, d=2048, ff=768, fmt=packs.MF_SEED4P4), "c3": dict(E=64, k=4, d=2880, ff=2880, fmt=packs.MF_SEED4)}
     c = cfgs[name[:2]]
@@ -142,7 +164,7 @@ def moe_workload(name, steps, warmup, n_layers, no_graph):
         st.set_layer(l, gate, up, down, rw)
         del gate, up, down
     st.finalize()
-    q4 = Q4Projections(rng, n_layers, d, T) if name[:2] == "c3" else None
+    q4 = Q4Projections(rng, n_layers, d, T, q4_gemm_from) if name[:2] == "c3" else None
     NX = 16
     xs = [moe.DevBuf.from_array(packs.round_bf16(rng.standard_normal((T, d)).astype(np.float32))) for _ in range(NX)]
     out = moe.DevBuf(4 * T * d)
@@ -531,6 +553,7 @@ def main():
     ap.add_argument("--layers", type=int, default=4)
     ap.add_argument("--matrices", type=int, default=64, help="c0: matrices the launches rotate over (64: records from HBM; 1: resident in the Infinity Cache)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--q4-gemm-from", type=int, default=9, help="c3: rows from which the Q4 projections take the grouped GEMM launches instead of matvecs")
     ap.add_argument("--no-graph", action="store_true", help="c4: plain stream launches instead of one hipGraph per step (c2 / c3 steps are stream launches unless --graph)")
     ap.add_argument("--graph", action="store_true", help="c2 / c3: one hipGraph per step")
     ap.add_argument("--splits", type=int, default=32, help="c4: pieces the attention of a (row, head group) is split into over the context")
@@ -547,7 +570,7 @@ def main():
         # Layer steps are issued as plain launches on the stream: a step of up to 24 rows of C2 is ONE launch, and around the
         # about ten launches of a batched step (or the five of C3 with its projections) a hipGraph replay a step measured
         # 5 us slower than the launches themselves (C2 at 32 rows 253.9 against 248.4 us, C3 at 1 row 92.2 against 87.1).
-        r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or not a.graph)
+        r = moe_workload(a.workload, a.steps, a.warmup, a.layers, a.no_graph or not a.graph, a.q4_gemm_from)
     elif a.workload[:2] == "c4":
         r = model_workload(a.workload, a.steps, a.warmup, a.no_graph, a.branches, a.splits)
     else:

@@ -788,3 +788,54 @@ def test_mm_grouped_packed_rows_marks_a_broken_bound():
     assert np.array_equal(np.sort(pm), np.arange(40))
     assert np.array_equal(b[pm[:32]], a[pm[:32]])
     assert (b[pm[32:]] == 0x7FC00000).all()
+
+
+@pytest.mark.parametrize("T", [9, 16, 32])
+def test_grouped_launches_over_matrices_that_share_an_input(T):
+    """Three affine-int4 matrices over the same rows as one grouped launch - every matrix a tile of T pairs, pair (e, t) reading
+    row perm / 3 = t and writing row perm = 3 t + e - against kc_mm_packed on each matrix alone, and two of them with SwiGLU as one
+    kc_mm_grouped_swiglu launch (one tile) against kc_swiglu_pack of the two products: bit for bit."""
+    import ctypes as C
+    from nanoseedlm_amd import backend, moe
+    backend.require_gpu()
+    L = backend.hip()
+    rng = np.random.default_rng(77 + T)
+    K, R, Q4 = 256, 128, packs.MF_Q4
+    pk = packs.affine(rng, 3, R, K, bits=4, group=64)
+    bufs = [moe.DevBuf.from_array(pk[k]) for k in ("words", "scales", "biases")]
+    arr = (backend.WSlice * 3)()
+    for i in range(3):
+        arr[i].p[0] = bufs[0].ptr.value + i * R * K // 2
+        arr[i].p[1] = bufs[1].ptr.value + i * R * (K // 64) * 2
+        arr[i].p[2] = bufs[2].ptr.value + i * R * (K // 64) * 2
+        arr[i].gs = 6
+    tab = moe.DevBuf(C.sizeof(arr))
+    backend.check(L.nh_memcpy_h2d(tab.ptr, arr, C.c_size_t(C.sizeof(arr))), "nh_memcpy_h2d")
+    px = moe.DevBuf.from_array(packs.f32_to_bf16_bits(rng.standard_normal((T, K)).astype(np.float32)))
+    alone = [moe.DevBuf(4 * T * R) for _ in range(3)]
+    for i in range(3):
+        L.kc_mm_packed(None, Q4, arr[i], K, R, px.ptr, K, alone[i].ptr, R, T, 0, None)
+    y3 = moe.DevBuf(4 * T * 3 * R)
+    L.nh_memset(y3.ptr, 0xFF, C.c_size_t(y3.nbytes))
+    perm = moe.DevBuf.from_array(np.array([t * 3 + e for e in range(3) for t in range(T)], dtype=np.int32))
+    tiles = moe.DevBuf.from_array(np.array([[e, e * T, T, 0] for e in range(3)], dtype=np.int32))
+    nt = moe.DevBuf.from_array(np.array([3], dtype=np.int32))
+    L.kc_mm_grouped_packed_rows(None, Q4, tab.ptr, K, R, px.ptr, K, y3.ptr, R, 3, perm.ptr, tiles.ptr, nt.ptr, 3, T)
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    got = y3.to_array(np.uint32, (T, 3, R))
+    for i in range(3):
+        assert np.array_equal(got[:, i, :], alone[i].to_array(np.uint32, (T, R))), i
+    # gate = matrix 0, up = matrix 1
+    want16, got16 = moe.DevBuf(2 * T * R), moe.DevBuf(2 * T * R)
+    L.kc_swiglu_pack(None, alone[0].ptr, alone[1].ptr, want16.ptr, C.c_size_t(T * R))
+    perm1 = moe.DevBuf.from_array(np.arange(T, dtype=np.int32))
+    tile1 = moe.DevBuf.from_array(np.array([[0, 0, T, 0]], dtype=np.int32))
+    nt1 = moe.DevBuf.from_array(np.array([1], dtype=np.int32))
+    ws = C.sizeof(arr[0])
+    assert L.kc_mm_grouped_swiglu(None, Q4, tab.ptr, tab.at(ws), K, R, px.ptr, K, got16.ptr, R, 1, perm1.ptr, tile1.ptr, nt1.ptr, 1, T) == 0
+    moe.device_sync()
+    assert L.kc_last_error() == 0
+    assert np.array_equal(got16.to_array(np.uint16, (T, R)), want16.to_array(np.uint16, (T, R)))
+    for b in bufs + alone + [tab, px, y3, perm, tiles, nt, want16, got16, perm1, tile1, nt1]:
+        b.free()
