@@ -312,8 +312,13 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         ring[sl] = v;
         if (sl < NTHR) ring[sl + RING] = v;
     };
+    // (down rows whose chunks are a power of two inside a wave: whole rows an iteration, the thread's place in them fixed)
+    auto deal_d = [&](int it) {
+        if constexpr (SHFL_D) return Deal{it * NTHR + tid, it * c.rpi + dl, dch, 0, false};
+        else return deal(it, c.nit, ltd, Ld, c.by_Ld);
+    };
     auto fetch_d = [&](int t, int it) {   // (unconditional too: rows and pairs past the end are clamped)
-        const Deal q = deal(it, c.nit, ltd, Ld, c.by_Ld);
+        const Deal q = deal_d(it);
         const int g = min(q.row, c.rows_t - 1), jj = (int) ((uint32_t) g / c.by_rpc), rr = g - jj * rpc;
         const WSlice& w = slice(min(t, T - 1), jj, 2);
         return load_chunk<P>(w, (uint32_t) min(r0 + rr, a.d - 1) * (uint32_t) Ld + (uint32_t) q.ch);
@@ -388,7 +393,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         // (the loads are unconditional: a load under a condition keeps the compiler from counting the loads in flight, and it
         // then waits for the next task's records before it computes the current one.  Past the last task the slot requests
         // the thread's first down records instead.)
-        const Deal q_d = deal(0, c.nit, ltd, Ld, c.by_Ld);   // (fetch_d(0, 0)'s records)
+        const Deal q_d = deal_d(0);   // (fetch_d(0, 0)'s records)
         const int g_d = min(q_d.row, c.rows_t - 1), jj_d = (int) ((uint32_t) g_d / c.by_rpc);
         const uint32_t unit_d = (uint32_t) min(r0 + g_d - jj_d * rpc, a.d - 1) * (uint32_t) Ld + (uint32_t) q_d.ch;
         auto fetch = [&](int t, int i) {
@@ -616,7 +621,7 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
         for (int it = 0; it < c.nit; ++it) {
             const bool last = it + 1 == c.nit;
             const Chunk dnxt = fetch_d(last ? t + 1 : t, last ? 0 : it + 1);
-            const Deal q = deal(it, c.nit, ltd, Ld, c.by_Ld);
+            const Deal q = deal_d(it);
             const int g = q.row, j = min((int) ((uint32_t) g / c.by_rpc), kk - 1), rr = g - (int) ((uint32_t) g / c.by_rpc) * rpc;
             const bool ok = g < c.rows_t && rr < nr;
             float acc[1] = {0.0f};
@@ -735,7 +740,7 @@ int launch_moe_decode_cu(hipStream_t st, FusedArgs& a, int P, bool sd) {
     auto take = [&](int words) { const int at = o; o += (words + 3) & ~3; return at; };
     c.xg = take(a.T * a.Lg * xp);
     c.xd = take(a.kk * a.Ld * xp);
-    c.scr = take(4 * nthr);
+    c.scr = take(sg && sd ? 2 * nthr : 4 * nthr);   // (both passes by shuffles: unused)
     c.pk = take(a.T * c.KP);
     c.rv = take(a.T * c.E4);
     c.dsum = take(a.kk * c.rpc);
