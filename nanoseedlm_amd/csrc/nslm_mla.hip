@@ -381,15 +381,21 @@ __device__ __forceinline__ uint32_t bf2(float lo, float hi) {   // v_cvt_pk_bf16
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
-template <int R, int ROPE, int FMT>
-__global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* out) {
+// NG = 2 (launches that leave most of the chip idle: a workgroup a CU or fewer): two groups of four waves, each with tiles of its
+// own in LDS, take the split's key tiles alternately - the chain of tiles a workgroup walks is half as long - and group 1's running
+// maximum, sum and accumulators are merged into group 0's through LDS before the split's partial result leaves, as two splits'
+// would be by the reduce.  The groups meet at the same workgroup barriers (a group without a tile in an iteration only waits).
+template <int R, int ROPE, int FMT, int NG>
+__global__ void __launch_bounds__(256 * NG) k_mla_attn_mfma(MlaArgs a, const float* ql, const float* qr, KvView kv, const RowInfo* ri, float* out) {
     static_assert(R == 512 && ROPE == 64, "the thread mapping of the decode covers 64 latent dim groups and 8 RoPE dim groups");
+    static_assert(NG == 1 || NG == 2, "one group of four waves, or two");
     constexpr int KW = R + ROPE, KLD = KW + 8, NKS = KW / 32, MT = R / 64, NW = FMT == KV_FP8 ? 2 : 4;
     extern __shared__ __attribute__((aligned(16))) uint8_t mla_lds[];
-    uint16_t* Ks = (uint16_t*) mla_lds;
+    const int grp = NG > 1 ? (int) threadIdx.x >> 8 : 0;
+    uint16_t* Ks = (uint16_t*) (mla_lds + grp * mla_mfma_lds<R, ROPE>());
     uint16_t* Vt = Ks + MA_KB * KLD;
     f32x4* Sx = (f32x4*) (Vt + R * MA_KB);   // [wave][lane]: the waves' partial score tiles
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int tid = (int) threadIdx.x & 255, w = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;   // (tid, w: within the group)
     const int split = (int) blockIdx.x, t = (int) blockIdx.z, h = (int) blockIdx.y * 16 + c;
     const int pos = ri[t].pos, kv0 = ri[t].kv0;
     int p0, p1;
@@ -540,7 +546,7 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     float m = -INFINITY, l = 0.0f;
-    if (p0 < p1) load_tile(p0);
+    if (p0 + grp * MA_KB < p1) load_tile(p0 + grp * MA_KB);
     // scores: wave w sums k-slices [9 (w >> 1), + 9) of key tile w & 1
     constexpr int KH = NKS / 2;
     const int su = w & 1, sk = (w >> 1) * KH;
@@ -560,19 +566,27 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
         for (int ks = 0; ks < KH; ++ks) qf[ks] = *(const bf16x8*) &Qs[c * KLD + 32 * (sk + ks) + 8 * g];
         __syncthreads();
     }
-    for (int p = p0; p < p1; p += MA_KB) {
-        store_tile();
+    for (int pb = p0; pb < p1; pb += MA_KB * NG) {
+        const int p = pb + grp * MA_KB;
+        const bool mine = NG == 1 || p < p1;   // (uniform over the group)
+        if (mine) store_tile();
         __syncthreads();
-        if (p + MA_KB < p1) load_tile(p + MA_KB);
+        if (p + MA_KB * NG < p1) load_tile(p + MA_KB * NG);
         f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;   // two chains over the wave's 9 k-slices
+        if (mine) {
 #pragma unroll
-        for (int ks = 0; ks < KH; ++ks) {
-            const bf16x8 a0 = *(const bf16x8*) &Ks[(16 * su + c) * KLD + 32 * (sk + ks) + 8 * g];
-            if (ks & 1) s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s1, 0, 0, 0);
-            else s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
+            for (int ks = 0; ks < KH; ++ks) {
+                const bf16x8 a0 = *(const bf16x8*) &Ks[(16 * su + c) * KLD + 32 * (sk + ks) + 8 * g];
+                if (ks & 1) s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s1, 0, 0, 0);
+                else s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, qf[ks], s0, 0, 0, 0);
+            }
+            Sx[tid] = s0 + s1;
         }
-        Sx[tid] = s0 + s1;
         __syncthreads();
+        if (!mine) {   // no tile of this group's in the split's last iteration: the third barrier, nothing else
+            __syncthreads();
+            continue;
+        }
         s0 = Sx[lane] + Sx[128 + lane];        // key tile 0: waves 0 and 2
         s1 = Sx[64 + lane] + Sx[192 + lane];   // key tile 1: waves 1 and 3
         float sv[8], mx = -INFINITY;
@@ -612,6 +626,27 @@ __global__ void __launch_bounds__(256) k_mla_attn_mfma(MlaArgs a, const float* q
     }
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
+    if (NG > 1) {   // group 1's state into group 0's, thread by thread (the same head, the same latent dims), as two splits merge
+        float* mg = (float*) (mla_lds + mla_mfma_lds<R, ROPE>()) + tid * (4 * MT + 2);   // (group 1's tiles: read for the last time before the loop's last barrier)
+        if (grp == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mg[4 * mt + i] = acc[mt][i];
+            mg[4 * MT] = m;
+            mg[4 * MT + 1] = l;
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = mg[4 * MT], l1 = mg[4 * MT + 1], mn = fmaxf(m, m1);
+        const float f0 = m == mn ? 1.0f : __expf(m - mn), f1 = m1 == mn ? 1.0f : __expf(m1 - mn);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[mt][i] = acc[mt][i] * f0 + mg[4 * mt + i] * f1;
+        l = l * f0 + l1 * f1;
+        m = mn;
+    }
     if (!live) return;
     if (a.n_splits == 1) {
         float* o = out + ((size_t) t * a.n_head + h) * R;
@@ -854,13 +889,19 @@ static bool mla_attn_launch(kc_stream_t s, MlaArgs a, const float* ql, const flo
     if (a.n_splits > MLA_RED_MAXS) { host_note_unsupported(); return false; }
     if (a.r == 512 && rope == 64 && (((uintptr_t) ql | (uintptr_t) qr) & 15u) == 0) {   // the matrix-core kernel: 16 heads a workgroup
         constexpr int lds = mla_mfma_lds<512, 64>();
-        static const hipError_t once[2] = {
-            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_BF16>, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
-            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_FP8>, hipFuncAttributeMaxDynamicSharedMemorySize, lds)};
+        static const hipError_t once[4] = {
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_BF16, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_FP8, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, lds),
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_BF16, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * lds),
+            hipFuncSetAttribute((const void*) k_mla_attn_mfma<512, 64, KV_FP8, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * lds)};
         (void) once;
         const dim3 grid((unsigned) a.n_splits, (unsigned) (a.n_head + 15) / 16, (unsigned) T);
-        if (kv.fmt == KV_FP8) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_FP8>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
-        else hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_BF16>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+        // a workgroup a CU or fewer: two groups of waves a workgroup walk a split's tiles (a step of a few rows is a chain of tiles)
+        const bool two = (long) grid.x * grid.y * grid.z <= 256;
+        if (two && kv.fmt == KV_FP8) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_FP8, 2>), grid, dim3(512), 2 * lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+        else if (two) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_BF16, 2>), grid, dim3(512), 2 * lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+        else if (kv.fmt == KV_FP8) hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_FP8, 1>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
+        else hipLaunchKernelGGL((k_mla_attn_mfma<512, 64, KV_BF16, 1>), grid, dim3(256), lds, (hipStream_t) s, a, ql, qr, kv, ri, o);
     } else {
         const size_t lds = sizeof(float) * (size_t) (GA_KT + GA_HW) * (size_t) (a.r + rope + 4);
         static const hipError_t once = hipFuncSetAttribute((const void*) k_mla_attn_any, hipFuncAttributeMaxDynamicSharedMemorySize,
