@@ -609,7 +609,26 @@ __global__ void __launch_bounds__(NTHR) k_moe_decode_cu(FusedArgs a, CuParams c)
             wait_stage(0);
             float acc0 = 0.0f;
             if (ok) cols_post(zp, dcur.codes, slice(0, j, 2).eb, xd + j * (Ld * XP) + dch * XP, acc0);
-            rows_out(0, 0, acc0, ok, g, j, rr, true, tid);
+            if constexpr (SHFL_D) rows_out(0, 0, acc0, ok, g, j, rr, true, tid);
+            else {
+                // (one iteration: the threads' sums side by side, no ring - this path is the C2 step's, and every instruction of it counts)
+                part[tid] = acc0;
+                __syncthreads();
+                const int js = min((int) ((uint32_t) tid / c.by_rpc), kk - 1), rs = tid - (int) ((uint32_t) tid / c.by_rpc) * rpc;
+                if (tid < c.rows_t && rs < nr) {
+                    float sm = 0.0f;
+                    for (int c0 = 0; c0 < Ld; c0 += 8) {
+                        float pv[8];
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) pv[cc] = part[tid * Ld + min(c0 + cc, Ld - 1)];
+#pragma unroll
+                        for (int cc = 0; cc < 8; ++cc) sm += c0 + cc < Ld ? pv[cc] : 0.0f;
+                    }
+                    const float dv = bfr(sm * NSLM_R32);
+                    dsum[tid] = dv;
+                    a.D[(size_t) js * a.d + r0 + rs] = dv;
+                }
+            }
             __syncthreads();
             combine(0);
         }
