@@ -250,7 +250,8 @@ void kc_mla_rope(kc_stream_t s, MlaArgs a, float* qr, const float* kr, const flo
                  const float* inv, int T);
 /* engine/kernels_cuda.h:157-161, engine/kernels_moe.cu:1217-1323,2459-2489.  olat[t][h] = bf16(sum_p softmax_p(scale (ql_th .
  * c_p + qr_th . k_p)) c_p) over p <= pos_t; n_splits > 1 splits the keys (partials in part: T x n_head x n_splits x (r + 2)
- * floats) and reduces.  r % 8 == 0, r <= 1024. */
+ * floats) and reduces.  r % 8 == 0, r <= 1024.  (r = 512, rope = 64: the matrix-core kernel, a workgroup a (split, 16 heads, row); a
+ * launch of at most 256 such workgroups runs two groups of four waves a workgroup over a split's keys and uses 149 KB of LDS a workgroup.) */
 /* No counterpart in the reference (three launches there): kc_heads_mv(hq: query -> RoPE mix, O = rope) + kc_heads_mv(hl: query
  * -> latent, O = r) + kc_mla_rope in ONE launch, the same bits.  Both maps in fmt over the same query rows (equal I, xs, hs, no
  * gate).  0, or -1 when the shapes are outside it (r % 64, I / 8 not a power of two <= 64 ...): nothing is launched. */
